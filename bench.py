@@ -1,0 +1,347 @@
+#!/usr/bin/env python3
+"""Roofline benchmark of the amd-gpu operator path (RMSNorm, RoPE, SwiGLU, Add).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--ops-table]
+
+One *step* is one pass of the Llama-70B-shaped bf16 prefill chain on 8192
+tokens (the largest configuration of every operator):
+
+    RMSNorm [8192, 8192] (w fp32)  ->  RoPE q [8192, 64, 128] and k [8192, 8, 128]
+    (strided views of one fused qkv buffer [8192, 80, 128])  ->  SwiGLU [8192, 28672]
+    from a fused gate/up buffer [8192, 57344]  ->  Add [8192, 8192]
+
+five launches through the public C API on one stream.  Inputs are synthetic
+(seeded N(0,1) / U(0.5,1.5)), resident in HBM before the timed region, and the
+steps rotate over several independent buffer sets so that nothing is served
+from the 256 MB Infinity Cache.  The line printed at the end is one JSON
+object: `value` is algorithmic bytes moved per second over the whole chain;
+`roofline` describes the dominant kernel (SwiGLU) timed on its own with events
+on the launch stream; `cpu_baseline` is the CPU oracle timed on this host on a
+bounded sample of the same workload; `ops` lists every operator/configuration
+with its own time, bandwidth and fraction of the 8 TB/s peak.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate over")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-ops-table", action="store_true", help="skip the per-operator table (C1-C4 and per-op C5)")
+    ap.add_argument("--only", default=None, help="time a single named entry of the per-operator table and exit (for profiling)")
+    ap.add_argument("--tokens", type=int, default=8192, help="tokens of the chain (default: the full configuration)")
+    return ap.parse_args()
+
+
+# ---------------------------------------------------------------------------------
+# workloads
+# ---------------------------------------------------------------------------------
+class Launch:
+    """One prepared stage-4 call: bound function + arguments, and its algorithmic bytes."""
+
+    def __init__(self, name, fn, args, nbytes, keep):
+        self.name, self.fn, self.args, self.nbytes, self.keep = name, fn, args, nbytes, keep
+
+    def __call__(self, stream):
+        st = self.fn(*self.args, stream)
+        if st != 0:
+            raise RuntimeError(f"{self.name}: status {st}")
+
+
+def _randn(shape, dtype, gen):
+    import torch
+
+    return torch.randn(shape, generator=gen, device="cuda", dtype=torch.float32).to(dtype)
+
+
+def make_rms_norm(ctx, n, d, dtype, w_dtype, gen, name):
+    import torch
+
+    from operators_amd.ops import RMSNormPlan
+
+    x = _randn((n, d), dtype, gen)
+    y = torch.empty_like(x)
+    w = (torch.rand(d, generator=gen, device="cuda") + 0.5).to(w_dtype)
+    plan = RMSNormPlan(ctx, y, x, w, 1e-5)
+    nbytes = 2 * n * d * x.element_size() + d * w.element_size()
+    return Launch(name, ctx.lib.infiniopRMSNorm, (plan.desc, None, 0, y.data_ptr(), x.data_ptr(), w.data_ptr()), nbytes, (plan, x, y, w))
+
+
+def make_rope(ctx, qkv, head0, heads, pos, sin_t, cos_t, name):
+    from operators_amd.ops import RoPEPlan
+
+    t = qkv[:, head0:head0 + heads, :]
+    plan = RoPEPlan(ctx, t, pos, sin_t, cos_t)
+    distinct = int(pos.view(dtype=__import__("torch").int64).unique().numel())
+    nbytes = 2 * t.numel() * t.element_size() + pos.numel() * 8 + 2 * distinct * t.shape[2] * 4
+    return Launch(name, ctx.lib.infiniopRoPE, (plan.desc, None, 0, t.data_ptr(), pos.data_ptr(), sin_t.data_ptr(), cos_t.data_ptr()),
+                  nbytes, (plan, qkv, pos, sin_t, cos_t))
+
+
+def make_swiglu(ctx, n, di, dtype, fused, gen, name):
+    import torch
+
+    from operators_amd.ops import SwiGLUPlan
+
+    if fused:
+        gate_up = _randn((n, 2 * di), dtype, gen)
+        b, a = gate_up[:, :di], gate_up[:, di:]
+        keep = gate_up
+    else:
+        a, b = _randn((n, di), dtype, gen), _randn((n, di), dtype, gen)
+        keep = (a, b)
+    c = torch.empty((n, di), dtype=dtype, device="cuda")
+    plan = SwiGLUPlan(ctx, c, a, b)
+    return Launch(name, ctx.lib.infiniopSwiGLU, (plan.desc, c.data_ptr(), a.data_ptr(), b.data_ptr()), 3 * n * di * c.element_size(), (plan, keep, c))
+
+
+def make_add(ctx, n, d, dtype, broadcast, gen, name):
+    import torch
+
+    from operators_amd.ops import AddPlan
+
+    a = _randn((n, d), dtype, gen)
+    b = _randn((d,) if broadcast else (n, d), dtype, gen)
+    c = torch.empty_like(a)
+    plan = AddPlan(ctx, c, a, b)
+    nbytes = (2 * n * d + b.numel()) * c.element_size()
+    return Launch(name, ctx.lib.infiniopAdd, (plan.desc, c.data_ptr(), a.data_ptr(), b.data_ptr()), nbytes, (plan, a, b, c))
+
+
+def chain_set(ctx, tokens, gen, tables):
+    """The five launches of one chain step on one private set of buffers."""
+    import torch
+
+    bf16 = torch.bfloat16
+    sin_t, cos_t, pos = tables
+    qkv = _randn((tokens, 80, 128), bf16, gen)
+    return [
+        make_rms_norm(ctx, tokens, 8192, bf16, torch.float32, gen, "rms_norm"),
+        make_rope(ctx, qkv, 0, 64, pos, sin_t, cos_t, "rope_q"),
+        make_rope(ctx, qkv, 64, 8, pos, sin_t, cos_t, "rope_k"),
+        make_swiglu(ctx, tokens, 28672, bf16, True, gen, "swiglu"),
+        make_add(ctx, tokens, 8192, bf16, False, gen, "add"),
+    ]
+
+
+# ---------------------------------------------------------------------------------
+# timing
+# ---------------------------------------------------------------------------------
+def time_rotating(sets, steps, warmup):
+    """sets: list of lists of Launch.  Runs warmup+steps passes, pass i on set
+    i % len(sets), all on torch's current stream.  Returns (wall seconds,
+    event seconds) for exactly `steps` passes."""
+    import torch
+
+    stream = torch.cuda.current_stream()
+    handle = stream.cuda_stream
+    for i in range(warmup):
+        for launch in sets[i % len(sets)]:
+            launch(handle)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for i in range(steps):
+        for launch in sets[i % len(sets)]:
+            launch(handle)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, e0.elapsed_time(e1) * 1e-3
+
+
+def op_entry(name, config, sets, steps, warmup):
+    wall, ev = time_rotating([[s] for s in sets], steps, warmup)
+    per_call = ev / steps
+    nbytes = sets[0].nbytes
+    gbps = nbytes / per_call / 1e9
+    return {"op": name, "config": config, "us_per_call": round(per_call * 1e6, 3), "bytes": nbytes,
+            "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+
+
+def ops_table(ctx, args, gen):
+    """Every operator at every BASELINE configuration, each timed alone."""
+    import torch
+
+    from operators_amd.ops import sin_cos_table
+
+    f16, bf16 = torch.float16, torch.bfloat16
+    nset = args.sets
+    T = args.tokens
+
+    def rope_sets(tokens, buf_heads, head0, heads, dtype, rows, theta, random_pos):
+        sin_t, cos_t = sin_cos_table(rows, 128, theta, device="cuda")
+        out = []
+        for _ in range(nset):
+            if random_pos:
+                pos = torch.randint(0, rows, (tokens,), generator=gen, device="cuda", dtype=torch.int64).view(torch.uint64)
+            else:
+                pos = torch.arange(tokens, device="cuda", dtype=torch.int64).view(torch.uint64)
+            qkv = _randn((tokens, buf_heads, 128), dtype, gen)
+            out.append(make_rope(ctx, qkv, head0, heads, pos, sin_t, cos_t, "rope"))
+        return out
+
+    builders = {
+        "C1 rms_norm f16 [16,2048] w f16": lambda: [make_rms_norm(ctx, 16, 2048, f16, f16, gen, "rms_norm") for _ in range(nset)],
+        "C2 swiglu f16 [4096,11008]": lambda: [make_swiglu(ctx, 4096, 11008, f16, False, gen, "swiglu") for _ in range(nset)],
+        "C2 swiglu f16 [4096,11008] fused gate/up": lambda: [make_swiglu(ctx, 4096, 11008, f16, True, gen, "swiglu") for _ in range(nset)],
+        "C3 rope f16 [4096,32,128] in [4096,96,128]": lambda: rope_sets(4096, 96, 0, 32, f16, 32768, 1e4, True),
+        "C4 add f16 [8192,4096]": lambda: [make_add(ctx, 8192, 4096, f16, False, gen, "add") for _ in range(nset)],
+        "C4 add f16 [8192,4096] + b[4096]": lambda: [make_add(ctx, 8192, 4096, f16, True, gen, "add") for _ in range(nset)],
+        f"C5 rms_norm bf16 [{T},8192] w f32": lambda: [make_rms_norm(ctx, T, 8192, bf16, torch.float32, gen, "rms_norm") for _ in range(nset)],
+        f"C5 rope_q bf16 [{T},64,128] in [{T},80,128]": lambda: rope_sets(T, 80, 0, 64, bf16, T, 5e5, False),
+        f"C5 rope_k bf16 [{T},8,128] in [{T},80,128]": lambda: rope_sets(T, 80, 64, 8, bf16, T, 5e5, False),
+        f"C5 swiglu bf16 [{T},28672] fused gate/up": lambda: [make_swiglu(ctx, T, 28672, bf16, True, gen, "swiglu") for _ in range(max(2, nset // 2))],
+        f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(nset)],
+    }
+    rows = []
+    for label, build in builders.items():
+        if args.only and args.only not in label:
+            continue
+        sets = build()
+        rows.append(op_entry(sets[0].name, label, sets, args.steps, args.warmup))
+        del sets
+        torch.cuda.empty_cache()
+    return rows
+
+
+# ---------------------------------------------------------------------------------
+# CPU baseline
+# ---------------------------------------------------------------------------------
+def cpu_baseline(tokens_full):
+    """The CPU oracle (a plain-C port of the reference's CPU path, extended to
+    bf16 - the reference itself accepts bf16 in none of the four operators) on
+    the first `tokens` tokens of the chain, one thread."""
+    import numpy as np
+
+    import oracle
+
+    tokens = min(2048, tokens_full)
+    rng = np.random.default_rng(0)
+
+    def bf16(shape):
+        return oracle.f32_to_bf16(rng.standard_normal(shape, dtype=np.float32))
+
+    x = bf16((tokens, 8192))
+    w = rng.uniform(0.5, 1.5, 8192).astype(np.float32)
+    qkv = bf16((tokens, 80, 128))
+    gate_up = bf16((tokens, 57344))
+    a, b = bf16((tokens, 8192)), bf16((tokens, 8192))
+    y, c_sw, c_add = np.empty_like(x), np.empty((tokens, 28672), np.uint16), np.empty_like(a)
+    pos = np.arange(tokens, dtype=np.uint64)
+    freqs = (1.0 / (np.float32(5e5) ** (np.arange(0, 128, 2, dtype=np.float32) / np.float32(128)))).astype(np.float32)
+    ang = np.outer(pos.astype(np.float32), np.repeat(freqs, 2)).astype(np.float32)
+    sin_t, cos_t = np.sin(ang), np.cos(ang)
+    nbytes = (2 * x.nbytes + w.nbytes) + (2 * tokens * 72 * 128 * 2 + 2 * (pos.nbytes + sin_t.nbytes + cos_t.nbytes)) + 3 * c_sw.nbytes + 3 * a.nbytes
+
+    def one_pass():
+        oracle.rms_norm(x, w, 1e-5, "bf16", "f32", y=y)
+        oracle.rope(qkv[:, :64, :], pos, sin_t, cos_t, "bf16")
+        oracle.rope(qkv[:, 64:72, :], pos, sin_t, cos_t, "bf16")
+        oracle.swiglu(gate_up[:, 28672:], gate_up[:, :28672], "bf16", c=c_sw)
+        oracle.add_into(c_add, a, b, "bf16")
+
+    one_pass()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[1]
+    cpu_model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {
+        "value": round(nbytes / med / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"first {tokens} of {tokens_full} tokens of every tensor of the chain, median of 3 passes after 1 warm-up, 1 thread",
+        "seconds_per_pass": round(med, 4), "ms_per_full_step_extrapolated": round(med * tokens_full / tokens * 1e3, 1),
+        "host_cpu": cpu_model, "host_logical_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU only (the operators are independent per token; "
+              "there is no multi-GPU path to measure) - run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from operators_amd.ops import Context, sin_cos_table
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the amd-gpu library has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    ctx = Context(0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    T = args.tokens
+
+    if args.only:
+        rows = ops_table(ctx, args, gen)
+        print(json.dumps({"ops": rows}))
+        return
+
+    # ---- the chain -------------------------------------------------------------
+    sin_t, cos_t = sin_cos_table(T, 128, 5e5, device="cuda")
+    pos = torch.arange(T, device="cuda", dtype=torch.int64).view(torch.uint64)
+    sets = [chain_set(ctx, T, gen, (sin_t, cos_t, pos)) for _ in range(args.sets)]
+    chain_bytes = sum(l.nbytes for l in sets[0])
+    wall, ev = time_rotating(sets, args.steps, args.warmup)
+    ms_per_step = wall / args.steps * 1e3
+    value = chain_bytes * args.steps / wall / 1e9
+
+    # ---- dominant kernel on its own: SwiGLU of the chain -------------------------
+    swiglu_sets = [[s[3]] for s in sets]
+    _, ev_sw = time_rotating(swiglu_sets, args.steps, args.warmup)
+    sw_time = ev_sw / args.steps
+    sw_bytes = sets[0][3].nbytes
+    roofline = {
+        "bound": "hbm", "achieved": round(sw_bytes / sw_time / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": round(sw_bytes / sw_time / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+        "kernel": f"swiglu_vec<bf16, row-strided> [{T},28672] from fused [{T},57344]",
+        "bytes_per_launch": sw_bytes, "us_per_launch": round(sw_time * 1e6, 2),
+    }
+    per_op_chain = {l.name: l.nbytes for l in sets[0]}
+    del sets, swiglu_sets
+    torch.cuda.empty_cache()
+
+    out = {
+        "metric": "achieved_hbm_bandwidth", "value": round(value, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"C5 Llama-70B-shaped bf16 prefill chain, {T} tokens: rms_norm[{T},8192] + rope q[{T},64,128], k[{T},8,128] in qkv[{T},80,128] + swiglu[{T},28672] (fused gate/up) + add[{T},8192]",
+                   "launches_per_step": 5, "buffer_sets": args.sets, "bytes_per_step": chain_bytes, "bytes_by_op": per_op_chain,
+                   "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4), "event_ms_per_step": round(ev / args.steps * 1e3, 4)},
+        "roofline": roofline,
+    }
+    if not args.no_ops_table:
+        out["ops"] = ops_table(ctx, args, gen)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(T)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,221 @@
+/*
+ * infiniop.h - the C ABI exported by this build of libinfiniop.so.
+ *
+ * The library implements ONE device of the InfiniOperators operator library,
+ * `DevAmdGpu` (AMD Instinct MI355X, gfx950), for the four memory-bound LLM-layer
+ * operators Add, RMSNorm, RoPE and SwiGLU.  The entry points below have the
+ * names, argument order, argument meaning and status codes of the reference
+ * library, so that a caller written against the reference (its ctypes harness,
+ * its composite operators, any C client) binds to this library unchanged and
+ * only selects another device number.  Each declaration names the reference
+ * declaration it stands in for (paths relative to the reference checkout).
+ *
+ * Calling convention ("3+1 stages"):
+ *   1. infiniopCreateHandle(&handle, DevAmdGpu, device_id)
+ *   2. infiniopCreate<Op>Descriptor(handle, &desc, tensor descriptors...)
+ *        all shape/stride/dtype checking happens here, once
+ *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE; always 0)
+ *   4. infiniop<Op>(desc, ..., data pointers..., stream)
+ *        enqueues on `stream` (a hipStream_t, NULL = the null stream) and
+ *        returns without synchronising
+ *   +  infiniopDestroy<Op>Descriptor(desc), infiniopDestroyHandle(handle)
+ *
+ * All data pointers are device pointers on the handle's GPU.  Strides are in
+ * elements.  Descriptors are immutable after creation: one descriptor may be
+ * used from several host threads and streams at once.
+ */
+#ifndef INFINIOP_AMD_INFINIOP_H
+#define INFINIOP_AMD_INFINIOP_H
+
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define INFINIOP_EXPORT __attribute__((visibility("default")))
+#else
+#define INFINIOP_EXPORT
+#endif
+
+#ifdef __cplusplus
+#define INFINIOP_C extern "C"
+#else
+#define INFINIOP_C
+#endif
+
+/* ---- status codes: replaces include/status.h:4-14 ---------------------- */
+typedef enum {
+    STATUS_SUCCESS = 0,
+    STATUS_EXECUTION_FAILED = 1,
+    STATUS_BAD_PARAM = 2,
+    STATUS_BAD_TENSOR_DTYPE = 3,
+    STATUS_BAD_TENSOR_SHAPE = 4,
+    STATUS_BAD_TENSOR_STRIDES = 5,
+    STATUS_MEMORY_NOT_ALLOCATED = 6,
+    STATUS_INSUFFICIENT_WORKSPACE = 7,
+    STATUS_BAD_DEVICE = 8,
+} infiniopStatus_t;
+
+/* ---- devices: replaces include/device.h:4-9 ----------------------------
+ * Values 0..3 are the reference's and keep their meaning; this library answers
+ * STATUS_BAD_DEVICE for them.  DevAmdGpu = 4 is the value a maintainer appends
+ * to the reference enum. */
+enum DeviceEnum {
+    DevCpu = 0,
+    DevNvGpu = 1,
+    DevCambriconMlu = 2,
+    DevAscendNpu = 3,
+    DevAmdGpu = 4,
+};
+typedef enum DeviceEnum Device;
+
+/* ---- element types: replaces include/data_type.h:4-46 ------------------
+ * A 4-byte bitfield passed BY VALUE; two layouts are the same type when their
+ * 32-bit images are equal. */
+typedef struct DataLayout {
+    unsigned short
+        packed : 8,
+        sign : 1,
+        size : 7,
+        mantissa : 8,
+        exponent : 8;
+} DataLayout;
+typedef struct DataLayout DT;
+
+#define INFINIOP_DT(p, s, z, m, e) {p, s, z, m, e}
+static const DataLayout
+    I8 = INFINIOP_DT(1, 1, 1, 7, 0),
+    I16 = INFINIOP_DT(1, 1, 2, 15, 0),
+    I32 = INFINIOP_DT(1, 1, 4, 31, 0),
+    I64 = INFINIOP_DT(1, 1, 8, 63, 0),
+    U8 = INFINIOP_DT(1, 0, 1, 8, 0),
+    U16 = INFINIOP_DT(1, 0, 2, 16, 0),
+    U32 = INFINIOP_DT(1, 0, 4, 32, 0),
+    U64 = INFINIOP_DT(1, 0, 8, 64, 0),
+    F16 = INFINIOP_DT(1, 1, 2, 10, 5),
+    BF16 = INFINIOP_DT(1, 1, 2, 7, 8),
+    F32 = INFINIOP_DT(1, 1, 4, 23, 8),
+    F64 = INFINIOP_DT(1, 1, 8, 52, 11);
+
+/* ---- tensor descriptor: replaces include/tensor.h:7-18 ----------------- */
+struct TensorDescriptor {
+    DT dt;            /* element type */
+    uint64_t ndim;    /* number of dimensions, 0 allowed */
+    uint64_t *shape;  /* ndim extents */
+    int64_t *strides; /* ndim strides, in elements */
+};
+typedef struct TensorDescriptor *infiniopTensorDescriptor_t;
+
+/* replaces include/tensor/tensor_descriptor.h:8 - deep-copies shape and strides;
+ * strides == NULL means contiguous row-major. */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateTensorDescriptor(
+    infiniopTensorDescriptor_t *desc_ptr, uint64_t ndim, uint64_t const *shape,
+    int64_t const *strides, DataLayout datatype);
+/* replaces include/tensor/tensor_descriptor.h:10 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyTensorDescriptor(infiniopTensorDescriptor_t desc);
+
+/* ---- handle: replaces include/handle.h:6-10 ----------------------------
+ * Every handle and every operator descriptor begins with its Device; callers
+ * may read that field and nothing else. */
+typedef struct HandleStruct {
+    Device device;
+} HandleStruct;
+typedef HandleStruct *infiniopHandle_t;
+
+/* replaces include/handle/handle_export.h:8.  NULL handle_ptr ->
+ * STATUS_MEMORY_NOT_ALLOCATED; device_id < 0 -> STATUS_BAD_PARAM; any device
+ * other than DevAmdGpu, no such GPU, or a GPU that is not gfx950 ->
+ * STATUS_BAD_DEVICE. */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateHandle(infiniopHandle_t *handle_ptr, Device device, int device_id);
+/* replaces include/handle/handle_export.h:10 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyHandle(infiniopHandle_t handle);
+
+/* ======================================================================== *
+ * Add:  c = a + b with numpy-style broadcasting of a and b onto c.
+ * F16, F32 (reference) and BF16 (extension).  c, a, b must be "contiguous" in
+ * the reference's sense; c is written in flat row-major order.  In-place on a
+ * or b is allowed when no broadcasting is involved.
+ * ======================================================================== */
+typedef struct AddDescriptor {
+    Device device;
+} AddDescriptor;
+typedef AddDescriptor *infiniopAddDescriptor_t;
+
+/* replaces include/ops/add/add.h:13-17 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateAddDescriptor(
+    infiniopHandle_t handle, infiniopAddDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t c, infiniopTensorDescriptor_t a, infiniopTensorDescriptor_t b);
+/* replaces include/ops/add/add.h:19-23 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopAdd(
+    infiniopAddDescriptor_t desc, void *c, void const *a, void const *b, void *stream);
+/* replaces include/ops/add/add.h:25 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyAddDescriptor(infiniopAddDescriptor_t desc);
+
+/* ======================================================================== *
+ * RMSNorm:  y[i][j] = x[i][j] * w[j] / sqrt(mean_j(x[i][j]^2) + epsilon)
+ * x, y: 2-D F16 (reference) or BF16 (extension) with unit inner stride and
+ * independent row strides; w: 1-D F16, BF16 or F32.
+ * ======================================================================== */
+typedef struct RMSNormDescriptor {
+    Device device;
+} RMSNormDescriptor;
+typedef RMSNormDescriptor *infiniopRMSNormDescriptor_t;
+
+/* replaces include/ops/rms_norm/rms_norm.h:13-19 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateRMSNormDescriptor(
+    infiniopHandle_t handle, infiniopRMSNormDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t y_desc, infiniopTensorDescriptor_t x_desc,
+    infiniopTensorDescriptor_t w_desc, float epsilon);
+/* replaces include/ops/rms_norm/rms_norm.h:21 - always 0 bytes */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetRMSNormWorkspaceSize(infiniopRMSNormDescriptor_t desc, uint64_t *size);
+/* replaces include/ops/rms_norm/rms_norm.h:23-24 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRMSNorm(
+    infiniopRMSNormDescriptor_t desc, void *workspace, uint64_t workspace_size,
+    void *y, void const *x, void const *w, void *stream);
+/* replaces include/ops/rms_norm/rms_norm.h:26 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyRMSNormDescriptor(infiniopRMSNormDescriptor_t desc);
+
+/* ======================================================================== *
+ * RoPE:  in-place rotation of adjacent pairs (2k, 2k+1) of t[token][head][:]
+ * by the angle whose sin/cos are rows pos_ids[token] of two caller-supplied
+ * F32 tables [rows, head_dim].  t: 3-D F16 (reference) or BF16 (extension)
+ * with arbitrary token and head strides, unit inner stride; pos_ids: 1-D U64.
+ * The tables are indexed with row stride head_dim, as the reference does.
+ * ======================================================================== */
+typedef struct RoPEDescriptor RoPEDescriptor; /* opaque, as in the reference */
+typedef RoPEDescriptor *infiniopRoPEDescriptor_t;
+
+/* replaces include/ops/rotary_embedding/rotary_embedding.h:10-16 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateRoPEDescriptor(
+    infiniopHandle_t handle, infiniopRoPEDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t t, infiniopTensorDescriptor_t pos_ids,
+    infiniopTensorDescriptor_t sin_table, infiniopTensorDescriptor_t cos_table);
+/* replaces include/ops/rotary_embedding/rotary_embedding.h:18 - always 0 bytes */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetRoPEWorkspaceSize(infiniopRoPEDescriptor_t desc, uint64_t *size);
+/* replaces include/ops/rotary_embedding/rotary_embedding.h:20-28 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRoPE(
+    infiniopRoPEDescriptor_t desc, void *workspace, uint64_t workspace_size,
+    void *t, void const *pos_ids, void const *sin_table, void const *cos_table, void *stream);
+/* replaces include/ops/rotary_embedding/rotary_embedding.h:30 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyRoPEDescriptor(infiniopRoPEDescriptor_t desc);
+
+/* ======================================================================== *
+ * SwiGLU:  c = a * b * sigmoid(b)   (b is the gated operand, a the linear one)
+ * 2-D F16 (reference) or BF16 (extension), unit inner stride, one row stride
+ * per tensor - so a and b may be the two halves of one fused gate/up buffer.
+ * In-place on a or on b is allowed.
+ * ======================================================================== */
+typedef struct SwiGLUDescriptor {
+    Device device;
+} SwiGLUDescriptor;
+typedef SwiGLUDescriptor *infiniopSwiGLUDescriptor_t;
+
+/* replaces include/ops/swiglu/swiglu.h:13-17 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateSwiGLUDescriptor(
+    infiniopHandle_t handle, infiniopSwiGLUDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t c_desc, infiniopTensorDescriptor_t a_desc, infiniopTensorDescriptor_t b_desc);
+/* replaces include/ops/swiglu/swiglu.h:19-23 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopSwiGLU(
+    infiniopSwiGLUDescriptor_t desc, void *c, void const *a, void const *b, void *stream);
+/* replaces include/ops/swiglu/swiglu.h:25 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroySwiGLUDescriptor(infiniopSwiGLUDescriptor_t desc);
+
+#endif /* INFINIOP_AMD_INFINIOP_H */

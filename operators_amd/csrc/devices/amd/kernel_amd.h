@@ -1,0 +1,189 @@
+// Device-side building blocks for the gfx950 kernels: 128-bit global access,
+// 16-bit <-> fp32 conversion with the reference's rounding, and wavefront /
+// workgroup reductions for 64-wide wavefronts.  Include from .hip files only.
+#ifndef INFINIOP_AMD_KERNEL_H
+#define INFINIOP_AMD_KERNEL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace amd {
+
+constexpr int kWave = 64;// CDNA wavefront width
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// ---- 128-bit global access ------------------------------------------------
+// One lane moves 16 bytes; a wavefront moves 1 KiB per instruction.  Streaming
+// operands are touched exactly once, so loads and stores carry the
+// non-temporal hint and do not displace reusable lines (weights, tables) from
+// L2.
+__device__ __forceinline__ u32x4 ld16_stream(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
+__device__ __forceinline__ void st16_stream(void *p, u32x4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+}
+__device__ __forceinline__ u32x4 ld16(const void *p) {
+    return *reinterpret_cast<const u32x4 *>(p);
+}
+__device__ __forceinline__ f32x4 ld16f(const float *p) {
+    return *reinterpret_cast<const f32x4 *>(p);
+}
+
+// ---- fp32 -> fp16 exactly as the reference's CPU path narrows --------------
+// The reference truncates the mantissa (round toward zero), produces
+// subnormals by a truncating shift, maps NaN to sign|0x7E00, +-Inf and any
+// exponent >= 31 to sign|0x7C00, and does not guard exponents 16..30, whose
+// bits spill upward and are cut to 16 bits
+// (reference src/devices/cpu/common_cpu.cc:41-64).  This is that rule for any
+// input, in integer arithmetic.
+__device__ __forceinline__ uint32_t narrow_f16_any(float v) {
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t s = (u >> 16) & 0x8000u;
+    const int e = static_cast<int>((u >> 23) & 0xFFu) - 127;
+    uint32_t m = u & 0x7FFFFFu;
+    if (e >= 31) return (e == 128 && m != 0) ? (s | 0x7E00u) : (s | 0x7C00u);
+    if (e >= -14) return (s | (static_cast<uint32_t>(e + 15) << 10) | (m >> 13)) & 0xFFFFu;
+    if (e >= -24) {
+        m = (m | 0x800000u) >> static_cast<uint32_t>(-14 - e);
+        return s | (m >> 13);
+    }
+    return s;
+}
+
+// True when the hardware round-toward-zero pack gives the reference's bits:
+// every finite |v| < 65536 (normal, subnormal or zero result).
+__device__ __forceinline__ bool f16_fast_ok(float v) {
+    return (__float_as_uint(v) & 0x7FFFFFFFu) < 0x47800000u;
+}
+
+// ---- element traits ---------------------------------------------------------
+// widen2: the two 16-bit elements of one 32-bit word -> two floats (exact).
+// narrow2: two floats -> one 32-bit word, with the type's rounding rule.
+struct F16Ref {
+    static constexpr bool kNeedsFixup = true;
+    __device__ static __forceinline__ float lo(uint32_t w) {
+        return static_cast<float>(__builtin_bit_cast(f16x2, w).x);
+    }
+    __device__ static __forceinline__ float hi(uint32_t w) {
+        return static_cast<float>(__builtin_bit_cast(f16x2, w).y);
+    }
+    __device__ static __forceinline__ float one(uint16_t h) {
+        return static_cast<float>(__builtin_bit_cast(_Float16, h));
+    }
+    // v_cvt_pkrtz_f16_f32: round toward zero, subnormals kept.
+    __device__ static __forceinline__ uint32_t narrow2_fast(float a, float b) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+    }
+    __device__ static __forceinline__ uint32_t narrow2_any(float a, float b) {
+        return narrow_f16_any(a) | (narrow_f16_any(b) << 16);
+    }
+    __device__ static __forceinline__ bool fast_ok(float v) { return f16_fast_ok(v); }
+    __device__ static __forceinline__ uint16_t narrow1(float a) {
+        return static_cast<uint16_t>(narrow_f16_any(a));
+    }
+};
+
+// bf16 is this back end's extension (the reference accepts it in none of the
+// four operators): exact widening, round-to-nearest-even narrowing
+// (v_cvt_pk_bf16_f32 on gfx950); NaN stays NaN.
+struct BF16Rne {
+    static constexpr bool kNeedsFixup = false;
+    __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+    __device__ static __forceinline__ float one(uint16_t h) {
+        return __uint_as_float(static_cast<uint32_t>(h) << 16);
+    }
+    __device__ static __forceinline__ uint32_t narrow2_fast(float a, float b) {
+        f32x2 v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+    }
+    __device__ static __forceinline__ uint32_t narrow2_any(float a, float b) { return narrow2_fast(a, b); }
+    __device__ static __forceinline__ bool fast_ok(float) { return true; }
+    __device__ static __forceinline__ uint16_t narrow1(float a) {
+        return __builtin_bit_cast(uint16_t, static_cast<__bf16>(a));
+    }
+};
+
+// Eight results -> one 128-bit word.  For fp16 the hardware pack is used when
+// all eight are inside its exact domain; the test is made wave-uniform with a
+// ballot so the rare integer path costs nothing when no lane needs it.
+template<typename T>
+__device__ __forceinline__ u32x4 narrow8(const float (&r)[8]) {
+    u32x4 out;
+    out.x = T::narrow2_fast(r[0], r[1]);
+    out.y = T::narrow2_fast(r[2], r[3]);
+    out.z = T::narrow2_fast(r[4], r[5]);
+    out.w = T::narrow2_fast(r[6], r[7]);
+    if constexpr (T::kNeedsFixup) {
+        uint32_t worst = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t mag = __float_as_uint(r[i]) & 0x7FFFFFFFu;
+            worst = mag > worst ? mag : worst;
+        }
+        if (__builtin_amdgcn_ballot_w64(worst >= 0x47800000u) != 0) {
+            out.x = T::narrow2_any(r[0], r[1]);
+            out.y = T::narrow2_any(r[2], r[3]);
+            out.z = T::narrow2_any(r[4], r[5]);
+            out.w = T::narrow2_any(r[6], r[7]);
+        }
+    }
+    return out;
+}
+
+template<typename T>
+__device__ __forceinline__ void widen8(u32x4 v, float (&r)[8]) {
+    r[0] = T::lo(v.x);
+    r[1] = T::hi(v.x);
+    r[2] = T::lo(v.y);
+    r[3] = T::hi(v.y);
+    r[4] = T::lo(v.z);
+    r[5] = T::hi(v.z);
+    r[6] = T::lo(v.w);
+    r[7] = T::hi(v.w);
+}
+
+// ---- reductions -------------------------------------------------------------
+// Sum over the 64 lanes of a wavefront with DPP cross-lane adds: four steps
+// inside each row of 16 lanes, then row broadcasts 15 and 31; the total lands
+// in lane 63 and is read back to every lane through an SGPR.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));// quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));// quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));// row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));// row_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));// row_bcast:15 -> rows 1,3
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));// row_bcast:31 -> rows 2,3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Sum over a workgroup of WAVES wavefronts.  `slots` is LDS with room for
+// 2*WAVES floats; `phase` alternates 0/1 between consecutive calls so that one
+// barrier per call is enough (a wave can only overwrite a slot set after every
+// wave has passed the barrier that follows the previous use of the other set).
+template<int WAVES>
+__device__ __forceinline__ float block_sum(float v, float *slots, int phase) {
+    v = wave_sum(v);
+    if constexpr (WAVES == 1) {
+        return v;
+    } else {
+        float *mine = slots + phase * WAVES;
+        const int wave = threadIdx.x / kWave;
+        if ((threadIdx.x & (kWave - 1)) == 0) mine[wave] = v;
+        __syncthreads();
+        float total = 0.0f;
+#pragma unroll
+        for (int i = 0; i < WAVES; ++i) total += mine[i];
+        return total;
+    }
+}
+
+}// namespace amd
+
+#endif

@@ -1,0 +1,291 @@
+// gfx950 kernels for Add and their launch.
+//
+// Arithmetic contract (reference src/ops/add/cpu/add_cpu.cc:72-89): fp16
+// operands are widened to fp32, added in fp32 and narrowed with the reference's
+// truncating conversion, bit for bit; fp32 is one IEEE add; bf16 (extension)
+// is widened, added in fp32 and rounded to nearest even.
+//
+// The operation moves 3 bytes per byte of output and computes almost nothing,
+// so everything here is about keeping HBM busy: 16 bytes per lane per access,
+// several independent accesses in flight per lane, non-temporal hints on data
+// that is touched once.
+#include "../../../devices/amd/kernel_amd.h"
+#include "add_amd.h"
+
+namespace {
+
+using namespace amd;
+
+constexpr int kBlock = 256;// 4 wavefronts
+constexpr int kUnroll = 4; // independent 16-byte accesses per lane per operand
+
+// ---- per-type arithmetic on one 128-bit word ---------------------------------
+template<typename T>
+struct Add16 {
+    typedef uint16_t scalar;
+    static constexpr int kPerVec = 8;
+    __device__ static __forceinline__ u32x4 vec(u32x4 a, u32x4 b) {
+        float x[8], y[8];
+        widen8<T>(a, x);
+        widen8<T>(b, y);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += y[i];
+        return narrow8<T>(x);
+    }
+    __device__ static __forceinline__ scalar one(scalar a, scalar b) {
+        return T::narrow1(T::one(a) + T::one(b));
+    }
+    __device__ static __forceinline__ u32x4 splat(scalar s) {
+        const uint32_t w = static_cast<uint32_t>(s) * 0x00010001u;
+        return u32x4{w, w, w, w};
+    }
+};
+
+struct Add32 {
+    typedef float scalar;
+    static constexpr int kPerVec = 4;
+    __device__ static __forceinline__ u32x4 vec(u32x4 a, u32x4 b) {
+        const f32x4 r = __builtin_bit_cast(f32x4, a) + __builtin_bit_cast(f32x4, b);
+        return __builtin_bit_cast(u32x4, r);
+    }
+    __device__ static __forceinline__ scalar one(scalar a, scalar b) { return a + b; }
+    __device__ static __forceinline__ u32x4 splat(scalar s) {
+        const uint32_t w = __float_as_uint(s);
+        return u32x4{w, w, w, w};
+    }
+};
+
+// ---- no broadcasting: c[i] = a[i] + b[i] over a flat range -------------------
+// Each workgroup walks tiles of kBlock*kUnroll vectors; inside a tile lane l
+// takes vectors l, l+kBlock, ... so every access instruction of a wavefront
+// covers 1 KiB of consecutive memory.  All loads of a tile are issued before
+// the first add.
+template<typename Op>
+__global__ __launch_bounds__(kBlock) void add_flat_vec(u32x4 *c, const u32x4 *a, const u32x4 *b, uint64_t nvec) {
+    constexpr uint64_t kTile = static_cast<uint64_t>(kBlock) * kUnroll;
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kTile;
+    for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kTile; base < nvec; base += step) {
+        u32x4 va[kUnroll], vb[kUnroll];
+        if (base + kTile <= nvec) {
+#pragma unroll
+            for (int k = 0; k < kUnroll; ++k) {
+                const uint64_t i = base + k * kBlock + threadIdx.x;
+                va[k] = ld16_stream(a + i);
+                vb[k] = ld16_stream(b + i);
+            }
+#pragma unroll
+            for (int k = 0; k < kUnroll; ++k) {
+                const uint64_t i = base + k * kBlock + threadIdx.x;
+                st16_stream(c + i, Op::vec(va[k], vb[k]));
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < kUnroll; ++k) {
+                const uint64_t i = base + k * kBlock + threadIdx.x;
+                if (i < nvec) {
+                    va[k] = ld16_stream(a + i);
+                    vb[k] = ld16_stream(b + i);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < kUnroll; ++k) {
+                const uint64_t i = base + k * kBlock + threadIdx.x;
+                if (i < nvec) st16_stream(c + i, Op::vec(va[k], vb[k]));
+            }
+        }
+    }
+}
+
+// Element-at-a-time form for ranges that are not 16-byte aligned and for the
+// few elements left after the last whole vector.
+template<typename Op>
+__global__ __launch_bounds__(kBlock) void add_flat_scalar(typename Op::scalar *c, const typename Op::scalar *a,
+                                                          const typename Op::scalar *b, uint64_t first, uint64_t n) {
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
+    for (uint64_t i = first + static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += step) {
+        c[i] = Op::one(a[i], b[i]);
+    }
+}
+
+// ---- broadcasting -------------------------------------------------------------
+// Merged dimensions, innermost first.  c is flat; an operand's offset is the
+// sum of index*stride over the dimensions.
+struct BcastDims {
+    int ndim;
+    uint64_t shape[kAddMaxDims];
+    int64_t a_stride[kAddMaxDims];
+    int64_t b_stride[kAddMaxDims];
+};
+
+// Split a flat position (in units of `first_extent` along the innermost
+// dimension) into operand offsets.  Idx is 32-bit when every quantity fits,
+// which keeps the divisions cheap.
+template<typename Idx>
+__device__ __forceinline__ void bcast_offsets(const BcastDims &d, Idx pos, Idx inner_extent, int64_t inner_scale,
+                                              int64_t &off_a, int64_t &off_b) {
+    const Idx in = pos % inner_extent;
+    Idx rest = pos / inner_extent;
+    off_a = static_cast<int64_t>(in) * inner_scale * d.a_stride[0];
+    off_b = static_cast<int64_t>(in) * inner_scale * d.b_stride[0];
+#pragma unroll
+    for (int k = 1; k < kAddMaxDims; ++k) {
+        if (k < d.ndim) {
+            const Idx ext = static_cast<Idx>(d.shape[k]);
+            const Idx i = rest % ext;
+            rest /= ext;
+            off_a += static_cast<int64_t>(i) * d.a_stride[k];
+            off_b += static_cast<int64_t>(i) * d.b_stride[k];
+        }
+    }
+}
+
+// Vector form: the innermost merged dimension is a multiple of the vector
+// width and each operand either runs along it with stride 1 (128-bit load) or
+// stands still (one element, replicated).  A_RUNS / B_RUNS say which.
+template<typename Op, typename Idx, bool A_RUNS, bool B_RUNS>
+__global__ __launch_bounds__(kBlock) void add_bcast_vec(u32x4 *c, const typename Op::scalar *a,
+                                                        const typename Op::scalar *b, BcastDims d, uint64_t nvec) {
+    const Idx inner_vecs = static_cast<Idx>(d.shape[0] / Op::kPerVec);
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
+    for (uint64_t v = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; v < nvec; v += step) {
+        int64_t oa, ob;
+        bcast_offsets<Idx>(d, static_cast<Idx>(v), inner_vecs, Op::kPerVec, oa, ob);
+        u32x4 va, vb;
+        if constexpr (A_RUNS) va = ld16_stream(a + oa);
+        else va = Op::splat(a[oa]);
+        if constexpr (B_RUNS) vb = ld16_stream(b + ob);
+        else vb = Op::splat(b[ob]);
+        st16_stream(c + v, Op::vec(va, vb));
+    }
+}
+
+// Element form: any strides.
+template<typename Op, typename Idx>
+__global__ __launch_bounds__(kBlock) void add_bcast_scalar(typename Op::scalar *c, const typename Op::scalar *a,
+                                                           const typename Op::scalar *b, BcastDims d, uint64_t n) {
+    const Idx inner = static_cast<Idx>(d.shape[0]);
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += step) {
+        int64_t oa, ob;
+        bcast_offsets<Idx>(d, static_cast<Idx>(i), inner, 1, oa, ob);
+        c[i] = Op::one(a[oa], b[ob]);
+    }
+}
+
+// ---- launch -------------------------------------------------------------------
+inline unsigned grid_for(uint64_t work_items, uint64_t per_block, int cu_count, int blocks_per_cu) {
+    const uint64_t want = ceil_div(work_items, per_block);
+    const uint64_t cap = static_cast<uint64_t>(cu_count) * blocks_per_cu;
+    const uint64_t g = want < cap ? want : cap;
+    return static_cast<unsigned>(g == 0 ? 1 : g);
+}
+
+template<typename Op>
+infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a, const void *b, hipStream_t stream) {
+    typedef typename Op::scalar S;
+    const uint64_t n = desc.total;
+    const int cus = desc.cu_count;
+
+    if (desc.flat) {
+        uint64_t done = 0;
+        if (aligned16(c) && aligned16(a) && aligned16(b)) {
+            const uint64_t nvec = n / Op::kPerVec;
+            if (nvec > 0) {
+                const unsigned grid = grid_for(nvec, static_cast<uint64_t>(kBlock) * kUnroll, cus, 32);
+                add_flat_vec<Op><<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const u32x4 *>(a),
+                                                              static_cast<const u32x4 *>(b), nvec);
+            }
+            done = nvec * Op::kPerVec;
+        }
+        if (done < n) {
+            const unsigned grid = grid_for(n - done, kBlock, cus, 32);
+            add_flat_scalar<Op><<<grid, kBlock, 0, stream>>>(static_cast<S *>(c), static_cast<const S *>(a),
+                                                             static_cast<const S *>(b), done, n);
+        }
+        return STATUS_SUCCESS;
+    }
+
+    BcastDims d;
+    d.ndim = desc.ndim;
+    bool small = n < (1ull << 31);
+    for (int k = 0; k < kAddMaxDims; ++k) {
+        d.shape[k] = k < desc.ndim ? desc.shape[k] : 1;
+        d.a_stride[k] = k < desc.ndim ? desc.a_stride[k] : 0;
+        d.b_stride[k] = k < desc.ndim ? desc.b_stride[k] : 0;
+    }
+
+    // 128-bit access needs: inner extent a multiple of the vector width, inner
+    // strides 0 or 1, and every address a running operand can reach 16-byte
+    // aligned (base pointer and all outer strides multiples of the width).
+    const int64_t w = Op::kPerVec;
+    bool vec_ok = desc.shape[0] % w == 0 && aligned16(c) &&
+                  (desc.a_stride[0] == 0 || desc.a_stride[0] == 1) && (desc.b_stride[0] == 0 || desc.b_stride[0] == 1);
+    const bool a_runs = desc.a_stride[0] == 1, b_runs = desc.b_stride[0] == 1;
+    for (int k = 1; k < desc.ndim && vec_ok; ++k) {
+        if (a_runs && desc.a_stride[k] % w != 0) vec_ok = false;
+        if (b_runs && desc.b_stride[k] % w != 0) vec_ok = false;
+    }
+    if (a_runs && !aligned16(a)) vec_ok = false;
+    if (b_runs && !aligned16(b)) vec_ok = false;
+
+    if (vec_ok) {
+        const uint64_t nvec = n / w;
+        const unsigned grid = grid_for(nvec, kBlock, cus, 64);
+        auto go = [&](auto kernel) {
+            kernel<<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const S *>(a), static_cast<const S *>(b), d, nvec);
+        };
+        if (small) {
+            if (a_runs && b_runs) go(add_bcast_vec<Op, uint32_t, true, true>);
+            else if (a_runs) go(add_bcast_vec<Op, uint32_t, true, false>);
+            else if (b_runs) go(add_bcast_vec<Op, uint32_t, false, true>);
+            else go(add_bcast_vec<Op, uint32_t, false, false>);
+        } else {
+            if (a_runs && b_runs) go(add_bcast_vec<Op, uint64_t, true, true>);
+            else if (a_runs) go(add_bcast_vec<Op, uint64_t, true, false>);
+            else if (b_runs) go(add_bcast_vec<Op, uint64_t, false, true>);
+            else go(add_bcast_vec<Op, uint64_t, false, false>);
+        }
+    } else {
+        const unsigned grid = grid_for(n, kBlock, cus, 64);
+        if (small) {
+            add_bcast_scalar<Op, uint32_t><<<grid, kBlock, 0, stream>>>(static_cast<S *>(c), static_cast<const S *>(a),
+                                                                        static_cast<const S *>(b), d, n);
+        } else {
+            add_bcast_scalar<Op, uint64_t><<<grid, kBlock, 0, stream>>>(static_cast<S *>(c), static_cast<const S *>(a),
+                                                                        static_cast<const S *>(b), d, n);
+        }
+    }
+    return STATUS_SUCCESS;
+}
+
+}// namespace
+
+// Stage 4 of Add (reference src/ops/add/cuda/add.cu:104-120 for the NVIDIA
+// device): bind the descriptor's GPU, enqueue on the caller's stream, return
+// without waiting.
+infiniopStatus_t amdAdd(AddAmdDescriptor_t desc, void *c, void const *a, void const *b, void *stream) {
+    if (desc->total == 0) {
+        return STATUS_SUCCESS;
+    }
+    if (c == nullptr || a == nullptr || b == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    infiniopStatus_t st;
+    switch (desc->elem) {
+        case amd::Elem::F16:
+            st = launch_add<Add16<amd::F16Ref>>(*desc, c, a, b, s);
+            break;
+        case amd::Elem::BF16:
+            st = launch_add<Add16<amd::BF16Rne>>(*desc, c, a, b, s);
+            break;
+        case amd::Elem::F32:
+            st = launch_add<Add32>(*desc, c, a, b, s);
+            break;
+        default:
+            return STATUS_BAD_TENSOR_DTYPE;
+    }
+    AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+    return st;
+}

@@ -1,0 +1,244 @@
+// gfx950 kernels for RMSNorm and their launch.
+//
+// Arithmetic contract (reference src/ops/rms_norm/cpu/rms_norm_cpu.cc:46-86):
+//     ss   = sum_j x[j]^2                      fp32
+//     k    = (ss / d + eps) ^ -1/2             fp32 mean, double power
+//     y[j] = narrow( (k * x[j]) * w[j] )
+// The reference adds the squares left to right and carries the two products
+// in double before narrowing; here the sum is a tree over lanes and waves and
+// the products are fp32.  Both differences are below one fp32 ulp of y and
+// show up, after narrowing to 16 bits, as a last-bit difference on roughly one
+// element in 10^4.  fp16 narrows by the reference's truncation, bf16
+// (extension) rounds to nearest even.
+//
+// Data movement is the whole cost: x is read once and kept in registers
+// between the reduction and the scaling pass, y is written once, and the
+// weight row - re-used by every row - is staged once per workgroup in LDS as
+// fp32 when a workgroup serves more than one row.
+#include "../../../devices/amd/kernel_amd.h"
+#include "rms_norm_amd.h"
+
+namespace {
+
+using namespace amd;
+
+// ---- weight row access ----------------------------------------------------------
+struct WF32 {
+    typedef float scalar;
+    __device__ static __forceinline__ void load8(const void *w, uint32_t vec, float (&g)[8]) {
+        const float *p = static_cast<const float *>(w) + static_cast<uint64_t>(vec) * 8;
+        const f32x4 a = ld16f(p), b = ld16f(p + 4);
+        g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
+        g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
+    }
+    __device__ static __forceinline__ float one(const void *w, uint64_t j) { return static_cast<const float *>(w)[j]; }
+};
+template<typename T>
+struct W16 {
+    typedef uint16_t scalar;
+    __device__ static __forceinline__ void load8(const void *w, uint32_t vec, float (&g)[8]) {
+        widen8<T>(ld16(static_cast<const uint16_t *>(w) + static_cast<uint64_t>(vec) * 8), g);
+    }
+    __device__ static __forceinline__ float one(const void *w, uint64_t j) {
+        return T::one(static_cast<const uint16_t *>(w)[j]);
+    }
+};
+
+__device__ __forceinline__ float inv_rms(float sum_sq, uint64_t d, float eps) {
+    const float mean_eps = sum_sq / static_cast<float>(d) + eps;
+    return static_cast<float>(1.0 / sqrt(static_cast<double>(mean_eps)));
+}
+
+// ---- rows that fit in registers -----------------------------------------------
+// One workgroup of BS lanes per row at a time; lane l owns vectors l, l+BS, ...
+// (NV of them, 8 elements each), so d <= 8*BS*NV.  Workgroups stride over rows.
+//
+// LDS layout of the staged weight row: the 8 floats of vector v are split into
+// two 16-byte halves stored at lo[v] and hi[v] (hi = lo + nvec).  A wavefront
+// reading lo[v..v+63] or hi[v..v+63] then touches 64 consecutive 16-byte words
+// - no two lanes on the same bank in the same phase - where the natural
+// 32-byte-per-lane layout would be a two-way conflict.
+template<typename T, typename W, int BS, int NV, bool W_LDS>
+__global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w,
+                                                     uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps) {
+    constexpr int WAVES = BS / kWave;
+    __shared__ float red[2 * WAVES];
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
+    f32x4 *w_lo = reinterpret_cast<f32x4 *>(dyn_lds);
+    const uint32_t nvec = d / 8;
+    f32x4 *w_hi = w_lo + nvec;
+
+    if constexpr (W_LDS) {
+        for (uint32_t v = threadIdx.x; v < nvec; v += BS) {
+            float g[8];
+            W::load8(w, v, g);
+            w_lo[v] = f32x4{g[0], g[1], g[2], g[3]};
+            w_hi[v] = f32x4{g[4], g[5], g[6], g[7]};
+        }
+        __syncthreads();
+    }
+
+    int phase = 0;
+    for (uint64_t row = blockIdx.x; row < n; row += gridDim.x, phase ^= 1) {
+        const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
+        uint16_t *yr = y + static_cast<int64_t>(row) * stride_y;
+
+        u32x4 xv[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            xv[k] = v < nvec ? ld16_stream(xr + static_cast<uint64_t>(v) * 8) : u32x4{0, 0, 0, 0};
+        }
+
+        float part = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            float f[8];
+            widen8<T>(xv[k], f);
+            // pairwise inside the vector, then onto the running partial
+            const float s01 = f[0] * f[0] + f[1] * f[1], s23 = f[2] * f[2] + f[3] * f[3];
+            const float s45 = f[4] * f[4] + f[5] * f[5], s67 = f[6] * f[6] + f[7] * f[7];
+            part += (s01 + s23) + (s45 + s67);
+        }
+        const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
+
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            if (v < nvec) {
+                float f[8], g[8];
+                widen8<T>(xv[k], f);
+                if constexpr (W_LDS) {
+                    const f32x4 a = w_lo[v], b = w_hi[v];
+                    g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
+                    g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
+                } else {
+                    W::load8(w, v, g);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
+                st16_stream(yr + static_cast<uint64_t>(v) * 8, narrow8<T>(f));
+            }
+        }
+    }
+}
+
+// ---- any row length, any alignment ----------------------------------------------
+// Two passes over the row with element accesses; the second pass re-reads x,
+// which the first pass left in cache for rows of ordinary length.
+template<typename T, typename W>
+__global__ __launch_bounds__(256) void rms_norm_generic(uint16_t *y, const uint16_t *x, const void *w,
+                                                         uint64_t n, uint64_t d, int64_t stride_y, int64_t stride_x, float eps) {
+    constexpr int BS = 256, WAVES = BS / kWave;
+    __shared__ float red[2 * WAVES];
+    int phase = 0;
+    for (uint64_t row = blockIdx.x; row < n; row += gridDim.x, phase ^= 1) {
+        const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
+        uint16_t *yr = y + static_cast<int64_t>(row) * stride_y;
+        float part = 0.0f;
+        for (uint64_t j = threadIdx.x; j < d; j += BS) {
+            const float f = T::one(xr[j]);
+            part += f * f;
+        }
+        const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
+        for (uint64_t j = threadIdx.x; j < d; j += BS) {
+            yr[j] = T::narrow1((k_row * T::one(xr[j])) * W::one(w, j));
+        }
+        // y may alias x: every lane re-reads only elements it wrote itself.
+    }
+}
+
+// ---- launch -----------------------------------------------------------------------
+template<typename T, typename W>
+void launch_rms_norm(const RMSNormAmdDescriptor &desc, void *y, const void *x, const void *w, hipStream_t stream) {
+    auto *py = static_cast<uint16_t *>(y);
+    auto *px = static_cast<const uint16_t *>(x);
+    const uint64_t n = desc.n, d = desc.d;
+    const uint64_t nvec = d / 8;
+
+    const bool vec_ok = d % 8 == 0 && nvec <= 8192 && desc.stride_x % 8 == 0 && desc.stride_y % 8 == 0 &&
+                        aligned16(x) && aligned16(y) && aligned16(w);
+    if (!vec_ok) {
+        const uint64_t cap = static_cast<uint64_t>(desc.cu_count) * 8;
+        rms_norm_generic<T, W><<<static_cast<unsigned>(n < cap ? n : cap), 256, 0, stream>>>(
+            py, px, w, n, d, desc.stride_y, desc.stride_x, desc.epsilon);
+        return;
+    }
+
+    // Stage w in LDS when a workgroup will serve several rows and the fp32 row
+    // leaves room for at least two workgroups per compute unit.
+    const uint64_t lds_bytes = d * sizeof(float);
+    const uint64_t lds_limit = static_cast<uint64_t>(desc.lds_per_block) - 1024;
+    uint64_t per_cu = 8;
+    bool use_lds = lds_bytes <= lds_limit && lds_bytes <= 48 * 1024;
+    if (use_lds) {
+        const uint64_t fit = (160 * 1024) / (lds_bytes + 256);
+        per_cu = fit < per_cu ? fit : per_cu;
+    }
+    uint64_t grid = static_cast<uint64_t>(desc.cu_count) * per_cu;
+    if (n <= grid) {
+        grid = n;
+        use_lds = false;// one row per workgroup: staging would only add a pass
+    }
+
+#define RMS_LAUNCH(BS, NV)                                                                                              \
+    do {                                                                                                                \
+        if (use_lds)                                                                                                    \
+            rms_norm_rows<T, W, BS, NV, true><<<static_cast<unsigned>(grid), BS, lds_bytes, stream>>>(                  \
+                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon);                    \
+        else                                                                                                            \
+            rms_norm_rows<T, W, BS, NV, false><<<static_cast<unsigned>(grid), BS, 0, stream>>>(                         \
+                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon);                    \
+    } while (0)
+
+    if (nvec <= 64) RMS_LAUNCH(64, 1);
+    else if (nvec <= 128) RMS_LAUNCH(128, 1);
+    else if (nvec <= 256) RMS_LAUNCH(256, 1);
+    else if (nvec <= 512) RMS_LAUNCH(256, 2);
+    else if (nvec <= 1024) RMS_LAUNCH(256, 4);
+    else if (nvec <= 2048) RMS_LAUNCH(512, 4);
+    else if (nvec <= 4096) RMS_LAUNCH(1024, 4);
+    else RMS_LAUNCH(1024, 8);
+#undef RMS_LAUNCH
+}
+
+template<typename T>
+infiniopStatus_t launch_by_weight(const RMSNormAmdDescriptor &desc, void *y, const void *x, const void *w, hipStream_t s) {
+    switch (desc.w_elem) {
+        case amd::Elem::F32:
+            launch_rms_norm<T, WF32>(desc, y, x, w, s);
+            return STATUS_SUCCESS;
+        case amd::Elem::F16:
+            launch_rms_norm<T, W16<amd::F16Ref>>(desc, y, x, w, s);
+            return STATUS_SUCCESS;
+        case amd::Elem::BF16:
+            launch_rms_norm<T, W16<amd::BF16Rne>>(desc, y, x, w, s);
+            return STATUS_SUCCESS;
+        default:
+            return STATUS_BAD_TENSOR_DTYPE;
+    }
+}
+
+}// namespace
+
+// Stage 4 of RMSNorm.  The workspace is unused (its size is 0).
+infiniopStatus_t amdRMSNorm(RMSNormAmdDescriptor_t desc, void *, uint64_t, void *y, void const *x, void const *w, void *stream) {
+    if (desc->elem != amd::Elem::F16 && desc->elem != amd::Elem::BF16) {
+        return STATUS_BAD_TENSOR_DTYPE;
+    }
+    if (desc->n == 0 || desc->d == 0) {
+        return STATUS_SUCCESS;
+    }
+    if (y == nullptr || x == nullptr || w == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const infiniopStatus_t st = desc->elem == amd::Elem::F16 ? launch_by_weight<amd::F16Ref>(*desc, y, x, w, s)
+                                                             : launch_by_weight<amd::BF16Rne>(*desc, y, x, w, s);
+    if (st != STATUS_SUCCESS) {
+        return st;
+    }
+    AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+    return STATUS_SUCCESS;
+}

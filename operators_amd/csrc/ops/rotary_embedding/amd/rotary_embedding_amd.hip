@@ -1,0 +1,169 @@
+// gfx950 kernels for RoPE and their launch.
+//
+// Arithmetic contract (reference
+// src/ops/rotary_embedding/cpu/rotary_embedding_cpu.cc:16-44): for token i the
+// table rows start at pos[i]*head_dim; for pair k of every head, with
+// a = t[2k], b = t[2k+1] widened to fp32,
+//     t[2k]   = narrow( a*cos[2k]   - b*sin[2k]   )
+//     t[2k+1] = narrow( a*sin[2k+1] + b*cos[2k+1] )
+// each product rounded to fp32 on its own (the CPU build has no fused
+// multiply-add), four distinct table reads per pair.  Only IEEE multiply,
+// add and the reference's truncating narrowing are involved, so fp16 results
+// are bit-identical to the CPU's.  bf16 (extension) rounds to nearest even.
+//
+// t is read and written exactly once through arbitrary token/head strides;
+// the table rows of a token are fetched once per lane and reused for every
+// head that lane rotates.
+#include "../../../devices/amd/kernel_amd.h"
+#include "rotary_embedding_amd.h"
+
+// Products must not be fused into the add/subtract that follows them.
+#pragma clang fp contract(off)
+
+namespace {
+
+using namespace amd;
+
+constexpr int kBlock = 256;
+
+// One lane = one 8-element column group `cv` of up to HPT heads of one token.
+// Work items are numbered (token, head group g, cv) with cv fastest, so the
+// lanes of a wavefront cover consecutive 16-byte pieces of consecutive heads.
+// Lane (g, cv) rotates heads g, g+G, g+2G, ... (G = number of head groups):
+// at every step the wavefront's accesses are again to neighbouring heads.
+template<typename T, typename Idx, int HPT>
+__global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
+                                                   uint64_t total_items, Idx items_per_token, Idx vecs_per_head, Idx groups,
+                                                   uint32_t heads, uint32_t head_dim, int64_t stride_token, int64_t stride_head) {
+    const uint64_t item64 = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (item64 >= total_items) return;
+    const Idx item = static_cast<Idx>(item64);
+    const Idx token = item / items_per_token;
+    const Idx rem = item - token * items_per_token;
+    const Idx g = rem / vecs_per_head;
+    const Idx cv = rem - g * vecs_per_head;
+
+    uint16_t *base = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(cv) * 8;
+
+    u32x4 tv[HPT];
+#pragma unroll
+    for (int i = 0; i < HPT; ++i) {
+        const uint32_t h = static_cast<uint32_t>(g) + i * static_cast<uint32_t>(groups);
+        if (h < heads) tv[i] = ld16_stream(base + static_cast<int64_t>(h) * stride_head);
+    }
+
+    const uint64_t row = pos[token] * head_dim + static_cast<uint64_t>(cv) * 8;
+    const f32x4 s_lo = ld16f(sin_t + row), s_hi = ld16f(sin_t + row + 4);
+    const f32x4 c_lo = ld16f(cos_t + row), c_hi = ld16f(cos_t + row + 4);
+    const float sn[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+    const float cs[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+
+#pragma unroll
+    for (int i = 0; i < HPT; ++i) {
+        const uint32_t h = static_cast<uint32_t>(g) + i * static_cast<uint32_t>(groups);
+        if (h < heads) {
+            float f[8], r[8];
+            widen8<T>(tv[i], f);
+#pragma unroll
+            for (int k = 0; k < 8; k += 2) {
+                const float a = f[k], b = f[k + 1];
+                const float ac = a * cs[k], bs = b * sn[k];
+                const float as = a * sn[k + 1], bc = b * cs[k + 1];
+                r[k] = ac - bs;
+                r[k + 1] = as + bc;
+            }
+            st16_stream(base + static_cast<int64_t>(h) * stride_head, narrow8<T>(r));
+        }
+    }
+}
+
+// Any even head_dim, any strides and alignment: one lane per pair.
+template<typename T>
+__global__ __launch_bounds__(kBlock) void rope_pairs(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
+                                                     uint64_t total_pairs, uint64_t heads, uint64_t head_dim,
+                                                     int64_t stride_token, int64_t stride_head) {
+    const uint64_t half = head_dim / 2;
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < total_pairs; i += step) {
+        const uint64_t k = i % half;
+        const uint64_t th = i / half;
+        const uint64_t h = th % heads, token = th / heads;
+        uint16_t *p = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(h) * stride_head + 2 * k;
+        const uint64_t row = pos[token] * head_dim + 2 * k;
+        const float a = T::one(p[0]), b = T::one(p[1]);
+        const float ac = a * cos_t[row], bs = b * sin_t[row];
+        const float as = a * sin_t[row + 1], bc = b * cos_t[row + 1];
+        p[0] = T::narrow1(ac - bs);
+        p[1] = T::narrow1(as + bc);
+    }
+}
+
+template<typename T, typename Idx>
+void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, const float *sn, const float *cs, hipStream_t stream) {
+    const uint64_t vph = d.head_dim / 8;
+    const int hpt = d.heads >= 4 ? 4 : (d.heads >= 2 ? 2 : 1);
+    const uint64_t groups = ceil_div(d.heads, hpt);
+    const uint64_t ipt = groups * vph;
+    const uint64_t total = d.tokens * ipt;
+    const unsigned grid = static_cast<unsigned>(ceil_div(total, kBlock));
+#define ROPE_LAUNCH(HPT)                                                                                                   \
+    rope_vec<T, Idx, HPT><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph), \
+                                                       static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),            \
+                                                       static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
+    if (hpt == 4) ROPE_LAUNCH(4);
+    else if (hpt == 2) ROPE_LAUNCH(2);
+    else ROPE_LAUNCH(1);
+#undef ROPE_LAUNCH
+}
+
+template<typename T>
+void launch_rope(const RoPEAmdDescriptor &d, void *t, const void *pos_ids, const void *sin_table, const void *cos_table, hipStream_t stream) {
+    auto *pt = static_cast<uint16_t *>(t);
+    auto *pos = static_cast<const uint64_t *>(pos_ids);
+    auto *sn = static_cast<const float *>(sin_table);
+    auto *cs = static_cast<const float *>(cos_table);
+
+    const uint64_t elems = d.tokens * d.heads * d.head_dim;
+    const bool vec_ok = d.head_dim % 8 == 0 && d.stride_token % 8 == 0 && d.stride_head % 8 == 0 &&
+                        aligned16(t) && aligned16(sin_table) && aligned16(cos_table) &&
+                        d.heads < (1ull << 31) && d.head_dim < (1ull << 31) && elems / 8 < (1ull << 38);
+    if (!vec_ok) {
+        const uint64_t pairs = elems / 2;
+        const uint64_t want = ceil_div(pairs, kBlock), cap = static_cast<uint64_t>(d.cu_count) * 64;
+        rope_pairs<T><<<static_cast<unsigned>(want < cap ? want : cap), kBlock, 0, stream>>>(
+            pt, pos, sn, cs, pairs, d.heads, d.head_dim, d.stride_token, d.stride_head);
+        return;
+    }
+    if (elems / 8 < (1ull << 31)) launch_vec<T, uint32_t>(d, pt, pos, sn, cs, stream);
+    else launch_vec<T, uint64_t>(d, pt, pos, sn, cs, stream);
+}
+
+}// namespace
+
+// Stage 4 of RoPE.  Null data pointers are a bad parameter, as in
+// rotary_embedding_cpu.cc:119-120.  The workspace is unused (its size is 0).
+// pos_ids are not checked against the table length, as in the reference: a
+// position beyond the table is the caller's error.
+infiniopStatus_t amdRoPE(RoPEAmdDescriptor_t desc, void *, uint64_t, void *t, void const *pos_ids,
+                         void const *sin_table, void const *cos_table, void *stream) {
+    if (t == nullptr || pos_ids == nullptr || sin_table == nullptr || cos_table == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    if (desc->tokens == 0 || desc->heads == 0 || desc->head_dim == 0) {
+        return STATUS_SUCCESS;
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (desc->elem) {
+        case amd::Elem::F16:
+            launch_rope<amd::F16Ref>(*desc, t, pos_ids, sin_table, cos_table, s);
+            break;
+        case amd::Elem::BF16:
+            launch_rope<amd::BF16Rne>(*desc, t, pos_ids, sin_table, cos_table, s);
+            break;
+        default:
+            return STATUS_BAD_TENSOR_DTYPE;
+    }
+    AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+    return STATUS_SUCCESS;
+}

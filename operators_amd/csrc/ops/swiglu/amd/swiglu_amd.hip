@@ -1,0 +1,159 @@
+// gfx950 kernels for SwiGLU and their launch.
+//
+// Arithmetic contract (reference src/ops/swiglu/cpu/swiglu_cpu.cc:49-72):
+//     c = narrow( a * ( b / (1 + expf(-b)) ) )       all in fp32,
+// b gated, a linear; fp16 narrows with the reference's truncating conversion,
+// bf16 (extension) rounds to nearest even.  Division and expf are the
+// correctly-rounded / 1-ulp device routines, not the fast approximations, so
+// the fp32 value matches the CPU's except for expf's last bit.
+//
+// Three streams (two in, one out), ~30 VALU operations per element: bandwidth
+// bound.  Rows are addressed through one row stride per tensor, so the same
+// kernel serves separate a/b tensors and the gate/up halves of one fused
+// buffer (reference caller: src/ops/mlp/operator.cc:50-57,111-115).
+#include "../../../devices/amd/kernel_amd.h"
+#include "swiglu_amd.h"
+
+namespace {
+
+using namespace amd;
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 2;// independent 16-byte accesses per lane per operand
+
+__device__ __forceinline__ float swiglu1(float up, float gate) {
+    return up * (gate / (1.0f + expf(-gate)));
+}
+
+template<typename T>
+__device__ __forceinline__ u32x4 swiglu8(u32x4 va, u32x4 vb) {
+    float up[8], gate[8];
+    widen8<T>(va, up);
+    widen8<T>(vb, gate);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) up[i] = swiglu1(up[i], gate[i]);
+    return narrow8<T>(up);
+}
+
+// Position of vector `v` of the [rows, di/8] index space in a tensor whose row
+// stride is `stride` elements.  ROWWISE = false means all three tensors are
+// dense and the flat index is the address.
+template<typename Idx, bool ROWWISE>
+struct Where {
+    Idx vecs_per_row;
+    __device__ __forceinline__ void split(uint64_t v, Idx &row, Idx &col) const {
+        if constexpr (ROWWISE) {
+            row = static_cast<Idx>(v) / vecs_per_row;
+            col = static_cast<Idx>(v) - row * vecs_per_row;
+        } else {
+            row = 0;
+            col = static_cast<Idx>(v);
+        }
+    }
+};
+
+template<typename T, typename Idx, bool ROWWISE>
+__global__ __launch_bounds__(kBlock) void swiglu_vec(uint16_t *c, const uint16_t *a, const uint16_t *b,
+                                                      uint64_t nvec, Idx vecs_per_row,
+                                                      int64_t stride_c, int64_t stride_a, int64_t stride_b) {
+    constexpr uint64_t kTile = static_cast<uint64_t>(kBlock) * kUnroll;
+    const Where<Idx, ROWWISE> where{vecs_per_row};
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kTile;
+    for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kTile; base < nvec; base += step) {
+        u32x4 va[kUnroll], vb[kUnroll];
+        int64_t oc[kUnroll];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const uint64_t v = base + k * kBlock + threadIdx.x;
+            if (v < nvec) {
+                Idx row, col;
+                where.split(v, row, col);
+                const int64_t e = static_cast<int64_t>(col) * 8;
+                va[k] = ld16_stream(a + static_cast<int64_t>(row) * stride_a + e);
+                vb[k] = ld16_stream(b + static_cast<int64_t>(row) * stride_b + e);
+                oc[k] = static_cast<int64_t>(row) * stride_c + e;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const uint64_t v = base + k * kBlock + threadIdx.x;
+            if (v < nvec) st16_stream(c + oc[k], swiglu8<T>(va[k], vb[k]));
+        }
+    }
+}
+
+// Any width, any alignment: one element per lane per step.
+template<typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_scalar(uint16_t *c, const uint16_t *a, const uint16_t *b,
+                                                        uint64_t rows, uint64_t di,
+                                                        int64_t stride_c, int64_t stride_a, int64_t stride_b) {
+    const uint64_t n = rows * di;
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += step) {
+        const uint64_t row = i / di, col = i - row * di;
+        const float up = T::one(a[static_cast<int64_t>(row) * stride_a + col]);
+        const float gate = T::one(b[static_cast<int64_t>(row) * stride_b + col]);
+        c[static_cast<int64_t>(row) * stride_c + col] = T::narrow1(swiglu1(up, gate));
+    }
+}
+
+template<typename T>
+void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const void *b, hipStream_t stream) {
+    auto *pc = static_cast<uint16_t *>(c);
+    auto *pa = static_cast<const uint16_t *>(a);
+    auto *pb = static_cast<const uint16_t *>(b);
+    const uint64_t n = d.rows * d.di;
+    const int64_t di = static_cast<int64_t>(d.di);
+
+    const bool vec_ok = d.di % 8 == 0 && d.stride_a % 8 == 0 && d.stride_b % 8 == 0 && d.stride_c % 8 == 0 &&
+                        aligned16(c) && aligned16(a) && aligned16(b);
+    if (!vec_ok) {
+        const uint64_t want = ceil_div(n, kBlock), cap = static_cast<uint64_t>(d.cu_count) * 64;
+        swiglu_scalar<T><<<static_cast<unsigned>(want < cap ? want : cap), kBlock, 0, stream>>>(
+            pc, pa, pb, d.rows, d.di, d.stride_c, d.stride_a, d.stride_b);
+        return;
+    }
+
+    const uint64_t nvec = n / 8;
+    const uint64_t vpr = d.di / 8;
+    const uint64_t want = ceil_div(nvec, static_cast<uint64_t>(kBlock) * kUnroll);
+    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * 32;
+    const unsigned grid = static_cast<unsigned>(want < cap ? want : cap);
+    // One row, or every row stride equal to the width: the tensors are dense.
+    const bool dense = d.rows == 1 || (d.stride_a == di && d.stride_b == di && d.stride_c == di);
+    const bool small = nvec < (1ull << 31);
+    if (dense) {
+        swiglu_vec<T, uint64_t, false><<<grid, kBlock, 0, stream>>>(pc, pa, pb, nvec, vpr, d.stride_c, d.stride_a, d.stride_b);
+    } else if (small) {
+        swiglu_vec<T, uint32_t, true><<<grid, kBlock, 0, stream>>>(pc, pa, pb, nvec, static_cast<uint32_t>(vpr),
+                                                                   d.stride_c, d.stride_a, d.stride_b);
+    } else {
+        swiglu_vec<T, uint64_t, true><<<grid, kBlock, 0, stream>>>(pc, pa, pb, nvec, vpr, d.stride_c, d.stride_a, d.stride_b);
+    }
+}
+
+}// namespace
+
+// Stage 4 of SwiGLU: enqueue on the caller's stream and return.
+infiniopStatus_t amdSwiGLU(SwiGLUAmdDescriptor_t desc, void *c, void const *a, void const *b, void *stream) {
+    if (desc->rows == 0 || desc->di == 0) {
+        return STATUS_SUCCESS;
+    }
+    if (c == nullptr || a == nullptr || b == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (desc->elem) {
+        case amd::Elem::F16:
+            launch_swiglu<amd::F16Ref>(*desc, c, a, b, s);
+            break;
+        case amd::Elem::BF16:
+            launch_swiglu<amd::BF16Rne>(*desc, c, a, b, s);
+            break;
+        default:
+            return STATUS_BAD_TENSOR_DTYPE;
+    }
+    AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+    return STATUS_SUCCESS;
+}

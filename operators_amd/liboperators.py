@@ -1,0 +1,137 @@
+"""Loader and ctypes prototypes for libinfiniop.so (amd-gpu build).
+
+Counterpart of the reference's operatorspy/liboperators.py:11-73: the library is
+looked up under $INFINI_ROOT/lib when INFINI_ROOT is set, otherwise in this
+package's own lib/ directory (where `python -m operators_amd.build` puts it).
+There is no fallback implementation: if the library is missing, `open_lib`
+raises.
+"""
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_float, c_int, c_int32, c_int64, c_uint64, c_void_p
+
+from .data_layout import DataLayout
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libinfiniop.so"
+
+
+class TensorDescriptor(Structure):
+    _fields_ = [
+        ("dt", DataLayout),
+        ("ndim", c_uint64),
+        ("shape", POINTER(c_uint64)),
+        ("strides", POINTER(c_int64)),
+    ]
+
+
+infiniopTensorDescriptor_t = POINTER(TensorDescriptor)
+
+
+class Handle(Structure):
+    _fields_ = [("device", c_int)]
+
+
+infiniopHandle_t = POINTER(Handle)
+
+
+class _OpDescriptor(Structure):
+    """Every operator descriptor starts with its device number; nothing else
+    of it is visible to callers."""
+    _fields_ = [("device", c_int32)]
+
+
+class AddDescriptor(_OpDescriptor):
+    pass
+
+
+class RMSNormDescriptor(_OpDescriptor):
+    pass
+
+
+class RoPEDescriptor(_OpDescriptor):
+    pass
+
+
+class SwiGLUDescriptor(_OpDescriptor):
+    pass
+
+
+infiniopAddDescriptor_t = POINTER(AddDescriptor)
+infiniopRMSNormDescriptor_t = POINTER(RMSNormDescriptor)
+infiniopRoPEDescriptor_t = POINTER(RoPEDescriptor)
+infiniopSwiGLUDescriptor_t = POINTER(SwiGLUDescriptor)
+
+
+class CTensor:
+    """A tensor descriptor together with the address of its data."""
+
+    def __init__(self, desc, data):
+        self.descriptor = desc
+        self.data = data
+
+
+def library_path():
+    root = os.environ.get("INFINI_ROOT")
+    if root:
+        return os.path.join(root, "lib", LIB_NAME)
+    return os.path.join(_PKG_DIR, "lib", LIB_NAME)
+
+
+# name -> (argtypes); every entry point returns an infiniopStatus_t (int32)
+_PROTOTYPES = {
+    "infiniopCreateHandle": [POINTER(infiniopHandle_t), c_int, c_int],
+    "infiniopDestroyHandle": [infiniopHandle_t],
+    "infiniopCreateTensorDescriptor": [POINTER(infiniopTensorDescriptor_t), c_uint64, POINTER(c_uint64), POINTER(c_int64), DataLayout],
+    "infiniopDestroyTensorDescriptor": [infiniopTensorDescriptor_t],
+    "infiniopCreateAddDescriptor": [infiniopHandle_t, POINTER(infiniopAddDescriptor_t)] + [infiniopTensorDescriptor_t] * 3,
+    "infiniopAdd": [infiniopAddDescriptor_t, c_void_p, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroyAddDescriptor": [infiniopAddDescriptor_t],
+    "infiniopCreateRMSNormDescriptor": [infiniopHandle_t, POINTER(infiniopRMSNormDescriptor_t)] + [infiniopTensorDescriptor_t] * 3 + [c_float],
+    "infiniopGetRMSNormWorkspaceSize": [infiniopRMSNormDescriptor_t, POINTER(c_uint64)],
+    "infiniopRMSNorm": [infiniopRMSNormDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroyRMSNormDescriptor": [infiniopRMSNormDescriptor_t],
+    "infiniopCreateRoPEDescriptor": [infiniopHandle_t, POINTER(infiniopRoPEDescriptor_t)] + [infiniopTensorDescriptor_t] * 4,
+    "infiniopGetRoPEWorkspaceSize": [infiniopRoPEDescriptor_t, POINTER(c_uint64)],
+    "infiniopRoPE": [infiniopRoPEDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroyRoPEDescriptor": [infiniopRoPEDescriptor_t],
+    "infiniopCreateSwiGLUDescriptor": [infiniopHandle_t, POINTER(infiniopSwiGLUDescriptor_t)] + [infiniopTensorDescriptor_t] * 3,
+    "infiniopSwiGLU": [infiniopSwiGLUDescriptor_t, c_void_p, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroySwiGLUDescriptor": [infiniopSwiGLUDescriptor_t],
+}
+
+EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
+
+
+def bind_prototypes(lib):
+    """Attach argument and result types for the 18 entry points.  Works on any
+    library exporting the same C ABI (this one, or a build of the reference)."""
+    for name, argtypes in _PROTOTYPES.items():
+        fn = getattr(lib, name)  # AttributeError names the missing symbol
+        fn.argtypes = argtypes
+        fn.restype = c_int32
+    return lib
+
+
+_cached = {}
+
+
+def open_lib(path=None):
+    path = path or library_path()
+    if path in _cached:
+        return _cached[path]
+    # PyTorch-ROCm ships its own copy of the HIP runtime (same SONAME as the
+    # system one).  Two HIP runtimes in one process cannot both own the GPU, so
+    # when torch is going to be used in this process it has to be loaded first:
+    # the dynamic linker then binds this library to the copy torch brought.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+    if not os.path.isfile(path):
+        raise FileNotFoundError(
+            f"{path} not found: build it with `python -m operators_amd.build` "
+            "or point INFINI_ROOT at an installed copy")
+    lib = bind_prototypes(ctypes.CDLL(path))
+    _cached[path] = lib
+    return lib

@@ -1,0 +1,177 @@
+"""Torch-level convenience layer over the 3+1-stage C API.
+
+Each `*Plan` object is one operator descriptor: it is created from example
+tensors (stage 2, where the library validates shapes, strides and dtypes),
+can be launched any number of times on tensors of that layout (stage 4) and
+destroys the descriptor when closed.  `Context` owns a handle (stage 1).
+
+Launches go to the stream given (a raw hipStream_t value, e.g.
+`torch.cuda.current_stream().cuda_stream`); None is the null stream, which is
+what the reference's harness passes.  Nothing here synchronises.
+"""
+import ctypes
+
+from .devices import DeviceEnum
+from .liboperators import (
+    infiniopAddDescriptor_t,
+    infiniopRMSNormDescriptor_t,
+    infiniopRoPEDescriptor_t,
+    infiniopSwiGLUDescriptor_t,
+    open_lib,
+)
+from .utils import check_error, create_handle, destroy_handle, destroy_tensor, to_tensor
+
+
+class _Plan:
+    _destroy = None
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+        self.lib = ctx.lib
+        self.desc = None
+
+    def _describe(self, *tensors):
+        cts = [to_tensor(t, self.lib) for t in tensors]
+        return cts
+
+    def _release(self, cts):
+        for ct in cts:
+            destroy_tensor(self.lib, ct)
+
+    def close(self):
+        if self.desc is not None:
+            check_error(getattr(self.lib, self._destroy)(self.desc))
+            self.desc = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
+class AddPlan(_Plan):
+    _destroy = "infiniopDestroyAddDescriptor"
+
+    def __init__(self, ctx, c, a, b):
+        super().__init__(ctx)
+        cts = self._describe(c, a, b)
+        desc = infiniopAddDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateAddDescriptor(ctx.handle, ctypes.byref(desc), *[ct.descriptor for ct in cts]))
+        finally:
+            self._release(cts)
+        self.desc = desc
+
+    def __call__(self, c, a, b, stream=None):
+        check_error(self.lib.infiniopAdd(self.desc, c.data_ptr(), a.data_ptr(), b.data_ptr(), stream))
+        return c
+
+
+class SwiGLUPlan(_Plan):
+    _destroy = "infiniopDestroySwiGLUDescriptor"
+
+    def __init__(self, ctx, c, a, b):
+        super().__init__(ctx)
+        cts = self._describe(c, a, b)
+        desc = infiniopSwiGLUDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateSwiGLUDescriptor(ctx.handle, ctypes.byref(desc), *[ct.descriptor for ct in cts]))
+        finally:
+            self._release(cts)
+        self.desc = desc
+
+    def __call__(self, c, a, b, stream=None):
+        check_error(self.lib.infiniopSwiGLU(self.desc, c.data_ptr(), a.data_ptr(), b.data_ptr(), stream))
+        return c
+
+
+class RMSNormPlan(_Plan):
+    _destroy = "infiniopDestroyRMSNormDescriptor"
+
+    def __init__(self, ctx, y, x, w, epsilon):
+        super().__init__(ctx)
+        cts = self._describe(y, x, w)
+        desc = infiniopRMSNormDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateRMSNormDescriptor(ctx.handle, ctypes.byref(desc), *[ct.descriptor for ct in cts], epsilon))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetRMSNormWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value  # 0 for this library; the query is part of the calling sequence
+
+    def __call__(self, y, x, w, stream=None):
+        check_error(self.lib.infiniopRMSNorm(self.desc, None, self.workspace_size, y.data_ptr(), x.data_ptr(), w.data_ptr(), stream))
+        return y
+
+
+class RoPEPlan(_Plan):
+    _destroy = "infiniopDestroyRoPEDescriptor"
+
+    def __init__(self, ctx, t, pos_ids, sin_table, cos_table):
+        super().__init__(ctx)
+        cts = self._describe(t, pos_ids, sin_table, cos_table)
+        desc = infiniopRoPEDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateRoPEDescriptor(ctx.handle, ctypes.byref(desc), *[ct.descriptor for ct in cts]))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetRoPEWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value
+
+    def __call__(self, t, pos_ids, sin_table, cos_table, stream=None):
+        check_error(self.lib.infiniopRoPE(self.desc, None, self.workspace_size, t.data_ptr(), pos_ids.data_ptr(),
+                                          sin_table.data_ptr(), cos_table.data_ptr(), stream))
+        return t
+
+
+class Context:
+    """A library handle on one GPU plus one-shot forms of the four operators."""
+
+    def __init__(self, device_id=0, lib=None, device=DeviceEnum.DEVICE_AMD):
+        self.lib = lib or open_lib()
+        self.handle = create_handle(self.lib, device, device_id)
+
+    def close(self):
+        if self.handle is not None:
+            destroy_handle(self.lib, self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def add(self, c, a, b, stream=None):
+        with AddPlan(self, c, a, b) as plan:
+            return plan(c, a, b, stream)
+
+    def swiglu(self, c, a, b, stream=None):
+        with SwiGLUPlan(self, c, a, b) as plan:
+            return plan(c, a, b, stream)
+
+    def rms_norm(self, y, x, w, epsilon=1e-5, stream=None):
+        with RMSNormPlan(self, y, x, w, epsilon) as plan:
+            return plan(y, x, w, stream)
+
+    def rope(self, t, pos_ids, sin_table, cos_table, stream=None):
+        with RoPEPlan(self, t, pos_ids, sin_table, cos_table) as plan:
+            return plan(t, pos_ids, sin_table, cos_table, stream)
+
+
+def sin_cos_table(rows, head_dim, theta, device="cpu"):
+    """fp32 sin/cos tables [rows, head_dim] with each frequency repeated for
+    the two members of a pair, all arithmetic in fp32 (the table layout the
+    reference's harness builds, operatorspy/tests/rotary_embedding.py:54-64)."""
+    import torch
+
+    pos = torch.arange(0, rows, dtype=torch.float32, device=device)
+    freqs = 1.0 / (theta ** (torch.arange(0, head_dim, 2, device=device)[: head_dim // 2].float() / head_dim))
+    freqs = torch.repeat_interleave(freqs, repeats=2)
+    angles = torch.outer(pos, freqs)
+    return torch.sin(angles).contiguous(), torch.cos(angles).contiguous()

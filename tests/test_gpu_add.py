@@ -1,0 +1,153 @@
+"""Add on the GPU through the C ABI, against the oracle and the reference's
+golden vectors.  Bar: bit-exact (a generated NaN may differ in sign only)."""
+import json
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_codes_equal, golden, golden_json, to_codes, to_torch
+
+pytestmark = pytest.mark.gpu
+
+
+def run_add(ctx, a, b, c_shape, dtype):
+    import torch
+
+    ta, tb = to_torch(a, dtype).reshape(a.shape), to_torch(b, dtype).reshape(b.shape)
+    tc = torch.empty(tuple(c_shape), dtype=ta.dtype, device="cuda")
+    ctx.add(tc, ta, tb)
+    torch.cuda.synchronize()
+    return to_codes(tc).reshape(c_shape)
+
+
+def check(got, want, dtype, what):
+    if dtype == "f32":
+        g, w = got.view(np.uint32), want.view(np.uint32)
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan), what
+        assert np.array_equal(g[~nan], w[~nan]), what
+    else:
+        assert_codes_equal(got, want, dtype, what=what)
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_golden_cases(ctx, dt):
+    g = golden("add")
+    cases = golden_json()["add_cases"]
+    for i, (cs, as_, bs) in enumerate(cases):
+        a, b, want = g[f"add{i}_{dt}_a"], g[f"add{i}_{dt}_b"], g[f"add{i}_{dt}_c"]
+        got = run_add(ctx, a.reshape(as_), b.reshape(bs), tuple(cs), dt)
+        check(got, want.reshape(cs), dt, f"golden add case {i} {cs} = {as_} + {bs} {dt}")
+
+
+def test_golden_all_codes_plus_zero(ctx):
+    g = golden("add")
+    codes = np.arange(65536, dtype=np.uint16)
+    got = run_add(ctx, codes, np.zeros(65536, np.uint16), (65536,), "f16")
+    assert_codes_equal(got, g["add_all_codes_plus_zero"], "f16", nan_sign_free=False, what="x + 0")
+
+
+def test_golden_table_block(ctx):
+    g = golden("add")
+    rows, cols = g["add_table_rows"], g["add_table_cols"]
+    got = run_add(ctx, rows.reshape(-1, 1), cols, (rows.size, cols.size), "f16")
+    assert_codes_equal(got, g["add_table_c"], "f16", what="fp16 addition table block")
+
+
+SHAPES = [
+    # c, a, b
+    ((1000003,), (1000003,), (1000003,)),           # flat, odd length: vector body + tail
+    ((257, 4096), (257, 4096), (4096,)),            # residual-style leading broadcast
+    ((6, 1, 40), (6, 1, 40), (1, 5, 1)),            # NOT broadcastable onto c -> skipped below
+    ((7, 33, 16), (7, 1, 16), (33, 1)),             # alternating broadcast, inner vectorisable
+    ((7, 33, 15), (7, 1, 15), (33, 1)),             # same with an odd inner extent: element path
+    ((5, 6, 7, 8), (5, 6, 7, 8), (1,)),             # scalar-like operand
+    ((3, 64, 64), (64,), (3, 64, 1)),               # a broadcast along leading dims, b along inner
+    ((2, 3, 4, 5, 6, 8), (2, 1, 4, 1, 6, 8), (3, 1, 5, 1, 8)),  # six merged dims
+]
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32", "bf16"])
+@pytest.mark.parametrize("case", range(len(SHAPES)))
+def test_against_oracle(ctx, dt, case):
+    cs, as_, bs = SHAPES[case]
+    spec = lambda s: oracle.Spec(dt, s)  # noqa: E731
+    if oracle.add_check(spec(cs), spec(as_), spec(bs), allow_bf16=True) != 0:
+        pytest.skip("shape triple is not a valid broadcast (covered by the status tests)")
+    rng = np.random.default_rng(100 + case)
+    a = oracle.encode(rng.standard_normal(as_).astype(np.float32) * 3, dt)
+    b = oracle.encode(rng.standard_normal(bs).astype(np.float32) * 3, dt)
+    want = oracle.add(a, b, cs, dt)
+    got = run_add(ctx, a, b, cs, dt)
+    check(got, want, dt, f"{cs} = {as_} + {bs} {dt}")
+
+
+@pytest.mark.parametrize("which", ["a", "b"])
+def test_in_place(ctx, which):
+    import torch
+
+    rng = np.random.default_rng(5)
+    a = oracle.encode(rng.standard_normal((32, 20, 512)).astype(np.float32), "f16")
+    b = oracle.encode(rng.standard_normal((32, 20, 512)).astype(np.float32), "f16")
+    want = oracle.add(a, b, a.shape, "f16")
+    ta, tb = to_torch(a, "f16"), to_torch(b, "f16")
+    tc = ta if which == "a" else tb
+    ctx.add(tc, ta, tb)
+    torch.cuda.synchronize()
+    assert_codes_equal(to_codes(tc), want, "f16", what=f"in place on {which}")
+
+
+def test_misaligned_pointers_take_the_element_path(ctx):
+    import torch
+
+    rng = np.random.default_rng(6)
+    n = 5000
+    a = oracle.encode(rng.standard_normal(n + 3).astype(np.float32), "f16")
+    b = oracle.encode(rng.standard_normal(n + 5).astype(np.float32), "f16")
+    ta, tb = to_torch(a, "f16")[3:], to_torch(b, "f16")[5:]  # 2-byte aligned only
+    tc = torch.empty(n + 1, dtype=torch.float16, device="cuda")[1:]
+    ctx.add(tc, ta, tb)
+    torch.cuda.synchronize()
+    assert_codes_equal(to_codes(tc), oracle.add(a[3:].copy(), b[5:].copy(), (n,), "f16"), "f16", what="misaligned")
+
+
+def test_empty_tensor_is_a_no_op(ctx):
+    import torch
+
+    t = torch.empty((0, 8), dtype=torch.float16, device="cuda")
+    ctx.add(t, t, t)
+    torch.cuda.synchronize()
+
+
+def test_special_values_against_oracle(ctx):
+    """Every finite/infinite/NaN class against every other, both signs."""
+    specials = np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x03FF, 0x0400, 0x3C00, 0xBC00, 0x7BFF, 0xFBFF,
+                         0x7C00, 0xFC00, 0x7E00, 0xFE00, 0x7C01, 0x7BFE, 0x7800, 0xF800], dtype=np.uint16)
+    a = np.repeat(specials, specials.size).reshape(specials.size, specials.size)
+    b = np.ascontiguousarray(a.T)
+    want = oracle.add(a, b, a.shape, "f16")
+    got = run_add(ctx, a, b, a.shape, "f16")
+    assert_codes_equal(got, want, "f16", what="special values")
+
+
+def test_status_codes_match_reference(ctx):
+    """Create-time statuses recorded from the compiled reference."""
+    import ctypes
+
+    from operators_amd import infiniopAddDescriptor_t, make_descriptor
+    from oracle.ref import LAYOUT
+
+    lib = ctx.lib
+    for case in golden_json()["status"]:
+        if case["op"] != "add":
+            continue
+        descs = [make_descriptor(lib, t[1], t[2], LAYOUT[t[0]]) for t in case["tensors"]]
+        d = infiniopAddDescriptor_t()
+        st = lib.infiniopCreateAddDescriptor(ctx.handle, ctypes.byref(d), *descs)
+        want = 0 if case.get("bf16_extension") else case["status"]
+        assert st == want, (case, st)
+        if st == 0:
+            assert lib.infiniopDestroyAddDescriptor(d) == 0
+        for x in descs:
+            lib.infiniopDestroyTensorDescriptor(x)

@@ -1,0 +1,129 @@
+"""Create-time checks, without a GPU: the status codes recorded from the
+compiled reference (tests/golden/status_cases.json) against
+  * the oracle's restatement of the checks, and
+  * the shipped library's own host-side validation, reached through the public
+    C entry points with a hand-made handle (a handle is a plain struct whose
+    fields the create functions only read; no GPU call is made before stage 4).
+bf16 cases are this project's extension: the reference answers BAD_TENSOR_DTYPE,
+the oracle (with the extension switched on) and the library accept them."""
+import ctypes
+
+import pytest
+
+import operators_amd as oa
+import oracle
+from helpers import golden_json
+from oracle.ref import LAYOUT
+
+CASES = golden_json()["status"]
+
+
+def spec(t):
+    return oracle.Spec(t[0], t[1], t[2])
+
+
+@pytest.mark.parametrize("i", range(len(CASES)))
+def test_oracle_checks_reproduce_reference_status(i):
+    case = CASES[i]
+    specs = [spec(t) for t in case["tensors"]]
+    if case["op"] == "add":
+        st = oracle.add_check(*specs, allow_bf16=False)
+    elif case["op"] == "swiglu":
+        st = oracle.swiglu_check(*specs, allow_bf16=False)
+    elif case["op"] == "rope":
+        st = oracle.rope_check(*specs, allow_bf16=False)
+    else:
+        st = oracle.rms_norm_check(*specs)
+        if st == 0 and case.get("run"):  # the reference reports unsupported data types at compute time
+            import numpy as np
+            n, d = case["tensors"][0][1]
+            buf = np.zeros(n * d * 4, np.uint8)
+            st = oracle.lib().oracle_rms_norm(oracle.DT[case["tensors"][0][0]], oracle.DT[case["tensors"][2][0]], n, d, d, d,
+                                             ctypes.c_float(1e-5), buf.ctypes.data, buf.ctypes.data, buf.ctypes.data)
+            if case.get("bf16_extension"):
+                assert st == 0
+                return
+    assert st == case["status"], case
+    if case.get("bf16_extension") and case["op"] != "rms_norm":
+        again = {"add": oracle.add_check, "swiglu": oracle.swiglu_check, "rope": oracle.rope_check}[case["op"]](*specs, allow_bf16=True)
+        assert again == 0
+
+
+class FakeAmdContext(ctypes.Structure):
+    """Layout of the library's handle (operators_amd/csrc/devices/amd/amd_handle.h)."""
+    _fields_ = [("device", ctypes.c_int), ("device_id", ctypes.c_int), ("cu_count", ctypes.c_int),
+                ("lds_per_block", ctypes.c_int), ("max_grid_x", ctypes.c_int), ("wave_size", ctypes.c_int)]
+
+
+@pytest.fixture(scope="module")
+def fake_handle():
+    ctxt = FakeAmdContext(oa.DeviceEnum.DEVICE_AMD, 0, 256, 65536, 2 ** 31 - 1, 64)
+    return ctypes.cast(ctypes.pointer(ctxt), oa.infiniopHandle_t), ctxt
+
+
+CREATE = {
+    "add": ("infiniopCreateAddDescriptor", "infiniopDestroyAddDescriptor", oa.infiniopAddDescriptor_t),
+    "swiglu": ("infiniopCreateSwiGLUDescriptor", "infiniopDestroySwiGLUDescriptor", oa.infiniopSwiGLUDescriptor_t),
+    "rope": ("infiniopCreateRoPEDescriptor", "infiniopDestroyRoPEDescriptor", oa.infiniopRoPEDescriptor_t),
+    "rms_norm": ("infiniopCreateRMSNormDescriptor", "infiniopDestroyRMSNormDescriptor", oa.infiniopRMSNormDescriptor_t),
+}
+
+
+@pytest.mark.parametrize("i", range(len(CASES)))
+def test_library_host_validation_reproduces_reference_status(fake_handle, i):
+    case = CASES[i]
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    create, destroy, dtype = CREATE[case["op"]]
+    descs = [oa.make_descriptor(lib, t[1], t[2], LAYOUT[t[0]]) for t in case["tensors"]]
+    d = dtype()
+    extra = (ctypes.c_float(1e-5),) if case["op"] == "rms_norm" else ()
+    st = getattr(lib, create)(handle, ctypes.byref(d), *descs, *extra)
+    if case["op"] == "rms_norm" and case.get("run"):
+        # the dtype verdict comes at compute time, as in the reference; on a
+        # machine without a GPU only the "unsupported type" answer can be
+        # observed, because it is given before anything touches the device
+        assert st == 0
+        if case["status"] == 3 and not case.get("bf16_extension"):
+            assert lib.infiniopRMSNorm(d, None, 0, None, None, None, None) == 3
+        want = 0
+    else:
+        want = 0 if case.get("bf16_extension") else case["status"]
+    assert st == want, (case, st)
+    if st == 0:
+        size = ctypes.c_uint64(7)
+        if case["op"] == "rms_norm":
+            assert lib.infiniopGetRMSNormWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
+        if case["op"] == "rope":
+            assert lib.infiniopGetRoPEWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
+        assert getattr(lib, destroy)(d) == 0
+    for x in descs:
+        lib.infiniopDestroyTensorDescriptor(x)
+
+
+def test_descriptor_starts_with_device_number(fake_handle):
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    descs = [oa.make_descriptor(lib, (4, 8), None, oa.F16) for _ in range(3)]
+    d = oa.infiniopAddDescriptor_t()
+    assert lib.infiniopCreateAddDescriptor(handle, ctypes.byref(d), *descs) == 0
+    assert d.contents.device == oa.DeviceEnum.DEVICE_AMD
+    assert lib.infiniopDestroyAddDescriptor(d) == 0
+    # a handle of another device is refused by every create function
+    other = FakeAmdContext(oa.DeviceEnum.DEVICE_CPU, 0, 1, 1, 1, 1)
+    assert lib.infiniopCreateAddDescriptor(ctypes.cast(ctypes.pointer(other), oa.infiniopHandle_t), ctypes.byref(d), *descs) == 8
+    d2 = oa.infiniopSwiGLUDescriptor_t()
+    assert lib.infiniopCreateSwiGLUDescriptor(ctypes.cast(ctypes.pointer(other), oa.infiniopHandle_t), ctypes.byref(d2), *descs) == 8
+    for x in descs:
+        lib.infiniopDestroyTensorDescriptor(x)
+
+
+def test_null_output_pointer_is_memory_not_allocated(fake_handle):
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    t = oa.make_descriptor(lib, (4, 2, 8), None, oa.F16)
+    p = oa.make_descriptor(lib, (4,), None, oa.U64)
+    s = oa.make_descriptor(lib, (16, 8), None, oa.F32)
+    assert lib.infiniopCreateRoPEDescriptor(handle, None, t, p, s, s) == 6  # rotary_embedding_cpu.cc:54-55
+    for x in (t, p, s):
+        lib.infiniopDestroyTensorDescriptor(x)
