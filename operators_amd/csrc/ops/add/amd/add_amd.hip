@@ -16,8 +16,17 @@ namespace {
 
 using namespace amd;
 
-constexpr int kBlock = 256;// 4 wavefronts
-constexpr int kUnroll = 4; // independent 16-byte accesses per lane per operand
+#ifndef ADD_BLOCK
+#define ADD_BLOCK 256
+#endif
+#ifndef ADD_UNROLL
+#define ADD_UNROLL 4
+#endif
+#ifndef ADD_PER_CU
+#define ADD_PER_CU 32
+#endif
+constexpr int kBlock = ADD_BLOCK;  // lanes per workgroup
+constexpr int kUnroll = ADD_UNROLL;// independent 16-byte accesses per lane per operand
 
 // ---- per-type arithmetic on one 128-bit word ---------------------------------
 template<typename T>
@@ -139,22 +148,35 @@ __device__ __forceinline__ void bcast_offsets(const BcastDims &d, Idx pos, Idx i
     }
 }
 
+// How an operand is addressed by the vector form.
+//   kFull : it has c's full shape, so its offset is c's flat offset; it is
+//           touched once and streams past the caches like c.
+//   kRuns : stride 1 along the innermost dimension but broadcast along some
+//           outer one; 128-bit loads through the caches, because every
+//           element is wanted again by other lanes.
+//   kStill: broadcast along the innermost dimension; one element, replicated.
+enum OperandMode { kFull = 0, kRuns = 1, kStill = 2 };
+
+template<typename Op, int MODE>
+__device__ __forceinline__ u32x4 fetch_operand(const typename Op::scalar *p, uint64_t flat_vec, int64_t offset) {
+    if constexpr (MODE == kFull) return ld16_stream(p + flat_vec * Op::kPerVec);
+    else if constexpr (MODE == kRuns) return ld16(p + offset);
+    else return Op::splat(p[offset]);
+}
+
 // Vector form: the innermost merged dimension is a multiple of the vector
 // width and each operand either runs along it with stride 1 (128-bit load) or
-// stands still (one element, replicated).  A_RUNS / B_RUNS say which.
-template<typename Op, typename Idx, bool A_RUNS, bool B_RUNS>
+// stands still (one element, replicated).
+template<typename Op, typename Idx, int A_MODE, int B_MODE>
 __global__ __launch_bounds__(kBlock) void add_bcast_vec(u32x4 *c, const typename Op::scalar *a,
                                                         const typename Op::scalar *b, BcastDims d, uint64_t nvec) {
     const Idx inner_vecs = static_cast<Idx>(d.shape[0] / Op::kPerVec);
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
     for (uint64_t v = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; v < nvec; v += step) {
-        int64_t oa, ob;
+        int64_t oa = 0, ob = 0;
         bcast_offsets<Idx>(d, static_cast<Idx>(v), inner_vecs, Op::kPerVec, oa, ob);
-        u32x4 va, vb;
-        if constexpr (A_RUNS) va = ld16_stream(a + oa);
-        else va = Op::splat(a[oa]);
-        if constexpr (B_RUNS) vb = ld16_stream(b + ob);
-        else vb = Op::splat(b[ob]);
+        const u32x4 va = fetch_operand<Op, A_MODE>(a, v, oa);
+        const u32x4 vb = fetch_operand<Op, B_MODE>(b, v, ob);
         st16_stream(c + v, Op::vec(va, vb));
     }
 }
@@ -175,7 +197,7 @@ __global__ __launch_bounds__(kBlock) void add_bcast_scalar(typename Op::scalar *
 // ---- launch -------------------------------------------------------------------
 inline unsigned grid_for(uint64_t work_items, uint64_t per_block, int cu_count, int blocks_per_cu) {
     const uint64_t want = ceil_div(work_items, per_block);
-    const uint64_t cap = static_cast<uint64_t>(cu_count) * blocks_per_cu;
+    const uint64_t cap = blocks_per_cu > 0 ? static_cast<uint64_t>(cu_count) * blocks_per_cu : want;
     const uint64_t g = want < cap ? want : cap;
     return static_cast<unsigned>(g == 0 ? 1 : g);
 }
@@ -191,7 +213,7 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         if (aligned16(c) && aligned16(a) && aligned16(b)) {
             const uint64_t nvec = n / Op::kPerVec;
             if (nvec > 0) {
-                const unsigned grid = grid_for(nvec, static_cast<uint64_t>(kBlock) * kUnroll, cus, 32);
+                const unsigned grid = grid_for(nvec, static_cast<uint64_t>(kBlock) * kUnroll, cus, ADD_PER_CU);
                 add_flat_vec<Op><<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const u32x4 *>(a),
                                                               static_cast<const u32x4 *>(b), nvec);
             }
@@ -230,22 +252,38 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
 
     if (vec_ok) {
         const uint64_t nvec = n / w;
-        const unsigned grid = grid_for(nvec, kBlock, cus, 64);
+        const unsigned grid = grid_for(nvec, kBlock, cus, ADD_PER_CU > 0 ? 64 : 0);
+        auto mode_of = [&](const int64_t *stride) {
+            if (stride[0] == 0) return static_cast<int>(kStill);
+            for (int k = 1; k < desc.ndim; ++k)
+                if (stride[k] == 0) return static_cast<int>(kRuns);
+            return static_cast<int>(kFull);
+        };
+        const int ma = mode_of(desc.a_stride), mb = mode_of(desc.b_stride);
         auto go = [&](auto kernel) {
             kernel<<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const S *>(a), static_cast<const S *>(b), d, nvec);
         };
-        if (small) {
-            if (a_runs && b_runs) go(add_bcast_vec<Op, uint32_t, true, true>);
-            else if (a_runs) go(add_bcast_vec<Op, uint32_t, true, false>);
-            else if (b_runs) go(add_bcast_vec<Op, uint32_t, false, true>);
-            else go(add_bcast_vec<Op, uint32_t, false, false>);
-        } else {
-            if (a_runs && b_runs) go(add_bcast_vec<Op, uint64_t, true, true>);
-            else if (a_runs) go(add_bcast_vec<Op, uint64_t, true, false>);
-            else if (b_runs) go(add_bcast_vec<Op, uint64_t, false, true>);
-            else go(add_bcast_vec<Op, uint64_t, false, false>);
-        }
-    } else {
+        bool launched = false;
+#define ADD_BCAST_CASE(MA, MB)                                        \
+    if (ma == MA && mb == MB) {                                       \
+        if (small) go(add_bcast_vec<Op, uint32_t, MA, MB>);           \
+        else go(add_bcast_vec<Op, uint64_t, MA, MB>);                 \
+        launched = true;                                              \
+    }
+        ADD_BCAST_CASE(kFull, kRuns)
+        ADD_BCAST_CASE(kFull, kStill)
+        ADD_BCAST_CASE(kRuns, kFull)
+        ADD_BCAST_CASE(kRuns, kRuns)
+        ADD_BCAST_CASE(kRuns, kStill)
+        ADD_BCAST_CASE(kStill, kFull)
+        ADD_BCAST_CASE(kStill, kRuns)
+        ADD_BCAST_CASE(kStill, kStill)
+#undef ADD_BCAST_CASE
+        if (launched) return STATUS_SUCCESS;
+        // two full operands that did not merge into one flat range cannot reach
+        // this point; if a new layout ever does, the element form below handles it
+    }
+    {
         const unsigned grid = grid_for(n, kBlock, cus, 64);
         if (small) {
             add_bcast_scalar<Op, uint32_t><<<grid, kBlock, 0, stream>>>(static_cast<S *>(c), static_cast<const S *>(a),

@@ -18,11 +18,42 @@ namespace {
 
 using namespace amd;
 
-constexpr int kBlock = 256;
-constexpr int kUnroll = 2;// independent 16-byte accesses per lane per operand
+#ifndef SWIGLU_BLOCK
+#define SWIGLU_BLOCK 256
+#endif
+#ifndef SWIGLU_UNROLL
+#define SWIGLU_UNROLL 1
+#endif
+#ifndef SWIGLU_MATH
+#define SWIGLU_MATH 3
+#endif
+#ifndef SWIGLU_PER_CU
+#define SWIGLU_PER_CU 0
+#endif
+constexpr int kBlock = SWIGLU_BLOCK;
+constexpr int kUnroll = SWIGLU_UNROLL;// independent 16-byte accesses per lane per operand
 
 __device__ __forceinline__ float swiglu1(float up, float gate) {
+#if SWIGLU_MATH == 0
     return up * (gate / (1.0f + expf(-gate)));
+#else
+    // e = exp(-gate) through the hardware exp2.  gate has at most 11 significant
+    // bits and the high part of log2(e) below has 12, so t is exact.
+    constexpr float kL2eHi = 1.44287109375f;            // log2(e) rounded to 12 bits
+    constexpr float kL2eLoLn2 = -1.2203054e-4f;         // (log2(e) - kL2eHi) * ln 2
+    float t = fminf(gate * -kL2eHi, 126.0f);
+    float e = __builtin_amdgcn_exp2f(t);
+#if SWIGLU_MATH >= 2
+    e = __builtin_fmaf(e, gate * -kL2eLoLn2, e);
+#endif
+    const float d = 1.0f + e;
+    const float r = __builtin_amdgcn_rcpf(d);
+    float q = gate * r;
+#if SWIGLU_MATH >= 3
+    q = __builtin_fmaf(__builtin_fmaf(-d, q, gate), r, q);
+#endif
+    return up * q;
+#endif
 }
 
 template<typename T>
@@ -117,7 +148,7 @@ void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const v
     const uint64_t nvec = n / 8;
     const uint64_t vpr = d.di / 8;
     const uint64_t want = ceil_div(nvec, static_cast<uint64_t>(kBlock) * kUnroll);
-    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * 32;
+    const uint64_t cap = SWIGLU_PER_CU > 0 ? static_cast<uint64_t>(d.cu_count) * SWIGLU_PER_CU : want;
     const unsigned grid = static_cast<unsigned>(want < cap ? want : cap);
     // One row, or every row stride equal to the width: the tensors are dense.
     const bool dense = d.rows == 1 || (d.stride_a == di && d.stride_b == di && d.stride_c == di);
