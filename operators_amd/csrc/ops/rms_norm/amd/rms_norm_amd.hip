@@ -22,16 +22,6 @@ namespace {
 
 using namespace amd;
 
-#ifndef RMS_PREFETCH
-#define RMS_PREFETCH 1
-#endif
-#ifndef RMS_WHOME
-#define RMS_WHOME 1
-#endif
-#ifndef RMS_PER_CU
-#define RMS_PER_CU 8
-#endif
-
 // ---- weight row access ----------------------------------------------------------
 struct WF32 {
     typedef float scalar;
@@ -66,18 +56,25 @@ __device__ __forceinline__ float inv_rms(float sum_sq, uint64_t d, float eps) {
 // always in flight while the reduction, the barrier and the stores happen.
 //
 // Where the weight row lives while a workgroup works through its rows:
-//   kWGlobal: re-read from memory for every row (one row per workgroup)
+//   kWGlobal: re-read from memory for every row (one row per workgroup, or a
+//             row too long for LDS)
 //   kWLds   : staged once in LDS as fp32
-//   kWRegs  : the 8*NV weights of this lane's columns, kept in registers
+// (Keeping each lane's 8*NV weights in registers instead was measured and is
+// no faster: 47.3 vs 47.5 us at [8192, 8192] bf16 with fp32 weights.)
 //
 // LDS layout of the staged weight row: the 8 floats of vector v are split into
 // two 16-byte halves stored at lo[v] and hi[v] (hi = lo + nvec).  A wavefront
 // reading lo[v..v+63] or hi[v..v+63] then touches 64 consecutive 16-byte words
 // - no two lanes on the same bank in the same phase - where the natural
 // 32-byte-per-lane layout would be a two-way conflict.
-enum WeightHome { kWGlobal = 0, kWLds = 1, kWRegs = 2 };
+enum WeightHome { kWGlobal = 0, kWLds = 1 };
 
-template<typename T, typename W, int BS, int NV, int WHOME>
+// EXACT means d == 8*BS*NV: every lane owns NV whole vectors and no access is
+// predicated.  Otherwise loads of absent vectors are redirected to vector 0
+// (and their value replaced by zero) rather than branched around: with
+// straight-line loads the compiler can count how many are still in flight and
+// wait for the current row only, not for the prefetched one.
+template<typename T, typename W, int BS, int NV, int WHOME, bool EXACT>
 __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w,
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps) {
     constexpr int WAVES = BS / kWave;
@@ -87,7 +84,20 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
     const uint32_t nvec = d / 8;
     f32x4 *w_hi = w_lo + nvec;
 
-    float wreg[WHOME == kWRegs ? NV : 1][8];
+    auto load_row = [&](uint64_t row, u32x4(&dst)[NV]) {
+        const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            dst[k] = ld16_stream(xr + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
+        }
+    };
+
+    uint64_t row = blockIdx.x;
+    if (row >= n) return;
+    u32x4 xv[NV], xn[NV];
+    load_row(row, xv);// in flight while the weights are fetched below
+
     if constexpr (WHOME == kWLds) {
         for (uint32_t v = threadIdx.x; v < nvec; v += BS) {
             float g[8];
@@ -96,62 +106,39 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
             w_hi[v] = f32x4{g[4], g[5], g[6], g[7]};
         }
         __syncthreads();
-    } else if constexpr (WHOME == kWRegs) {
-#pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
-            if (v < nvec) W::load8(w, v, wreg[k]);
-        }
     }
 
-    auto load_row = [&](uint64_t row, u32x4(&dst)[NV]) {
-        const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
-#pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
-            dst[k] = v < nvec ? ld16_stream(xr + static_cast<uint64_t>(v) * 8) : u32x4{0, 0, 0, 0};
-        }
-    };
-
-    uint64_t row = blockIdx.x;
-    u32x4 xv[NV], xn[NV];
-    if (row < n) load_row(row, xv);
-    int phase = 0;
-    for (; row < n; row += gridDim.x, phase ^= 1) {
-        const uint64_t next = row + gridDim.x;
-#if RMS_PREFETCH
-        if (next < n) load_row(next, xn);
-#endif
+    // One row: reduce, scale by the weights, store.
+    auto finish_row = [&](uint64_t r, const u32x4(&cur)[NV], int phase) {
         float part = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             float f[8];
-            widen8<T>(xv[k], f);
+            widen8<T>(cur[k], f);
+            if constexpr (!EXACT) {
+                if (k * BS + threadIdx.x >= nvec) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) f[i] = 0.0f;
+                }
+            }
             // pairwise inside the vector, then onto the running partial
             const float s01 = f[0] * f[0] + f[1] * f[1], s23 = f[2] * f[2] + f[3] * f[3];
             const float s45 = f[4] * f[4] + f[5] * f[5], s67 = f[6] * f[6] + f[7] * f[7];
             part += (s01 + s23) + (s45 + s67);
         }
-#ifdef RMS_DBG_NOREDUCE
-        const float k_row = part > 1e30f ? 2.0f : 1.0f;
-#else
         const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
-#endif
 
-        uint16_t *yr = y + static_cast<int64_t>(row) * stride_y;
+        uint16_t *yr = y + static_cast<int64_t>(r) * stride_y;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = k * BS + threadIdx.x;
-            if (v < nvec) {
+            if (EXACT || v < nvec) {
                 float f[8], g[8];
-                widen8<T>(xv[k], f);
+                widen8<T>(cur[k], f);
                 if constexpr (WHOME == kWLds) {
                     const f32x4 a = w_lo[v], b = w_hi[v];
                     g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
                     g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
-                } else if constexpr (WHOME == kWRegs) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) g[i] = wreg[k][i];
                 } else {
                     W::load8(w, v, g);
                 }
@@ -160,12 +147,28 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
                 st16_stream(yr + static_cast<uint64_t>(v) * 8, narrow8<T>(f));
             }
         }
-#if RMS_PREFETCH
-#pragma unroll
-        for (int k = 0; k < NV; ++k) xv[k] = xn[k];
-#else
-        if (next < n) load_row(next, xv);
-#endif
+    };
+
+    // Steady state: the next row's loads are issued, unconditionally, before
+    // the current row is reduced.  Two register sets take turns (no copies, so
+    // the wait for a prefetched row comes only when that row is reduced) and a
+    // row's loads are never issued unless this workgroup owns that row.
+    const uint64_t hop = gridDim.x;
+    while (true) {
+        if (row + hop >= n) {
+            finish_row(row, xv, 0);
+            break;
+        }
+        load_row(row + hop, xn);
+        finish_row(row, xv, 0);
+        row += hop;
+        if (row + hop >= n) {
+            finish_row(row, xn, 1);
+            break;
+        }
+        load_row(row + hop, xv);
+        finish_row(row, xn, 1);
+        row += hop;
     }
 }
 
@@ -216,15 +219,13 @@ void launch_rms_norm(const RMSNormAmdDescriptor &desc, void *y, const void *x, c
     // unit, else it re-reads them from memory like a one-row workgroup does.
     const uint64_t lds_bytes = d * sizeof(float);
     const uint64_t lds_limit = static_cast<uint64_t>(desc.lds_per_block) - 1024;
-    uint64_t per_cu = RMS_PER_CU;
-    int home = RMS_WHOME;
-    if (home == kWLds) {
-        if (lds_bytes <= lds_limit && lds_bytes <= 64 * 1024) {
-            const uint64_t fit = (160 * 1024) / (lds_bytes + 256);
-            per_cu = fit < per_cu ? fit : per_cu;
-        } else {
-            home = kWGlobal;
-        }
+    uint64_t per_cu = 8;// workgroups per compute unit when LDS is not the limit
+    int home = kWLds;
+    if (lds_bytes <= lds_limit && lds_bytes <= 64 * 1024) {
+        const uint64_t fit = (160 * 1024) / (lds_bytes + 256);// 160 KiB of LDS per compute unit
+        per_cu = fit < per_cu ? fit : per_cu;
+    } else {
+        home = kWGlobal;
     }
     uint64_t grid = static_cast<uint64_t>(desc.cu_count) * per_cu;
     if (n <= grid) {
@@ -233,12 +234,17 @@ void launch_rms_norm(const RMSNormAmdDescriptor &desc, void *y, const void *x, c
     }
 
 #define RMS_LAUNCH_HOME(BS, NV, HOME, LDS)                                                                              \
-    rms_norm_rows<T, W, BS, NV, HOME><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(                                \
-        py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon)
+    do {                                                                                                                \
+        if (nvec == static_cast<uint64_t>(BS) * NV)                                                                     \
+            rms_norm_rows<T, W, BS, NV, HOME, true><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(                  \
+                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon);                    \
+        else                                                                                                            \
+            rms_norm_rows<T, W, BS, NV, HOME, false><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(                 \
+                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon);                    \
+    } while (0)
 #define RMS_LAUNCH(BS, NV)                                                                                              \
     do {                                                                                                                \
         if (home == kWLds) RMS_LAUNCH_HOME(BS, NV, kWLds, lds_bytes);                                                   \
-        else if (home == kWRegs) RMS_LAUNCH_HOME(BS, NV, kWRegs, 0);                                                    \
         else RMS_LAUNCH_HOME(BS, NV, kWGlobal, 0);                                                                      \
     } while (0)
 
@@ -246,11 +252,7 @@ void launch_rms_norm(const RMSNormAmdDescriptor &desc, void *y, const void *x, c
     else if (nvec <= 128) RMS_LAUNCH(128, 1);
     else if (nvec <= 256) RMS_LAUNCH(256, 1);
     else if (nvec <= 512) RMS_LAUNCH(256, 2);
-#if defined(RMS_BS8K) && defined(RMS_NV8K) // experiment hook
-    else if (nvec <= 1024) RMS_LAUNCH(RMS_BS8K, RMS_NV8K);
-#else
-    else if (nvec <= 1024) RMS_LAUNCH(256, 4);
-#endif
+    else if (nvec <= 1024) RMS_LAUNCH(256, 4);// d = 8192: 512x2 measures the same, 1024x1 is 8 % slower
     else if (nvec <= 2048) RMS_LAUNCH(512, 4);
     else if (nvec <= 4096) RMS_LAUNCH(1024, 4);
     else RMS_LAUNCH(1024, 8);
