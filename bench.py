@@ -31,6 +31,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 
+# HBM bytes per launch of the dominant kernel at the default workload
+# (swiglu bf16 [8192, 28672] from a fused [8192, 57344] buffer), measured with
+# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each scaled by what the same
+# counter reads for a plain 128 MiB device copy (1.99959 and 1.00000); the runs
+# are summarised in profiles/c5_kernels_hbm_traffic_pmc.txt.  Algorithmic bytes
+# for the same launch: 1 409 286 144.
+MEASURED_TRAFFIC_SWIGLU_8192 = 1409141790
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -337,8 +345,9 @@ def main():
     sw_bytes = sets[0][3].nbytes
     roofline = {
         "bound": "hbm", "achieved": round(sw_bytes / sw_time / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": round(sw_bytes / sw_time / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
-        "kernel": f"swiglu_vec<bf16, row-strided> [{T},28672] from fused [{T},57344]",
+        "frac": round(sw_bytes / sw_time / 1e9 / HBM_PEAK_GBPS, 4),
+        "traffic": MEASURED_TRAFFIC_SWIGLU_8192 if T == 8192 else None,
+        "kernel": f"swiglu_rows<bf16> [{T},28672] from fused [{T},57344]",
         "bytes_per_launch": sw_bytes, "us_per_launch": round(sw_time * 1e6, 2),
     }
     per_op_chain = {l.name: l.nbytes for l in sets[0]}

@@ -59,8 +59,10 @@ __device__ __forceinline__ float inv_rms(float sum_sq, uint64_t d, float eps) {
 //   kWGlobal: re-read from memory for every row (one row per workgroup, or a
 //             row too long for LDS)
 //   kWLds   : staged once in LDS as fp32
-// (Keeping each lane's 8*NV weights in registers instead was measured and is
-// no faster: 47.3 vs 47.5 us at [8192, 8192] bf16 with fp32 weights.)
+// Measured at [8192, 8192] bf16 with fp32 weights: 45.7 us with the weights in
+// LDS, 47.0-50.6 us when every row re-reads them through L2 (one workgroup per
+// row, or 8-16 looping workgroups per compute unit); keeping each lane's 8*NV
+// weights in registers instead of LDS is no faster than LDS.
 //
 // LDS layout of the staged weight row: the 8 floats of vector v are split into
 // two 16-byte halves stored at lo[v] and hi[v] (hi = lo + nvec).  A wavefront
@@ -219,7 +221,13 @@ void launch_rms_norm(const RMSNormAmdDescriptor &desc, void *y, const void *x, c
     // unit, else it re-reads them from memory like a one-row workgroup does.
     const uint64_t lds_bytes = d * sizeof(float);
     const uint64_t lds_limit = static_cast<uint64_t>(desc.lds_per_block) - 1024;
-    uint64_t per_cu = 8;// workgroups per compute unit when LDS is not the limit
+    // With the next row always in flight, one workgroup per compute unit already
+    // reaches the bandwidth this access pattern allows (measured at [8192, 8192]
+    // bf16: 1, 2, 3 and 4 per unit all give 73.3-74.0 % of peak); 2 keeps some
+    // slack while staging the weights only 512 times.  Shorter rows put fewer
+    // bytes in flight per workgroup, so they get proportionally more of them.
+    uint64_t per_cu = ceil_div(32 * 1024, d * sizeof(uint16_t));
+    per_cu = per_cu < 2 ? 2 : (per_cu > 16 ? 16 : per_cu);
     int home = kWLds;
     if (lds_bytes <= lds_limit && lds_bytes <= 64 * 1024) {
         const uint64_t fit = (160 * 1024) / (lds_bytes + 256);// 160 KiB of LDS per compute unit

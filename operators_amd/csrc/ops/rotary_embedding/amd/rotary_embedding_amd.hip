@@ -12,8 +12,10 @@
 // are bit-identical to the CPU's.  bf16 (extension) rounds to nearest even.
 //
 // t is read and written exactly once through arbitrary token/head strides;
-// the table rows of a token are fetched once per lane and reused for every
-// head that lane rotates.
+// the table rows of a token are fetched once per lane, through the caches, and
+// reused for every head that lane rotates.  (Staging the rows in LDS with one
+// head per lane was measured on MI355X and is slower: 52.7 against 48.9 us at
+// q = [8192, 64, 128] bf16.)
 #include "../../../devices/amd/kernel_amd.h"
 #include "rotary_embedding_amd.h"
 

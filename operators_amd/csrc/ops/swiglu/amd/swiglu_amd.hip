@@ -4,7 +4,7 @@
 //     c = narrow( a * ( b / (1 + expf(-b)) ) )       all in fp32,
 // b gated, a linear; fp16 narrows with the reference's truncating conversion,
 // bf16 (extension) rounds to nearest even.  The fp32 value is computed to
-// within about one unit in its last place of the CPU's (see swiglu1).
+// within about one unit in its last place of the CPU's (see swiglu1_lean).
 //
 // Three streams (two in, one out) and about 20 VALU slots per element:
 // bandwidth bound, but only just - the arithmetic is kept lean on purpose.  Rows are addressed through one row stride per tensor, so the same
@@ -23,26 +23,35 @@ constexpr int kBlock = 256;
 // for this kernel (77 % vs 74 % of the 8 TB/s peak at [8192, 28672] bf16).
 constexpr int kUnroll = 1;
 
-// up * gate / (1 + exp(-gate)) with two hardware transcendentals (exp2, rcp)
-// and three correction steps instead of libm's expf and an IEEE division.
-// The library routines cost about 35 VALU slots per element, which at 6 bytes
-// of traffic per element is more than the memory system leaves time for (the
-// kernel ran at 64 % of peak, compute bound); this form costs about 20.
+// The reference's formula with the library routines: expf and an IEEE
+// division.  About 35 VALU slots per element - more than the memory system
+// leaves time for at 6 bytes of traffic per element (a kernel built on this
+// alone ran at 64 % of peak, compute bound) - so it serves only the rare
+// elements the lean form below does not cover, and the element-wise fallback.
+__device__ __forceinline__ float swiglu1_any(float up, float gate) {
+    return up * (gate / (1.0f + expf(-gate)));
+}
+
+// The same value for |gate| <= 87 with two hardware transcendentals (exp2,
+// rcp) and three correction steps, about 20 VALU slots per element.
 //  - gate has at most 11 significant bits (it was an fp16 or bf16 value) and
 //    kL2eHi has 11, so t = gate * -kL2eHi is exact; the rest of log2(e) enters
-//    as the first-order factor (1 + gate * c) on the result of exp2.
-//  - t is capped at 126 so that e stays finite and the quotient's correction
-//    step never sees inf * 0; for such gates (< -87) the result is far below
-//    the smallest fp16 subnormal either way.
+//    as the first-order factor (1 + gate * c) on the result of exp2.  The
+//    neglected second-order term is (gate * 1.22e-4)^2 / 2 relative to e:
+//    below one fp32 ulp for |gate| < 3, 5e-7 at |gate| = 8, and where it grows
+//    further (gate < -10) the result is already in fp16's subnormal range or
+//    below, where one unit in the last place is far coarser than that.
+//  - |gate| <= 87 keeps e = exp(-gate) finite and normal, so the quotient's
+//    correction step never meets inf * 0.
 //  - q = gate * rcp(d) is refined once with the exact residual gate - d*q.
 // Against the CPU's expf-and-divide the narrowed fp16 result differs by one
 // unit in the last place on 2 to 9 elements in 10^5 (N(0,1) and N(0,16)
 // inputs), never by more; the library-routine form differs on 4 to 6 in 10^6.
-__device__ __forceinline__ float swiglu1(float up, float gate) {
+constexpr float kLeanGateLimit = 87.0f;
+__device__ __forceinline__ float swiglu1_lean(float up, float gate) {
     constexpr float kL2eHi = 1.44287109375f;   // log2(e) rounded to 11 bits
     constexpr float kL2eLoLn2 = -1.2203054e-4f;// (log2(e) - kL2eHi) * ln 2
-    const float t = fminf(gate * -kL2eHi, 126.0f);
-    float e = __builtin_amdgcn_exp2f(t);
+    float e = __builtin_amdgcn_exp2f(gate * -kL2eHi);
     e = __builtin_fmaf(e, gate * -kL2eLoLn2, e);
     const float d = 1.0f + e;
     const float r = __builtin_amdgcn_rcpf(d);
@@ -51,13 +60,29 @@ __device__ __forceinline__ float swiglu1(float up, float gate) {
     return up * q;
 }
 
+// Eight elements.  Gates beyond the lean form's range (|gate| > 87, infinities,
+// NaNs - none of which occur in activations of ordinary scale) send the whole
+// wavefront through the library form; the test is wave-uniform, so the lean
+// path carries no divergent branches.
 template<typename T>
 __device__ __forceinline__ u32x4 swiglu8(u32x4 va, u32x4 vb) {
     float up[8], gate[8];
     widen8<T>(va, up);
     widen8<T>(vb, gate);
+    bool out_of_range = false;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) up[i] = swiglu1(up[i], gate[i]);
+    for (int i = 0; i < 8; ++i) out_of_range |= !(fabsf(gate[i]) <= kLeanGateLimit);
+    if (__builtin_amdgcn_ballot_w64(out_of_range) == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) up[i] = swiglu1_lean(up[i], gate[i]);
+    } else {
+        // An empty volatile statement: it cannot be executed speculatively, so
+        // the compiler keeps this side a real (wave-uniform) branch instead of
+        // computing both forms for every element and selecting afterwards.
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < 8; ++i) up[i] = swiglu1_any(up[i], gate[i]);
+    }
     return narrow8<T>(up);
 }
 
@@ -108,6 +133,23 @@ __global__ __launch_bounds__(kBlock) void swiglu_vec(uint16_t *c, const uint16_t
     }
 }
 
+// Row-strided tensors whose rows hold at least a workgroup of vectors:
+// blockIdx.y walks the rows and blockIdx.x the row's vectors, so no lane
+// divides anything and no workgroup straddles two rows.
+template<typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_rows(uint16_t *c, const uint16_t *a, const uint16_t *b,
+                                                       uint64_t rows, uint32_t vecs_per_row,
+                                                       int64_t stride_c, int64_t stride_a, int64_t stride_b) {
+    const uint32_t col = blockIdx.x * kBlock + threadIdx.x;
+    if (col >= vecs_per_row) return;
+    const int64_t e = static_cast<int64_t>(col) * 8;
+    for (uint64_t row = blockIdx.y; row < rows; row += gridDim.y) {
+        const u32x4 va = ld16_stream(a + static_cast<int64_t>(row) * stride_a + e);
+        const u32x4 vb = ld16_stream(b + static_cast<int64_t>(row) * stride_b + e);
+        st16_stream(c + static_cast<int64_t>(row) * stride_c + e, swiglu8<T>(va, vb));
+    }
+}
+
 // Any width, any alignment: one element per lane per step.
 template<typename T>
 __global__ __launch_bounds__(kBlock) void swiglu_scalar(uint16_t *c, const uint16_t *a, const uint16_t *b,
@@ -119,7 +161,7 @@ __global__ __launch_bounds__(kBlock) void swiglu_scalar(uint16_t *c, const uint1
         const uint64_t row = i / di, col = i - row * di;
         const float up = T::one(a[static_cast<int64_t>(row) * stride_a + col]);
         const float gate = T::one(b[static_cast<int64_t>(row) * stride_b + col]);
-        c[static_cast<int64_t>(row) * stride_c + col] = T::narrow1(swiglu1(up, gate));
+        c[static_cast<int64_t>(row) * stride_c + col] = T::narrow1(swiglu1_any(up, gate));
     }
 }
 
@@ -148,6 +190,13 @@ void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const v
     // One row, or every row stride equal to the width: the tensors are dense.
     const bool dense = d.rows == 1 || (d.stride_a == di && d.stride_b == di && d.stride_c == di);
     const bool small = nvec < (1ull << 31);
+    // Measured at [8192, 28672] bf16 from a fused [8192, 57344] buffer: 216 us
+    // with the row form against 226 us with the flat index split by division.
+    if (!dense && vpr >= kBlock && vpr < (1ull << 31)) {
+        const dim3 g(static_cast<unsigned>(ceil_div(vpr, kBlock)), static_cast<unsigned>(d.rows < 65535 ? d.rows : 65535));
+        swiglu_rows<T><<<g, kBlock, 0, stream>>>(pc, pa, pb, d.rows, static_cast<uint32_t>(vpr), d.stride_c, d.stride_a, d.stride_b);
+        return;
+    }
     if (dense) {
         swiglu_vec<T, uint64_t, false><<<grid, kBlock, 0, stream>>>(pc, pa, pb, nvec, vpr, d.stride_c, d.stride_a, d.stride_b);
     } else if (small) {

@@ -109,6 +109,36 @@ def test_closed_forms(ctx):
     assert abs(got[4]) < 1e-10 and got[5] == 0
 
 
+def test_every_fp16_gate_code(ctx):
+    """All 65 536 gate codes (subnormals, huge magnitudes, infinities, NaNs)
+    against four `up` values: exercises the range test that routes extreme
+    gates to the library formula."""
+    import torch
+
+    gates = np.arange(65536, dtype=np.uint16)
+    for up_value in (1.0, -2.5, 300.0, 6.1e-5):
+        b = gates.reshape(64, 1024)
+        a = oracle.encode(np.full((64, 1024), up_value, np.float32), "f16")
+        tc = torch.empty((64, 1024), dtype=torch.float16, device="cuda")
+        ctx.swiglu(tc, to_torch(a, "f16"), to_torch(b, "f16"))
+        torch.cuda.synchronize()
+        want = oracle.swiglu(a, b, "f16")
+        frac, worst = assert_codes_close(to_codes(tc), want, "f16", max_ulp=1, max_frac=2e-3, what=f"all gate codes, up={up_value}")
+
+
+def test_bf16_extreme_gates(ctx):
+    """bf16 gates far outside the lean form's range, both signs, plus inf/NaN."""
+    import torch
+
+    gate_values = np.array([88.0, -88.0, 90.0, -90.0, 1e4, -1e4, 3e38, -3e38, np.inf, -np.inf, np.nan, 87.0, -87.0, 86.5, -86.5, 0.0], np.float32)
+    b = oracle.encode(np.tile(gate_values, (8, 64)), "bf16")
+    a = oracle.encode(np.full(b.shape, 1.25, np.float32), "bf16")
+    tc = torch.empty(b.shape, dtype=torch.bfloat16, device="cuda")
+    ctx.swiglu(tc, to_torch(a, "bf16"), to_torch(b, "bf16"))
+    torch.cuda.synchronize()
+    assert_codes_close(to_codes(tc), oracle.swiglu(a, b, "bf16"), "bf16", max_ulp=1, max_frac=0.2, what="bf16 extreme gates")
+
+
 def test_status_codes_match_reference(ctx):
     import ctypes
 
