@@ -190,7 +190,7 @@ def op_entry(name, config, sets, steps, warmup):
 
 
 def ops_table(ctx, args, gen):
-    """Every operator at every BASELINE configuration, each timed alone."""
+    """Every operator at every benchmark configuration (C1-C5), each timed alone."""
     import torch
 
     from operators_amd.ops import sin_cos_table

@@ -101,11 +101,21 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
     load_row(row, xv);// in flight while the weights are fetched below
 
     if constexpr (WHOME == kWLds) {
-        for (uint32_t v = threadIdx.x; v < nvec; v += BS) {
-            float g[8];
-            W::load8(w, v, g);
-            w_lo[v] = f32x4{g[0], g[1], g[2], g[3]};
-            w_hi[v] = f32x4{g[4], g[5], g[6], g[7]};
+        // all of this lane's weight loads are issued before the first is
+        // consumed: one memory latency for the staging, not one per vector
+        float g[NV][8];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            W::load8(w, EXACT || v < nvec ? v : 0, g[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            if (EXACT || v < nvec) {
+                w_lo[v] = f32x4{g[k][0], g[k][1], g[k][2], g[k][3]};
+                w_hi[v] = f32x4{g[k][4], g[k][5], g[k][6], g[k][7]};
+            }
         }
         __syncthreads();
     }

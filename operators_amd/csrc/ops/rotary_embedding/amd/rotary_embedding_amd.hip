@@ -80,6 +80,90 @@ __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *
     }
 }
 
+// The same lane-to-data map as rope_vec, as a looping kernel: a workgroup
+// walks tiles of kBlock work items and always has the next tile's loads (t
+// and table rows) in flight while it rotates and stores the current one.  All
+// loads are unconditional - items or heads past the end are redirected to the
+// last valid one and simply not stored - so the compiler can count the loads
+// in flight and wait for the current tile only.
+template<typename T, int HPT>
+struct RopeTile {
+    u32x4 tv[HPT];
+    f32x4 s_lo, s_hi, c_lo, c_hi;
+    uint16_t *base;
+    uint32_t g;
+    bool live;
+};
+
+template<typename T, typename Idx, int HPT>
+__global__ __launch_bounds__(kBlock) void rope_vec_loop(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
+                                                        uint64_t total_items, Idx items_per_token, Idx vecs_per_head, Idx groups,
+                                                        uint32_t heads, uint32_t head_dim, int64_t stride_token, int64_t stride_head) {
+    const uint64_t tiles = (total_items + kBlock - 1) / kBlock;
+    auto fetch = [&](uint64_t tile, RopeTile<T, HPT> &r) {
+        const uint64_t item64 = tile * kBlock + threadIdx.x;
+        r.live = item64 < total_items;
+        const Idx item = static_cast<Idx>(r.live ? item64 : total_items - 1);
+        const Idx token = item / items_per_token;
+        const Idx rem = item - token * items_per_token;
+        const Idx g = rem / vecs_per_head;
+        const Idx cv = rem - g * vecs_per_head;
+        r.g = static_cast<uint32_t>(g);
+        r.base = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(cv) * 8;
+#pragma unroll
+        for (int i = 0; i < HPT; ++i) {
+            uint32_t h = r.g + i * static_cast<uint32_t>(groups);
+            h = h < heads ? h : heads - 1;
+            r.tv[i] = ld16_stream(r.base + static_cast<int64_t>(h) * stride_head);
+        }
+        const uint64_t row = pos[token] * head_dim + static_cast<uint64_t>(cv) * 8;
+        r.s_lo = ld16f(sin_t + row), r.s_hi = ld16f(sin_t + row + 4);
+        r.c_lo = ld16f(cos_t + row), r.c_hi = ld16f(cos_t + row + 4);
+    };
+    auto rotate = [&](const RopeTile<T, HPT> &r) {
+        const float sn[8] = {r.s_lo.x, r.s_lo.y, r.s_lo.z, r.s_lo.w, r.s_hi.x, r.s_hi.y, r.s_hi.z, r.s_hi.w};
+        const float cs[8] = {r.c_lo.x, r.c_lo.y, r.c_lo.z, r.c_lo.w, r.c_hi.x, r.c_hi.y, r.c_hi.z, r.c_hi.w};
+#pragma unroll
+        for (int i = 0; i < HPT; ++i) {
+            const uint32_t h = r.g + i * static_cast<uint32_t>(groups);
+            float f[8], o[8];
+            widen8<T>(r.tv[i], f);
+#pragma unroll
+            for (int k = 0; k < 8; k += 2) {
+                const float a = f[k], b = f[k + 1];
+                const float ac = a * cs[k], bs = b * sn[k];
+                const float as = a * sn[k + 1], bc = b * cs[k + 1];
+                o[k] = ac - bs;
+                o[k + 1] = as + bc;
+            }
+            const u32x4 packed = narrow8<T>(o);
+            if (r.live && h < heads) st16_stream(r.base + static_cast<int64_t>(h) * stride_head, packed);
+        }
+    };
+
+    uint64_t tile = blockIdx.x;
+    if (tile >= tiles) return;
+    const uint64_t hop = gridDim.x;
+    RopeTile<T, HPT> a, b;
+    fetch(tile, a);
+    while (true) {
+        if (tile + hop >= tiles) {
+            rotate(a);
+            break;
+        }
+        fetch(tile + hop, b);
+        rotate(a);
+        tile += hop;
+        if (tile + hop >= tiles) {
+            rotate(b);
+            break;
+        }
+        fetch(tile + hop, a);
+        rotate(b);
+        tile += hop;
+    }
+}
+
 // Any even head_dim, any strides and alignment: one lane per pair.
 template<typename T>
 __global__ __launch_bounds__(kBlock) void rope_pairs(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
@@ -109,6 +193,26 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
     const uint64_t ipt = groups * vph;
     const uint64_t total = d.tokens * ipt;
     const unsigned grid = static_cast<unsigned>(ceil_div(total, kBlock));
+    // Enough tiles to keep every compute unit looping: the prefetching form.
+    // Measured on MI355X (256 compute units): q [8192,64,128] bf16, 8192 tiles,
+    // 47.0 us looping with 2 workgroups per unit against 48.5 us one tile per
+    // workgroup; [4096,32,128] fp16, 2048 tiles, 14.1 us (4 per unit) against
+    // 16.8 us; k [8192,8,128], 1024 tiles, is faster one tile per workgroup
+    // (9.7 against 10.5 us) and stays on rope_vec.
+    if (grid >= 8u * static_cast<unsigned>(d.cu_count)) {
+        const uint64_t per_cu = grid >= 16u * static_cast<unsigned>(d.cu_count) ? 2 : 4;
+        const uint64_t cap = static_cast<uint64_t>(d.cu_count) * per_cu;
+        const unsigned lgrid = static_cast<unsigned>(grid < cap ? grid : cap);
+#define ROPE_LAUNCH_LOOP(HPT)                                                                                                       \
+    rope_vec_loop<T, Idx, HPT><<<lgrid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph),   \
+                                                             static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),              \
+                                                             static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
+        if (hpt == 4) ROPE_LAUNCH_LOOP(4);
+        else if (hpt == 2) ROPE_LAUNCH_LOOP(2);
+        else ROPE_LAUNCH_LOOP(1);
+#undef ROPE_LAUNCH_LOOP
+        return;
+    }
 #define ROPE_LAUNCH(HPT)                                                                                                   \
     rope_vec<T, Idx, HPT><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph), \
                                                        static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),            \
