@@ -113,26 +113,27 @@ def test_misaligned_pointers_take_the_element_path(ctx):
 
 
 def test_more_than_2_to_31_elements_uses_64_bit_indexing(ctx):
-    """c = [2^15 + 2, 2^16] (just over 2^31 elements, 4 GiB of bf16) with a
-    column operand [rows, 1] and a row operand [2^16]: the general broadcast
-    kernel with 64-bit index arithmetic.  bf16 add is exactly torch's, so the
-    check runs on the GPU."""
+    """c = [2, 2^14 + 1, 2^16] (just over 2^31 elements, 4 GiB of bf16) from
+    a = [2, 1, 2^16] and b = [2^14 + 1, 1]: three merged dimensions, so the
+    general broadcast kernel runs with 64-bit index arithmetic.  bf16 add is
+    exactly torch's, so the check runs on the GPU."""
     import torch
 
-    rows, cols = (1 << 15) + 2, 1 << 16
+    d0, d1, d2 = 2, (1 << 14) + 1, 1 << 16
     g = torch.Generator(device="cuda")
     g.manual_seed(7)
-    a = torch.randn((rows, 1), generator=g, device="cuda").to(torch.bfloat16)
-    b = torch.randn((cols,), generator=g, device="cuda").to(torch.bfloat16)
-    c = torch.empty((rows, cols), dtype=torch.bfloat16, device="cuda")
+    a = torch.randn((d0, 1, d2), generator=g, device="cuda").to(torch.bfloat16)
+    b = torch.randn((d1, 1), generator=g, device="cuda").to(torch.bfloat16)
+    c = torch.empty((d0, d1, d2), dtype=torch.bfloat16, device="cuda")
     ctx.add(c, a, b)
     torch.cuda.synchronize()
-    for r0 in range(0, rows, 8192):  # compare in slabs to bound memory
-        want = a[r0:r0 + 8192] + b
-        assert torch.equal(c[r0:r0 + 8192].view(torch.int16), want.view(torch.int16)), r0
+    for i in range(d0):
+        for r0 in range(0, d1, 4096):  # compare in slabs to bound memory
+            want = a[i] + b[r0:r0 + 4096]
+            assert torch.equal(c[i, r0:r0 + 4096].view(torch.int16), want.view(torch.int16)), (i, r0)
     del c
     # the flat kernel over the same count
-    x = torch.randn((rows * cols // 4,), generator=g, device="cuda").to(torch.bfloat16).repeat(4)
+    x = torch.randn((d0 * d1 * d2 // 4,), generator=g, device="cuda").to(torch.bfloat16).repeat(4)
     y = torch.empty_like(x)
     ctx.add(y, x, x)
     torch.cuda.synchronize()
