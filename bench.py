@@ -247,6 +247,89 @@ def ops_table(ctx, args, gen):
 # ---------------------------------------------------------------------------------
 # CPU baseline
 # ---------------------------------------------------------------------------------
+def cpu_per_op(T):
+    """Host-CPU time of one call of every row of the per-operator table, one
+    thread: the reference's own CPU back end (compiled from its sources into
+    oracle/_ref, kind "reference") for the fp16 rows where that library is
+    present, otherwise - and for every bf16 row, which the reference rejects -
+    the plain-C port (kind "port").  Minimum of 2 calls after 1 warm-up."""
+    import numpy as np
+
+    import oracle
+    from oracle import ref
+
+    have_ref = ref.available()
+    rng = np.random.default_rng(0)
+
+    def codes(shape, dt):
+        v = rng.standard_normal(shape, dtype=np.float32)
+        return oracle.f32_to_bf16(v) if dt == "bf16" else v.astype(np.float16).view(np.uint16)
+
+    def table(rows, theta):
+        freqs = (1.0 / (np.float32(theta) ** (np.arange(0, 128, 2, dtype=np.float32) / np.float32(128)))).astype(np.float32)
+        ang = np.outer(np.arange(rows, dtype=np.float32), np.repeat(freqs, 2)).astype(np.float32)
+        return np.sin(ang), np.cos(ang)
+
+    def best(fn):
+        fn()
+        ts = []
+        for _ in range(2):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return min(ts)
+
+    out = {}
+
+    def run(label, dt, fn_port, fn_ref):
+        use_ref = have_ref and dt == "f16"
+        out[label] = {"cpu_us_per_call": round(best(fn_ref if use_ref else fn_port) * 1e6, 1), "cpu_kind": "reference" if use_ref else "port"}
+
+    x, w16 = codes((16, 2048), "f16"), codes((2048,), "f16")
+    run("C1 rms_norm", "f16", lambda: oracle.rms_norm(x, w16, 1e-5, "f16", "f16"), lambda: ref.rms_norm(x, w16, 1e-5, "f16", "f16"))
+    gu = codes((4096, 22016), "f16")
+    a2, b2 = np.ascontiguousarray(gu[:, 11008:]), np.ascontiguousarray(gu[:, :11008])
+    c2 = np.empty((4096, 11008), np.uint16)
+    run("C2 swiglu f16 [4096,11008]", "f16", lambda: oracle.swiglu(a2, b2, "f16", c=c2), lambda: ref.swiglu(a2, b2, "f16", c=c2))
+    run("C2 swiglu f16 [4096,11008] fused", "f16", lambda: oracle.swiglu(gu[:, 11008:], gu[:, :11008], "f16", c=c2),
+        lambda: ref.swiglu(gu[:, 11008:], gu[:, :11008], "f16", c=c2))
+    del gu, a2, b2, c2
+    qkv = codes((4096, 96, 128), "f16")
+    pos = rng.integers(0, 32768, 4096).astype(np.uint64)
+    s3, c3 = table(32768, 1e4)
+    run("C3 rope", "f16", lambda: oracle.rope(qkv[:, :32, :], pos, s3, c3, "f16"), lambda: ref.rope(qkv[:, :32, :], pos, s3, c3, "f16"))
+    del qkv, s3, c3
+    a4, b4, bb4 = codes((8192, 4096), "f16"), codes((8192, 4096), "f16"), codes((4096,), "f16")
+    c4 = np.empty_like(a4)
+    run("C4 add f16 [8192,4096]", "f16", lambda: oracle.add_into(c4, a4, b4, "f16"), lambda: ref.add(a4, b4, c4.shape, "f16", c=c4))
+    run("C4 add f16 [8192,4096] + b", "f16", lambda: oracle.add_into(c4, a4, bb4, "f16"), lambda: ref.add(a4, bb4, c4.shape, "f16", c=c4))
+    del a4, b4, c4
+    x5, w5 = codes((T, 8192), "bf16"), rng.uniform(0.5, 1.5, 8192).astype(np.float32)
+    y5 = np.empty_like(x5)
+    run("C5 rms_norm", "bf16", lambda: oracle.rms_norm(x5, w5, 1e-5, "bf16", "f32", y=y5), None)
+    run("C5 add", "bf16", lambda: oracle.add_into(y5, x5, x5, "bf16"), None)
+    del x5, y5
+    qkv5 = codes((T, 80, 128), "bf16")
+    pos5 = np.arange(T, dtype=np.uint64)
+    s5, c5 = table(T, 5e5)
+    run("C5 rope_q", "bf16", lambda: oracle.rope(qkv5[:, :64, :], pos5, s5, c5, "bf16"), None)
+    run("C5 rope_k", "bf16", lambda: oracle.rope(qkv5[:, 64:72, :], pos5, s5, c5, "bf16"), None)
+    del qkv5
+    gu5 = codes((T, 57344), "bf16")
+    o5 = np.empty((T, 28672), np.uint16)
+    run("C5 swiglu", "bf16", lambda: oracle.swiglu(gu5[:, 28672:], gu5[:, :28672], "bf16", c=o5), None)
+    return out
+
+
+def attach_cpu(rows, cpu):
+    """Match CPU timings to table rows by the longest label prefix."""
+    for r in rows:
+        hits = [k for k in cpu if r["config"].startswith(k)]
+        if hits:
+            k = max(hits, key=len)
+            r.update(cpu[k])
+            r["speedup_vs_cpu"] = round(cpu[k]["cpu_us_per_call"] / r["us_per_call"], 1)
+
 def cpu_baseline(tokens_full):
     """The CPU oracle (a plain-C port of the reference's CPU path, extended to
     bf16 - the reference itself accepts bf16 in none of the four operators) on
@@ -367,6 +450,8 @@ def main():
         out["ops"] = ops_table(ctx, args, gen)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(T)
+        if not args.no_ops_table:
+            attach_cpu(out["ops"], cpu_per_op(T))
     print(json.dumps(out))
 
 
