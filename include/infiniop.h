@@ -3,7 +3,7 @@
  *
  * The library implements ONE device of the InfiniOperators operator library,
  * `DevAmdGpu` (AMD Instinct MI355X, gfx950), for the four memory-bound LLM-layer
- * operators Add, RMSNorm, RoPE and SwiGLU.  The entry points below have the
+ * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax.  The entry points below have the
  * names, argument order, argument meaning and status codes of the reference
  * library, so that a caller written against the reference (its ctypes harness,
  * its composite operators, any C client) binds to this library unchanged and
@@ -14,7 +14,7 @@
  *   1. infiniopCreateHandle(&handle, DevAmdGpu, device_id)
  *   2. infiniopCreate<Op>Descriptor(handle, &desc, tensor descriptors...)
  *        all shape/stride/dtype checking happens here, once
- *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE; always 0)
+ *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax; always 0)
  *   4. infiniop<Op>(desc, ..., data pointers..., stream)
  *        enqueues on `stream` (a hipStream_t, NULL = the null stream) and
  *        returns without synchronising
@@ -217,5 +217,29 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopSwiGLU(
     infiniopSwiGLUDescriptor_t desc, void *c, void const *a, void const *b, void *stream);
 /* replaces include/ops/swiglu/swiglu.h:25 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroySwiGLUDescriptor(infiniopSwiGLUDescriptor_t desc);
+
+/* ======================================================================== *
+ * CausalSoftmax (first operator beyond the four-operator path):  in place,
+ * over the last dimension of a [seq, total] or [batch, seq, total] tensor,
+ * row i keeps columns j <= total - seq + i, is soft-maxed over them in fp32
+ * and gets exact zeros in the remaining columns.  F16 (reference) or BF16
+ * (extension); unit innermost stride (as the reference's GPU back end
+ * requires); total >= seq.
+ * ======================================================================== */
+typedef struct CausalSoftmaxDescriptor {
+    Device device;
+} CausalSoftmaxDescriptor;
+typedef CausalSoftmaxDescriptor *infiniopCausalSoftmaxDescriptor_t;
+
+/* replaces include/ops/causal_softmax/causal_softmax.h:13-15 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateCausalSoftmaxDescriptor(
+    infiniopHandle_t handle, infiniopCausalSoftmaxDescriptor_t *desc_ptr, infiniopTensorDescriptor_t y_desc);
+/* replaces include/ops/causal_softmax/causal_softmax.h:17 - always 0 bytes */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetCausalSoftmaxWorkspaceSize(infiniopCausalSoftmaxDescriptor_t desc, uint64_t *size);
+/* replaces include/ops/causal_softmax/causal_softmax.h:19-23 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCausalSoftmax(
+    infiniopCausalSoftmaxDescriptor_t desc, void *workspace, uint64_t workspace_size, void *data, void *stream);
+/* replaces include/ops/causal_softmax/causal_softmax.h:25 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyCausalSoftmaxDescriptor(infiniopCausalSoftmaxDescriptor_t desc);
 
 #endif /* INFINIOP_AMD_INFINIOP_H */

@@ -164,6 +164,43 @@ __device__ __forceinline__ float wave_sum(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// Maximum over the 64 lanes of a wavefront, same lane pattern as wave_sum.
+// Lanes the row broadcasts do not reach keep their own value (old = v).
+__device__ __forceinline__ float wave_max(float v) {
+    const auto step = [](float x, float other) { return fmaxf(x, other); };
+    const int b0 = __builtin_bit_cast(int, v);
+    v = step(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b0, b0, 0xB1, 0xF, 0xF, false)));
+    int b = __builtin_bit_cast(int, v);
+    v = step(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x4E, 0xF, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = step(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x141, 0xF, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = step(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x140, 0xF, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = step(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x142, 0xA, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = step(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x143, 0xC, 0xF, false)));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Maximum over a workgroup; same slot discipline as block_sum below.
+template<int WAVES>
+__device__ __forceinline__ float block_max(float v, float *slots, int phase) {
+    v = wave_max(v);
+    if constexpr (WAVES == 1) {
+        return v;
+    } else {
+        float *mine = slots + phase * WAVES;
+        const int wave = threadIdx.x / kWave;
+        if ((threadIdx.x & (kWave - 1)) == 0) mine[wave] = v;
+        __syncthreads();
+        float m = mine[0];
+#pragma unroll
+        for (int i = 1; i < WAVES; ++i) m = fmaxf(m, mine[i]);
+        return m;
+    }
+}
+
 // Sum over a workgroup of WAVES wavefronts.  `slots` is LDS with room for
 // 2*WAVES floats; `phase` alternates 0/1 between consecutive calls so that one
 // barrier per call is enough (a wave can only overwrite a slot set after every

@@ -57,10 +57,15 @@ class SwiGLUDescriptor(_OpDescriptor):
     pass
 
 
+class CausalSoftmaxDescriptor(_OpDescriptor):
+    pass
+
+
 infiniopAddDescriptor_t = POINTER(AddDescriptor)
 infiniopRMSNormDescriptor_t = POINTER(RMSNormDescriptor)
 infiniopRoPEDescriptor_t = POINTER(RoPEDescriptor)
 infiniopSwiGLUDescriptor_t = POINTER(SwiGLUDescriptor)
+infiniopCausalSoftmaxDescriptor_t = POINTER(CausalSoftmaxDescriptor)
 
 
 class CTensor:
@@ -98,13 +103,17 @@ _PROTOTYPES = {
     "infiniopCreateSwiGLUDescriptor": [infiniopHandle_t, POINTER(infiniopSwiGLUDescriptor_t)] + [infiniopTensorDescriptor_t] * 3,
     "infiniopSwiGLU": [infiniopSwiGLUDescriptor_t, c_void_p, c_void_p, c_void_p, c_void_p],
     "infiniopDestroySwiGLUDescriptor": [infiniopSwiGLUDescriptor_t],
+    "infiniopCreateCausalSoftmaxDescriptor": [infiniopHandle_t, POINTER(infiniopCausalSoftmaxDescriptor_t), infiniopTensorDescriptor_t],
+    "infiniopGetCausalSoftmaxWorkspaceSize": [infiniopCausalSoftmaxDescriptor_t, POINTER(c_uint64)],
+    "infiniopCausalSoftmax": [infiniopCausalSoftmaxDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p],
+    "infiniopDestroyCausalSoftmaxDescriptor": [infiniopCausalSoftmaxDescriptor_t],
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
 
 
 def bind_prototypes(lib):
-    """Attach argument and result types for the 18 entry points.  Works on any
+    """Attach argument and result types for every entry point.  Works on any
     library exporting the same C ABI (this one, or a build of the reference)."""
     for name, argtypes in _PROTOTYPES.items():
         fn = getattr(lib, name)  # AttributeError names the missing symbol

@@ -14,6 +14,7 @@ import ctypes
 from .devices import DeviceEnum
 from .liboperators import (
     infiniopAddDescriptor_t,
+    infiniopCausalSoftmaxDescriptor_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
     infiniopSwiGLUDescriptor_t,
@@ -129,6 +130,27 @@ class RoPEPlan(_Plan):
         return t
 
 
+class CausalSoftmaxPlan(_Plan):
+    _destroy = "infiniopDestroyCausalSoftmaxDescriptor"
+
+    def __init__(self, ctx, y):
+        super().__init__(ctx)
+        cts = self._describe(y)
+        desc = infiniopCausalSoftmaxDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateCausalSoftmaxDescriptor(ctx.handle, ctypes.byref(desc), cts[0].descriptor))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetCausalSoftmaxWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value
+
+    def __call__(self, y, stream=None):
+        check_error(self.lib.infiniopCausalSoftmax(self.desc, None, self.workspace_size, y.data_ptr(), stream))
+        return y
+
+
 class Context:
     """A library handle on one GPU plus one-shot forms of the four operators."""
 
@@ -158,6 +180,10 @@ class Context:
     def rms_norm(self, y, x, w, epsilon=1e-5, stream=None):
         with RMSNormPlan(self, y, x, w, epsilon) as plan:
             return plan(y, x, w, stream)
+
+    def causal_softmax(self, y, stream=None):
+        with CausalSoftmaxPlan(self, y) as plan:
+            return plan(y, stream)
 
     def rope(self, t, pos_ids, sin_table, cos_table, stream=None):
         with RoPEPlan(self, t, pos_ids, sin_table, cos_table) as plan:

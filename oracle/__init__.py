@@ -77,6 +77,9 @@ def lib():
         L.oracle_swiglu_check.argtypes, L.oracle_swiglu_check.restype = [tp, tp, tp, ctypes.c_int], ctypes.c_int
         L.oracle_swiglu.argtypes = [u32, u64, u64, i64, i64, i64, vp, vp, vp]
         L.oracle_swiglu.restype = ctypes.c_int
+        L.oracle_causal_softmax_check.argtypes, L.oracle_causal_softmax_check.restype = [tp, ctypes.c_int, ctypes.c_int], ctypes.c_int
+        L.oracle_causal_softmax.argtypes = [u32, u64, u64, u64, i64, i64, i64, vp]
+        L.oracle_causal_softmax.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -229,3 +232,18 @@ def swiglu(a, b, dtype, c=None):
     if st != 0:
         raise RuntimeError(f"oracle_swiglu status {st}")
     return c
+
+
+def causal_softmax_check(y, allow_bf16=False, unit_inner=False):
+    return lib().oracle_causal_softmax_check(y.ref(), int(allow_bf16), int(unit_inner))
+
+
+def causal_softmax(y, dtype):
+    """In place on y: [seq, total] or [batch, seq, total] storage array, any strides."""
+    assert y.ndim in (2, 3)
+    st = [s // 2 for s in y.strides]
+    batch, sb = (y.shape[0], st[0]) if y.ndim == 3 else (1, 0)
+    rc = lib().oracle_causal_softmax(DT[dtype], batch, y.shape[-2], y.shape[-1], sb, st[-2], st[-1], _ptr(y))
+    if rc != 0:
+        raise RuntimeError(f"oracle_causal_softmax status {rc}")
+    return y

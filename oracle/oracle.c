@@ -21,7 +21,12 @@
  *       by the compiled reference, the compiled reference itself where it is
  *       available, plus closed forms (identity elements, constant rows,
  *       pos = 0, norm preservation, b = 0).
- *   bf16 variants of the four operators      PARITY UNPINNED by the reference:
+ *   oracle_causal_softmax (fp16)             pinned  - golden vectors written
+ *       by the compiled reference, the compiled reference itself where it is
+ *       available, a float64 softmax, rows summing to one, zeros above the
+ *       diagonal.  (This operator is outside the four-operator hot path; it is
+ *       the first of the operators that come next.)
+ *   bf16 variants of the operators           PARITY UNPINNED by the reference:
  *       no reference back end accepts bf16 for these operators.  The bf16
  *       arithmetic here is this project's extension (exact widening, the same
  *       fp32/fp64 formulas, round-to-nearest-even narrowing) and is pinned only
@@ -454,6 +459,66 @@ ORACLE_API int oracle_swiglu(uint32_t dt, uint64_t n, uint64_t di,
             float gate = load16(dt, br + j);
             float act = gate / (1.0f + expf(-gate));
             store16(dt, cr + j, up * act);
+        }
+    }
+    return ST_SUCCESS;
+}
+
+/* ------------------------------------------------------------------------ *
+ * Causal softmax (next operator after the four-operator path)
+ * ------------------------------------------------------------------------ */
+
+/* Create-time checks of src/ops/causal_softmax/cpu/causal_softmax_cpu.cc:6-15:
+ * rank 2 or 3, then F16.  `allow_bf16` admits bf16; `unit_inner` additionally
+ * demands a unit innermost stride, which the reference's GPU back end does
+ * (cuda/causal_softmax.cc:22-24) and its CPU back end does not. */
+ORACLE_API int oracle_causal_softmax_check(const oracle_tensor *y, int allow_bf16, int unit_inner) {
+    if (y->ndim != 2 && y->ndim != 3) {
+        return ST_BAD_TENSOR_SHAPE;
+    }
+    if (y->dt != DT_F16 && !(allow_bf16 && y->dt == DT_BF16)) {
+        return ST_BAD_TENSOR_DTYPE;
+    }
+    if (unit_inner && y->strides[y->ndim - 1] != 1) {
+        return ST_BAD_TENSOR_STRIDES;
+    }
+    return ST_SUCCESS;
+}
+
+/* In-place masked softmax over the last dimension, following
+ * src/ops/causal_softmax/cpu/causal_softmax_cpu.cc:52-82.  Row i of a
+ * [seq, total] matrix keeps columns j <= total - seq + i (computed in unsigned
+ * 64-bit arithmetic, so for total < seq the early rows keep everything) and
+ * gets exact zeros elsewhere; the maximum starts from column 0; the sum of
+ * expf(x - max) runs left to right in fp32; each output is expf(x - max) / sum
+ * recomputed, then narrowed. */
+ORACLE_API int oracle_causal_softmax(uint32_t dt, uint64_t batch, uint64_t seq, uint64_t total,
+                                     int64_t stride_b, int64_t stride_i, int64_t stride_j, void *data) {
+    if (dt != DT_F16 && dt != DT_BF16) {
+        return ST_BAD_TENSOR_DTYPE;
+    }
+    uint16_t *y = (uint16_t *) data;
+    for (uint64_t b = 0; b < batch; ++b) {
+        for (uint64_t i = 0; i < seq; ++i) {
+            uint16_t *row = y + (int64_t) b * stride_b + (int64_t) i * stride_i;
+            const uint64_t last = total - seq + i; /* wraps when total < seq, as in the reference */
+            float mx = load16(dt, row);
+            for (uint64_t j = 1; j < total; ++j) {
+                if (j <= last) {
+                    float v = load16(dt, row + (int64_t) j * stride_j);
+                    mx = v > mx ? v : mx; /* std::max(a, b): b only if a < b */
+                } else {
+                    row[(int64_t) j * stride_j] = 0;
+                }
+            }
+            float sum = 0.0f;
+            for (uint64_t j = 0; j < total && j <= last; ++j) {
+                sum += expf(load16(dt, row + (int64_t) j * stride_j) - mx);
+            }
+            for (uint64_t j = 0; j < total && j <= last; ++j) {
+                float e = expf(load16(dt, row + (int64_t) j * stride_j) - mx) / sum;
+                store16(dt, row + (int64_t) j * stride_j, e);
+            }
         }
     }
     return ST_SUCCESS;

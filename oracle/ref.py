@@ -16,6 +16,7 @@ from operators_amd import data_layout as dl
 from operators_amd.liboperators import (
     bind_prototypes,
     infiniopAddDescriptor_t,
+    infiniopCausalSoftmaxDescriptor_t,
     infiniopHandle_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
@@ -191,3 +192,27 @@ def swiglu(a, b, dtype, c=None):
     lib().infiniopDestroySwiGLUDescriptor(desc)
     _free(dc, da, db)
     return c
+
+
+def causal_softmax_status(y):
+    d = descriptor(*y)
+    desc = infiniopCausalSoftmaxDescriptor_t()
+    st = lib().infiniopCreateCausalSoftmaxDescriptor(handle(), ctypes.byref(desc), d)
+    if st == 0:
+        lib().infiniopDestroyCausalSoftmaxDescriptor(desc)
+    _free(d)
+    return st
+
+
+def causal_softmax(y, dtype):
+    d = _desc_of(y, dtype)
+    desc = infiniopCausalSoftmaxDescriptor_t()
+    st = lib().infiniopCreateCausalSoftmaxDescriptor(handle(), ctypes.byref(desc), d)
+    assert st == 0, st
+    size = ctypes.c_uint64(99)
+    assert lib().infiniopGetCausalSoftmaxWorkspaceSize(desc, ctypes.byref(size)) == 0 and size.value == 0
+    st = lib().infiniopCausalSoftmax(desc, None, 0, y.ctypes.data, None)
+    assert st == 0, st
+    lib().infiniopDestroyCausalSoftmaxDescriptor(desc)
+    _free(d)
+    return y

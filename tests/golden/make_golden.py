@@ -189,6 +189,30 @@ def swiglu_vectors(rng):
     return out
 
 
+CAUSAL_CASES = [
+    # (shape, strides or None): the reference's test shape (operatorspy/tests/causal_softmax.py:111-115), smaller, plus odd ones
+    ((4, 20, 512), None), ((4, 20, 512), (20480, 512, 1)), ((7, 13), None), ((5, 5), None), ((1, 40), None),
+    ((3, 16, 16), None), ((2, 9, 1000), (9 * 1024, 1024, 1)),
+]
+
+
+def causal_softmax_vectors(rng):
+    out = {}
+    for i, (shape, strides) in enumerate(CAUSAL_CASES):
+        vals = f16(rng.standard_normal(shape) * (3.0 if i % 2 else 1.0))
+        if strides is None:
+            y = vals.copy()
+        else:
+            span = 1 + sum((n - 1) * s for n, s in zip(shape, strides))
+            buf = f16(rng.standard_normal(span))
+            y = np.lib.stride_tricks.as_strided(buf, shape, [s * 2 for s in strides])
+            y[...] = vals
+        out[f"causal{i}_in"] = np.array(y)
+        ref.causal_softmax(y, "f16")
+        out[f"causal{i}_out"] = np.array(y)
+    return out
+
+
 def status_cases():
     """Create-time (and, for RMSNorm, compute-time) status codes of the reference."""
     cases = []
@@ -203,6 +227,8 @@ def status_cases():
             st = ref.rope_status(*tensors)
         elif op == "rms_norm":
             st = ref.rms_norm_status(*tensors, run=extra.get("run", False))
+        elif op == "causal_softmax":
+            st = ref.causal_softmax_status(*tensors)
         cases.append({"op": op, "tensors": specs, "status": int(st), **extra})
 
     T = lambda dt, shape, st=None: (dt, tuple(shape), None if st is None else tuple(st))  # noqa: E731
@@ -258,6 +284,15 @@ def status_cases():
     rec("rms_norm", [T("f16", (128,)), T("f16", (128,)), T("f16", (128,))])
     rec("rms_norm", [T("f32", (4, 32)), T("f32", (4, 32)), T("f32", (32,))], run=True)
     rec("rms_norm", [T("bf16", (4, 32)), T("bf16", (4, 32)), T("f32", (32,))], run=True, bf16_extension=True)
+    # causal softmax (y)
+    rec("causal_softmax", [T("f16", (4, 8, 16))])
+    rec("causal_softmax", [T("f16", (8, 16))])
+    rec("causal_softmax", [T("f16", (8, 16), (32, 1))])
+    rec("causal_softmax", [T("f16", (16,))])
+    rec("causal_softmax", [T("f16", (2, 2, 8, 16))])
+    rec("causal_softmax", [T("f32", (8, 16))])
+    rec("causal_softmax", [T("bf16", (8, 16))], bf16_extension=True)
+    rec("causal_softmax", [T("f16", (8, 16), (32, 2))], cpu_only_layout=True)  # accepted by the CPU back end, refused by the GPU ones
     return cases
 
 
@@ -269,10 +304,12 @@ def main():
     np.savez_compressed(os.path.join(HERE, "rms_norm.npz"), **rms_norm_vectors(rng))
     np.savez_compressed(os.path.join(HERE, "rope.npz"), **rope_vectors(rng))
     np.savez_compressed(os.path.join(HERE, "swiglu.npz"), **swiglu_vectors(rng))
+    np.savez_compressed(os.path.join(HERE, "causal_softmax.npz"), **causal_softmax_vectors(rng))
     with open(os.path.join(HERE, "status_cases.json"), "w") as f:
         json.dump({"add_cases": [list(map(list, c)) for c in ADD_CASES],
                    "rope_cases": [[list(s), None if st is None else list(st), r] for s, st, r in ROPE_CASES],
                    "swiglu_cases": [[list(s), a, b, c] for s, a, b, c in SWIGLU_CASES],
+                   "causal_cases": [[list(s), None if st is None else list(st)] for s, st in CAUSAL_CASES],
                    "status": status_cases()}, f, indent=1)
     for name in sorted(os.listdir(HERE)):
         print(f"{name:24s} {os.path.getsize(os.path.join(HERE, name)):>9d} bytes")

@@ -1,0 +1,103 @@
+"""CausalSoftmax on the GPU through the C ABI, against the oracle and the
+reference's golden vectors.  Bar (fp16): |gpu - ref| <= 1e-3 + 1e-3*|ref| and
+at most one unit in the last place (tree sum on the GPU, running sum on the
+CPU; last bit of expf).  bf16: 1e-2.  Masked columns must be exact zeros."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_allclose16, assert_codes_close, golden, golden_json, strided_like, to_codes, to_torch
+
+pytestmark = pytest.mark.gpu
+TOL = {"f16": 1e-3, "bf16": 1e-2}
+
+
+def run(ctx, codes, shape, strides, dt):
+    import torch
+
+    if strides is None:
+        t = to_torch(codes, dt).reshape(shape)
+        buf = t
+    else:
+        t, buf = strided_like(codes, shape, strides, dt)
+    before = to_codes(buf)
+    ctx.causal_softmax(t)
+    torch.cuda.synchronize()
+    return to_codes(t), before, to_codes(buf)
+
+
+def check(got, want, dt, what, max_frac=5e-3):
+    assert np.array_equal(got == 0, want == 0) or np.all((got == 0) >= ((want & 0x7FFF) == 0)), what
+    assert_allclose16(oracle.decode(got, dt), oracle.decode(want, dt), TOL[dt], TOL[dt], what)
+    return assert_codes_close(got, want, dt, max_ulp=1, max_frac=max_frac, what=what)
+
+
+def test_golden_cases(ctx):
+    g = golden("causal_softmax")
+    for i, (shape, strides) in enumerate(golden_json()["causal_cases"]):
+        got, before, after = run(ctx, g[f"causal{i}_in"], shape, strides, "f16")
+        check(got, g[f"causal{i}_out"], "f16", f"golden causal case {i} {shape} {strides}")
+        if strides is not None:  # gaps between rows untouched
+            idx = np.zeros(shape, np.int64)
+            for ax, st in enumerate(strides):
+                ix = np.arange(shape[ax]).reshape([-1 if a == ax else 1 for a in range(len(shape))])
+                idx = idx + ix * st
+            mask = np.ones(before.size, bool)
+            mask[idx.ravel()] = False
+            assert np.array_equal(before[mask], after[mask])
+
+
+CASES = [
+    ((32, 20, 512), None), ((32, 20, 512), (20480, 512, 1)),   # the reference's test
+    ((7, 13), None), ((5, 5), None), ((1, 8), None), ((3, 16, 16), None),
+    ((2, 300, 4096), None), ((2, 64, 8192), None), ((1, 9, 32768), None), ((1, 5, 40000), None),
+    ((4, 33, 1000), None), ((2, 128, 136), (128 * 144, 144, 1)), ((3, 10, 64), (1000, 65, 1)),
+]
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_against_oracle(ctx, dt, case):
+    shape, strides = CASES[case]
+    rng = np.random.default_rng(500 + case)
+    y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 2, dt)
+    want = oracle.causal_softmax(y.copy(), dt)
+    got, _, _ = run(ctx, y, shape, strides, dt)
+    seq, total = shape[-2], shape[-1]
+    keep = np.arange(total)[None, :] <= total - seq + np.arange(seq)[:, None]
+    assert not got[..., ~keep].any(), "masked columns must be exact zeros"
+    check(got, want, dt, f"{shape} {strides} {dt}", max_frac=2e-2 if total > 4096 else 5e-3)
+
+
+def test_attention_scores_shape(ctx):
+    """[heads, seq, total] = [8, 2048, 2048] fp16 with a scale typical of q.k/sqrt(d)."""
+    rng = np.random.default_rng(77)
+    shape = (8, 2048, 2048)
+    y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 1.5, "f16")
+    want = oracle.causal_softmax(y.copy(), "f16")
+    got, _, _ = run(ctx, y, shape, None, "f16")
+    frac, worst = check(got, want, "f16", "attention scores")
+    print(f"causal softmax [8,2048,2048]: {frac:.2e} of elements differ by {worst} ulp")
+    rows = oracle.decode(got, "f16").astype(np.float64).sum(-1)
+    assert np.all(np.abs(rows - 1) < 0.02)
+
+
+def test_status_codes_match_reference(ctx):
+    import ctypes
+
+    from operators_amd import infiniopCausalSoftmaxDescriptor_t, make_descriptor
+    from oracle.ref import LAYOUT
+
+    lib = ctx.lib
+    for case in golden_json()["status"]:
+        if case["op"] != "causal_softmax":
+            continue
+        t = case["tensors"][0]
+        desc = make_descriptor(lib, t[1], t[2], LAYOUT[t[0]])
+        d = infiniopCausalSoftmaxDescriptor_t()
+        st = lib.infiniopCreateCausalSoftmaxDescriptor(ctx.handle, ctypes.byref(d), desc)
+        want = 0 if case.get("bf16_extension") else (5 if case.get("cpu_only_layout") else case["status"])
+        assert st == want, (case, st)
+        if st == 0:
+            assert lib.infiniopDestroyCausalSoftmaxDescriptor(d) == 0
+        lib.infiniopDestroyTensorDescriptor(desc)

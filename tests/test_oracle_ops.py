@@ -252,3 +252,39 @@ def test_swiglu_bf16_extension_matches_float64_formula():
     want = x * y / (1 + np.exp(-y))
     got = oracle.decode(oracle.swiglu(av, bv, "bf16"), "bf16")
     assert np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-30)
+
+
+# ---- causal softmax (first operator beyond the four-operator path) -------------------
+def test_causal_softmax_golden():
+    g = golden("causal_softmax")
+    for i, (shape, strides) in enumerate(golden_json()["causal_cases"]):
+        y = g[f"causal{i}_in"].copy()
+        oracle.causal_softmax(y, "f16")
+        assert_codes_close(y, g[f"causal{i}_out"], "f16", max_ulp=1, max_frac=1e-3, what=f"case {i} {shape}")
+
+
+@needs_ref
+def test_causal_softmax_vs_compiled_reference():
+    rng = np.random.default_rng(23)
+    for shape in [(3, 17, 64), (9, 9), (2, 5, 333)]:
+        y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 4, "f16")
+        assert np.array_equal(oracle.causal_softmax(y.copy(), "f16"), ref.causal_softmax(y.copy(), "f16"))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_causal_softmax_against_float64(dt):
+    rng = np.random.default_rng(24)
+    seq, total = 12, 40
+    y = oracle.encode(rng.standard_normal((3, seq, total)).astype(np.float32), dt)
+    x = oracle.decode(y, dt).astype(np.float64)
+    got = oracle.decode(oracle.causal_softmax(y.copy(), dt), dt).astype(np.float64)
+    j, i = np.arange(total)[None, :], np.arange(seq)[:, None]
+    keep = j <= total - seq + i                      # row i keeps columns up to total - seq + i
+    z = np.where(keep, x, -np.inf)
+    want = np.exp(z - z.max(-1, keepdims=True))
+    want /= want.sum(-1, keepdims=True)
+    ulp = 2.0 ** -10 if dt == "f16" else 2.0 ** -7
+    assert np.all(np.abs(got - want) <= ulp * want + 1e-7)
+    assert np.all(got[:, ~keep] == 0) and np.all(got[:, keep] > 0)
+    assert np.all(np.abs(got.sum(-1) - 1) < 40 * ulp)  # truncation loses up to one ulp per kept element
+    assert got[:, 0, : total - seq + 1].min() > 0 and np.count_nonzero(got[:, 0]) == 3 * (total - seq + 1)

@@ -32,6 +32,14 @@ def test_oracle_checks_reproduce_reference_status(i):
         st = oracle.swiglu_check(*specs, allow_bf16=False)
     elif case["op"] == "rope":
         st = oracle.rope_check(*specs, allow_bf16=False)
+    elif case["op"] == "causal_softmax":
+        st = oracle.causal_softmax_check(specs[0], allow_bf16=False, unit_inner=False)
+        assert st == case["status"], case
+        if case.get("bf16_extension"):
+            assert oracle.causal_softmax_check(specs[0], allow_bf16=True, unit_inner=True) == 0
+        if case.get("cpu_only_layout"):
+            assert oracle.causal_softmax_check(specs[0], allow_bf16=False, unit_inner=True) == 5
+        return
     else:
         st = oracle.rms_norm_check(*specs)
         if st == 0 and case.get("run"):  # the reference reports unsupported data types at compute time
@@ -66,6 +74,7 @@ CREATE = {
     "swiglu": ("infiniopCreateSwiGLUDescriptor", "infiniopDestroySwiGLUDescriptor", oa.infiniopSwiGLUDescriptor_t),
     "rope": ("infiniopCreateRoPEDescriptor", "infiniopDestroyRoPEDescriptor", oa.infiniopRoPEDescriptor_t),
     "rms_norm": ("infiniopCreateRMSNormDescriptor", "infiniopDestroyRMSNormDescriptor", oa.infiniopRMSNormDescriptor_t),
+    "causal_softmax": ("infiniopCreateCausalSoftmaxDescriptor", "infiniopDestroyCausalSoftmaxDescriptor", oa.infiniopCausalSoftmaxDescriptor_t),
 }
 
 
@@ -89,9 +98,13 @@ def test_library_host_validation_reproduces_reference_status(fake_handle, i):
         want = 0
     else:
         want = 0 if case.get("bf16_extension") else case["status"]
+        if case.get("cpu_only_layout"):
+            want = 5  # non-unit inner stride: accepted by the reference's CPU back end only, refused here as by its GPU back end
     assert st == want, (case, st)
     if st == 0:
         size = ctypes.c_uint64(7)
+        if case["op"] == "causal_softmax":
+            assert lib.infiniopGetCausalSoftmaxWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
         if case["op"] == "rms_norm":
             assert lib.infiniopGetRMSNormWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
         if case["op"] == "rope":
@@ -116,6 +129,17 @@ def test_descriptor_starts_with_device_number(fake_handle):
     assert lib.infiniopCreateSwiGLUDescriptor(ctypes.cast(ctypes.pointer(other), oa.infiniopHandle_t), ctypes.byref(d2), *descs) == 8
     for x in descs:
         lib.infiniopDestroyTensorDescriptor(x)
+
+
+def test_causal_softmax_refuses_fewer_columns_than_rows(fake_handle):
+    """The reference's column bound wraps around for total < seq and its CPU
+    loops then leave the row; this library refuses the shape instead."""
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    y = oa.make_descriptor(lib, (8, 4), None, oa.F16)
+    d = oa.infiniopCausalSoftmaxDescriptor_t()
+    assert lib.infiniopCreateCausalSoftmaxDescriptor(handle, ctypes.byref(d), y) == 4
+    lib.infiniopDestroyTensorDescriptor(y)
 
 
 def test_null_output_pointer_is_memory_not_allocated(fake_handle):
