@@ -115,6 +115,16 @@ def make_swiglu(ctx, n, di, dtype, fused, gen, name):
     return Launch(name, ctx.lib.infiniopSwiGLU, (plan.desc, c.data_ptr(), a.data_ptr(), b.data_ptr()), 3 * n * di * c.element_size(), (plan, keep, c))
 
 
+def make_causal_softmax(ctx, heads, seq, total, dtype, gen, name):
+    from operators_amd.ops import CausalSoftmaxPlan
+
+    y = _randn((heads, seq, total), dtype, gen)
+    plan = CausalSoftmaxPlan(ctx, y)
+    kept = seq * (total - seq) + seq * (seq + 1) // 2  # elements read per matrix; every element is written
+    nbytes = heads * (kept + seq * total) * y.element_size()
+    return Launch(name, ctx.lib.infiniopCausalSoftmax, (plan.desc, None, 0, y.data_ptr()), nbytes, (plan, y))
+
+
 def make_add(ctx, n, d, dtype, broadcast, gen, name):
     import torch
 
@@ -223,6 +233,8 @@ def ops_table(ctx, args, gen):
         f"C5 rope_k bf16 [{T},8,128] in [{T},80,128]": lambda: rope_sets(T, 80, 64, 8, bf16, T, 5e5, False),
         f"C5 swiglu bf16 [{T},28672] fused gate/up": lambda: [make_swiglu(ctx, T, 28672, bf16, True, gen, "swiglu") for _ in range(max(2, nset // 2))],
         f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(sets_needed(6 * T * 8192, nset))],
+        # beyond the four-operator path: attention scores of 32 heads, 4096 x 4096, in place
+        "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
         # Not an operator of the library: a plain device-to-device copy of known

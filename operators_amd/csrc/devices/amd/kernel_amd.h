@@ -138,6 +138,19 @@ __device__ __forceinline__ u32x4 narrow8(const float (&r)[8]) {
     return out;
 }
 
+// Eight results known to lie in [0, 1] (or to be NaN): the hardware pack alone.
+// Nothing in that range reaches the magnitudes where the reference's
+// conversion departs from round-toward-zero.
+template<typename T>
+__device__ __forceinline__ u32x4 narrow8_unit_range(const float (&r)[8]) {
+    u32x4 out;
+    out.x = T::narrow2_fast(r[0], r[1]);
+    out.y = T::narrow2_fast(r[2], r[3]);
+    out.z = T::narrow2_fast(r[4], r[5]);
+    out.w = T::narrow2_fast(r[6], r[7]);
+    return out;
+}
+
 template<typename T>
 __device__ __forceinline__ void widen8(u32x4 v, float (&r)[8]) {
     r[0] = T::lo(v.x);

@@ -20,53 +20,132 @@ namespace {
 
 using namespace amd;
 
+// expf(d) for d <= 0 through the hardware exp2: d * log2(e) is formed as an
+// unevaluated sum hi + lo (one fused multiply-add recovers the rounding error
+// of the product, a second term carries the rest of log2(e)), exp2 takes hi
+// and lo enters as the first-order factor (1 + lo * ln 2).  About 9 VALU slots
+// against about 12 for the library routine, and no range checks: the caller
+// guarantees -126 <= d <= 0, where everything is finite and normal.
+__device__ __forceinline__ float exp_nonpositive(float d) {
+    constexpr float kL2e = 1.44269502162933349609375f;    // log2(e) rounded to fp32
+    constexpr float kL2eLo = 1.92596299112661746e-8f;     // log2(e) - kL2e
+    constexpr float kLn2 = 0.693147182464599609375f;
+    const float hi = d * kL2e;
+    const float lo = __builtin_fmaf(d, kL2eLo, __builtin_fmaf(d, kL2e, -hi));
+    const float e = __builtin_amdgcn_exp2f(hi);
+    return __builtin_fmaf(e, lo * kLn2, e);
+}
+constexpr float kLeanExpLimit = -126.0f;
+
+// The library exponential for the rare arguments outside that range (-inf,
+// very long tails, NaN).  Deliberately not inlined: it is almost never
+// executed, and four inlined copies per kernel cost instruction-cache space
+// that the common path needs.
+__device__ __attribute__((noinline)) float exp_any(float d) { return expf(d); }
+
 // One workgroup of BS lanes per row at a time; lane l owns vectors l, l+BS, ...
 // (NV of them, 8 elements each), so total <= 8*BS*NV.  Workgroups stride over
-// the batch*seq rows; neighbouring rows have nearly the same kept length, so
-// the stride balances the causal triangle.
+// the batch*seq rows (neighbouring rows keep nearly the same number of
+// columns, so the stride balances the causal triangle) and always have the
+// next row's loads in flight.  Loads are unconditional - a lane whose vector
+// lies in the masked part re-reads the row's last kept vector, which the
+// memory pipeline merges into one request - so that the compiler can count
+// the loads in flight and wait for the current row only.
 template<typename T, int BS, int NV>
-__global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t rows, uint64_t seq, uint32_t total,
+__global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
                                                           int64_t stride_b, int64_t stride_i) {
     constexpr int WAVES = BS / kWave;
     __shared__ float red[4 * WAVES];// two slot sets for the maxima, two for the sums
     const uint32_t nvec = total / 8;
     const float neg_inf = -__builtin_inff();
-    int phase = 0;
-    for (uint64_t r = blockIdx.x; r < rows; r += gridDim.x, phase ^= 1) {
-        const uint64_t b = r / seq, i = r - b * seq;
-        uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
-        const uint32_t keep = static_cast<uint32_t>(total - seq + i) + 1;// columns kept, 1..total
-        const uint32_t keep_vecs = (keep + 7) / 8;
 
+    struct Row {
+        uint16_t *ptr;
+        uint32_t keep;// columns kept, 1..total
+    };
+    // Global row r = b*seq + i.  All workgroups work on neighbouring rows at
+    // any one time (measured: faster than giving each matrix of the batch its
+    // own workgroups); (b, i) is advanced by the constant hop without dividing.
+    const uint32_t hop = gridDim.x;
+    const uint32_t hop_b = hop / seq, hop_i = hop - hop_b * seq;
+    uint64_t b = blockIdx.x / seq;
+    uint32_t i = blockIdx.x - static_cast<uint32_t>(b) * seq;
+    auto here = [&]() { return Row{y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i, total - seq + i + 1}; };
+    auto advance = [&]() {
+        b += hop_b;
+        i += hop_i;
+        if (i >= seq) {
+            i -= seq;
+            ++b;
+        }
+    };
+    auto load_row = [&](const Row &row, u32x4(&dst)[NV]) {
+        const uint32_t last_vec = (row.keep - 1) / 8;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            dst[k] = ld16_stream(row.ptr + static_cast<uint64_t>(v < last_vec ? v : last_vec) * 8);
+        }
+    };
+    auto finish_row = [&](const Row &row, const u32x4(&cur)[NV], int phase) {
+        const uint32_t keep = row.keep;
+        const uint32_t keep_vecs = (keep + 7) / 8;
         float f[NV][8];
         float mx = neg_inf;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = k * BS + threadIdx.x;
-            if (v < keep_vecs) {
-                widen8<T>(ld16_stream(row + static_cast<uint64_t>(v) * 8), f[k]);
+            if (v >= keep_vecs) continue;// wholly masked: nothing to reduce, zeros are stored below
+            widen8<T>(cur[k], f[k]);
+            if (v * 8 + 8 > keep) {// the boundary vector
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    if (v * 8 + e >= keep) f[k][e] = neg_inf;
-                    mx = fmaxf(mx, f[k][e]);
-                }
+                for (int e = 0; e < 8; ++e) f[k][e] = v * 8 + e < keep ? f[k][e] : neg_inf;
             }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[k][e]);
         }
         mx = block_max<WAVES>(mx, red, phase);
 
+        // d = x - max <= 0.  The masked tail of the boundary vector takes d = 0
+        // here and is zeroed after the exponential.  Anything below the lean
+        // exponential's range (-inf inputs, very long tails) sends the wavefront
+        // through the library routine; NaN passes through either form as NaN.
+        float lowest = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            if (v >= keep_vecs) continue;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[k][e] -= mx;
+            if (v * 8 + 8 > keep) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[k][e] = v * 8 + e < keep ? f[k][e] : 0.0f;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) lowest = fminf(lowest, f[k][e]);
+        }
+        const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
         float part = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = k * BS + threadIdx.x;
-            if (v < keep_vecs) {
+            if (v >= keep_vecs) continue;
+            if (lean) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    f[k][e] = v * 8 + e < keep ? expf(f[k][e] - mx) : 0.0f;
-                    part += f[k][e];
-                }
+                for (int e = 0; e < 8; ++e) f[k][e] = exp_nonpositive(f[k][e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[k][e] = exp_any(f[k][e]);
             }
+            if (v * 8 + 8 > keep) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[k][e] = v * 8 + e < keep ? f[k][e] : 0.0f;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) part += f[k][e];
         }
         const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
+        const float rcp = 1.0f / sum;
 
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -74,12 +153,45 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
             if (v < keep_vecs) {
                 float o[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = f[k][e] / sum;
-                st16_stream(row + static_cast<uint64_t>(v) * 8, narrow8<T>(o));
+                for (int e = 0; e < 8; ++e) {
+                    const float q = f[k][e] * rcp;// e / sum: one residual step makes the quotient correctly rounded in all but rare cases
+                    o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, f[k][e]), rcp, q);
+                }
+                if (v * 8 + 8 > keep) {// boundary vector: its masked tail is zero even when the row turned to NaN
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o[e] = v * 8 + e < keep ? o[e] : 0.0f;
+                }
+                st16_stream(row.ptr + static_cast<uint64_t>(v) * 8, narrow8_unit_range<T>(o));
             } else if (v < nvec) {
-                st16_stream(row + static_cast<uint64_t>(v) * 8, u32x4{0, 0, 0, 0});
+                st16_stream(row.ptr + static_cast<uint64_t>(v) * 8, u32x4{0, 0, 0, 0});
             }
         }
+    };
+
+    uint64_t r = blockIdx.x;
+    if (r >= rows) return;
+    u32x4 xa[NV], xb[NV];
+    Row ra = here(), rb = ra;
+    load_row(ra, xa);
+    while (true) {
+        if (r + hop >= rows) {
+            finish_row(ra, xa, 0);
+            break;
+        }
+        advance();
+        rb = here();
+        load_row(rb, xb);
+        finish_row(ra, xa, 0);
+        r += hop;
+        if (r + hop >= rows) {
+            finish_row(rb, xb, 1);
+            break;
+        }
+        advance();
+        ra = here();
+        load_row(ra, xa);
+        finish_row(rb, xb, 1);
+        r += hop;
     }
 }
 
@@ -112,20 +224,26 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     auto *py = static_cast<uint16_t *>(data);
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
-    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * 8;
+    // Rows of up to 4096 elements are taken by single wavefronts (no barrier, no
+    // LDS; 32 such workgroups per compute unit), longer ones by 256-1024 lanes
+    // (8 per unit).  Measured on MI355X at [32, 4096, 4096] fp16: 317 us with
+    // one row per wavefront against 338-360 us with 128, 256 or 512 lanes per
+    // row; a plain kernel that reads half of every 8 KiB row and writes all of
+    // it - the traffic of this operator without any arithmetic - needs 284 us.
+    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * (nvec <= 512 ? 32 : 8);
     const unsigned grid = static_cast<unsigned>(rows < cap ? rows : cap);
 
-    const bool vec_ok = d.total % 8 == 0 && nvec <= 4096 && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);
+    const bool vec_ok = d.total % 8 == 0 && nvec <= 4096 && d.seq < (1ull << 31) && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);
     if (!vec_ok) {
         causal_softmax_generic<T><<<grid, 256, 0, stream>>>(py, rows, d.seq, d.total, d.stride_b, d.stride_i);
         return;
     }
 #define CS_LAUNCH(BS, NV) \
-    causal_softmax_rows<T, BS, NV><<<grid, BS, 0, stream>>>(py, rows, d.seq, static_cast<uint32_t>(d.total), d.stride_b, d.stride_i)
+    causal_softmax_rows<T, BS, NV><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i)
     if (nvec <= 64) CS_LAUNCH(64, 1);
-    else if (nvec <= 128) CS_LAUNCH(128, 1);
-    else if (nvec <= 256) CS_LAUNCH(256, 1);
-    else if (nvec <= 512) CS_LAUNCH(256, 2);
+    else if (nvec <= 128) CS_LAUNCH(64, 2);
+    else if (nvec <= 256) CS_LAUNCH(64, 4);
+    else if (nvec <= 512) CS_LAUNCH(64, 8);
     else if (nvec <= 1024) CS_LAUNCH(256, 4);
     else if (nvec <= 2048) CS_LAUNCH(512, 4);
     else CS_LAUNCH(1024, 4);
