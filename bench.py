@@ -125,6 +125,20 @@ def make_causal_softmax(ctx, heads, seq, total, dtype, gen, name):
     return Launch(name, ctx.lib.infiniopCausalSoftmax, (plan.desc, None, 0, y.data_ptr()), nbytes, (plan, y))
 
 
+def make_rearrange(ctx, tokens, heads, dtype, gen, name):
+    """[token, head, 128] heads of a fused qkv buffer -> contiguous [head, token, 128] (a cache write / head transpose)."""
+    import torch
+
+    from operators_amd.ops import RearrangePlan
+
+    qkv = _randn((tokens, heads + 16, 128), dtype, gen)
+    src = qkv[:, :heads, :]
+    cache = torch.empty((heads, tokens, 128), dtype=dtype, device="cuda")
+    dst = cache.permute(1, 0, 2)  # same logical shape as src, strides (128, tokens*128, 1)
+    plan = RearrangePlan(ctx, dst, src)
+    return Launch(name, ctx.lib.infiniopRearrange, (plan.desc, dst.data_ptr(), src.data_ptr()), 2 * src.numel() * src.element_size(), (plan, qkv, cache))
+
+
 def make_add(ctx, n, d, dtype, broadcast, gen, name):
     import torch
 
@@ -234,6 +248,7 @@ def ops_table(ctx, args, gen):
         f"C5 swiglu bf16 [{T},28672] fused gate/up": lambda: [make_swiglu(ctx, T, 28672, bf16, True, gen, "swiglu") for _ in range(max(2, nset // 2))],
         f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(sets_needed(6 * T * 8192, nset))],
         # beyond the four-operator path: attention scores of 32 heads, 4096 x 4096, in place
+        f"N2 rearrange bf16 [{T},64,128] of [{T},80,128] -> [64,{T},128]": lambda: [make_rearrange(ctx, T, 64, bf16, gen, "rearrange") for _ in range(sets_needed(4 * T * 64 * 128, nset))],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:

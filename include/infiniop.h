@@ -3,7 +3,7 @@
  *
  * The library implements ONE device of the InfiniOperators operator library,
  * `DevAmdGpu` (AMD Instinct MI355X, gfx950), for the four memory-bound LLM-layer
- * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax.  The entry points below have the
+ * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax and Rearrange.  The entry points below have the
  * names, argument order, argument meaning and status codes of the reference
  * library, so that a caller written against the reference (its ctypes harness,
  * its composite operators, any C client) binds to this library unchanged and
@@ -241,5 +241,27 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCausalSoftmax(
     infiniopCausalSoftmaxDescriptor_t desc, void *workspace, uint64_t workspace_size, void *data, void *stream);
 /* replaces include/ops/causal_softmax/causal_softmax.h:25 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyCausalSoftmaxDescriptor(infiniopCausalSoftmaxDescriptor_t desc);
+
+/* ======================================================================== *
+ * Rearrange (second operator beyond the four-operator path):  dst = src for
+ * two tensors of equal shape and element type whose other strides are free
+ * (KV-cache writes, head transposes).  Any element type; unit innermost
+ * strides; for rank >= 4 the leading dimensions must nest as the reference
+ * demands.
+ * ======================================================================== */
+typedef struct RearrangeDescriptor {
+    Device device;
+} RearrangeDescriptor;
+typedef RearrangeDescriptor *infiniopRearrangeDescriptor_t;
+
+/* replaces include/ops/rearrange/rearrange.h:12-15 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateRearrangeDescriptor(
+    infiniopHandle_t handle, infiniopRearrangeDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t dst, infiniopTensorDescriptor_t src);
+/* replaces include/ops/rearrange/rearrange.h:17 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRearrange(
+    infiniopRearrangeDescriptor_t desc, void *dst, void const *src, void *stream);
+/* replaces include/ops/rearrange/rearrange.h:19 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyRearrangeDescriptor(infiniopRearrangeDescriptor_t desc);
 
 #endif /* INFINIOP_AMD_INFINIOP_H */

@@ -13,6 +13,7 @@ from .liboperators import (  # noqa: F401
     infiniopAddDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
     infiniopHandle_t,
+    infiniopRearrangeDescriptor_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
     infiniopSwiGLUDescriptor_t,

@@ -1,0 +1,143 @@
+// gfx950 kernels for Rearrange and their launch: a strided copy that moves
+// each innermost row as a block of bytes (reference
+// src/ops/rearrange/cpu/rearrange_cpu.cc:70-92).  No arithmetic at all: the
+// only questions are how wide an access the layout allows and how to find a
+// row's two addresses cheaply.
+#include "../../../devices/amd/kernel_amd.h"
+#include "rearrange_amd.h"
+
+namespace {
+
+using namespace amd;
+
+constexpr int kBlock = 256;
+
+struct OuterDims {
+    int ndim;
+    uint32_t shape[kRearrangeMaxDims];
+    int64_t dst_stride[kRearrangeMaxDims];
+    int64_t src_stride[kRearrangeMaxDims];
+};
+
+// The access unit: the widest of 16, 8, 4, 2, 1 bytes that divides the row
+// length, every stride and both base addresses.
+template<int BYTES> struct Unit;
+template<> struct Unit<16> { typedef u32x4 type; };
+template<> struct Unit<8> { typedef uint64_t type; };
+template<> struct Unit<4> { typedef uint32_t type; };
+template<> struct Unit<2> { typedef uint16_t type; };
+template<> struct Unit<1> { typedef uint8_t type; };
+
+// blockIdx.y walks the rows, blockIdx.x the units of a row: rows of at least a
+// wavefront of units.  The row's offsets are found by dividing the row number
+// by the merged outer extents - once per workgroup row, on the scalar unit,
+// since the row number is uniform.
+template<int BYTES>
+__global__ __launch_bounds__(kBlock) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row) {
+    typedef typename Unit<BYTES>::type U;
+    const uint32_t col = blockIdx.x * kBlock + threadIdx.x;
+    if (col >= units_per_row) return;
+    for (uint64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        int64_t od = 0, os = 0;
+        uint64_t rest = r;
+#pragma unroll
+        for (int k = 0; k < kRearrangeMaxDims; ++k) {
+            if (k < d.ndim) {
+                const uint64_t i = rest % d.shape[k];
+                rest /= d.shape[k];
+                od += static_cast<int64_t>(i) * d.dst_stride[k];
+                os += static_cast<int64_t>(i) * d.src_stride[k];
+            }
+        }
+        const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
+        __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+    }
+}
+
+// Short rows: one lane per unit over the flat (row, unit) space, one unit per
+// lane and one workgroup per 256 units.  Idx is 32-bit when the unit count
+// allows, which makes the divisions cheap.
+template<int BYTES, typename Idx>
+__global__ __launch_bounds__(kBlock) void rearrange_flat(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t total_units, Idx units_per_row) {
+    typedef typename Unit<BYTES>::type U;
+    const uint64_t idx64 = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (idx64 >= total_units) return;
+    const Idx idx = static_cast<Idx>(idx64);
+    Idx rest = idx / units_per_row;
+    const Idx col = idx - rest * units_per_row;
+    int64_t od = 0, os = 0;
+#pragma unroll
+    for (int k = 0; k < kRearrangeMaxDims; ++k) {
+        if (k < d.ndim) {
+            const Idx ext = static_cast<Idx>(d.shape[k]);
+            const Idx q = rest / ext;
+            const Idx i = rest - q * ext;
+            rest = q;
+            od += static_cast<int64_t>(i) * d.dst_stride[k];
+            os += static_cast<int64_t>(i) * d.src_stride[k];
+        }
+    }
+    const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
+    __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+}
+
+template<int BYTES>
+bool launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, const void *src, hipStream_t stream) {
+    auto *pd = static_cast<uint8_t *>(dst);
+    auto *ps = static_cast<const uint8_t *>(src);
+    const uint64_t upr = desc.row_bytes / BYTES;
+    if (upr >= kWave && upr < (1ull << 31)) {
+        const dim3 grid(static_cast<unsigned>(ceil_div(upr, kBlock)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
+        rearrange_rows<BYTES><<<grid, kBlock, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+    } else {// short rows, or a single row too long for 32-bit column numbers
+        const uint64_t total = desc.rows * upr;
+        const uint64_t blocks = ceil_div(total, kBlock);
+        if (blocks > 0x7FFFFFFFull) {
+            return false;
+        }
+        if (total < (1ull << 32)) {
+            rearrange_flat<BYTES, uint32_t><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr));
+        } else {
+            rearrange_flat<BYTES, uint64_t><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, upr);
+        }
+    }
+    return true;
+}
+
+}// namespace
+
+// Stage 4 of Rearrange.
+infiniopStatus_t amdRearrange(RearrangeAmdDescriptor_t desc, void *dst, void const *src, void *stream) {
+    if (desc->rows == 0 || desc->row_bytes == 0) {
+        return STATUS_SUCCESS;
+    }
+    if (dst == nullptr || src == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    OuterDims d;
+    d.ndim = desc->ndim;
+    uint64_t align = desc->row_bytes | reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+    for (int k = 0; k < kRearrangeMaxDims; ++k) {
+        const bool used = k < desc->ndim;
+        if (used && desc->shape[k] >= (1ull << 32)) {
+            return STATUS_BAD_TENSOR_SHAPE;
+        }
+        d.shape[k] = used ? static_cast<uint32_t>(desc->shape[k]) : 1;
+        d.dst_stride[k] = used ? desc->dst_stride[k] : 0;
+        d.src_stride[k] = used ? desc->src_stride[k] : 0;
+        if (used) align |= static_cast<uint64_t>(desc->dst_stride[k]) | static_cast<uint64_t>(desc->src_stride[k]);
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    bool ok;
+    if (align % 16 == 0) ok = launch<16>(*desc, d, dst, src, s);
+    else if (align % 8 == 0) ok = launch<8>(*desc, d, dst, src, s);
+    else if (align % 4 == 0) ok = launch<4>(*desc, d, dst, src, s);
+    else if (align % 2 == 0) ok = launch<2>(*desc, d, dst, src, s);
+    else ok = launch<1>(*desc, d, dst, src, s);
+    if (!ok) {// more than 2^31 workgroups of short rows: beyond what one launch addresses
+        return STATUS_BAD_TENSOR_SHAPE;
+    }
+    AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+    return STATUS_SUCCESS;
+}

@@ -61,11 +61,16 @@ class CausalSoftmaxDescriptor(_OpDescriptor):
     pass
 
 
+class RearrangeDescriptor(_OpDescriptor):
+    pass
+
+
 infiniopAddDescriptor_t = POINTER(AddDescriptor)
 infiniopRMSNormDescriptor_t = POINTER(RMSNormDescriptor)
 infiniopRoPEDescriptor_t = POINTER(RoPEDescriptor)
 infiniopSwiGLUDescriptor_t = POINTER(SwiGLUDescriptor)
 infiniopCausalSoftmaxDescriptor_t = POINTER(CausalSoftmaxDescriptor)
+infiniopRearrangeDescriptor_t = POINTER(RearrangeDescriptor)
 
 
 class CTensor:
@@ -107,6 +112,9 @@ _PROTOTYPES = {
     "infiniopGetCausalSoftmaxWorkspaceSize": [infiniopCausalSoftmaxDescriptor_t, POINTER(c_uint64)],
     "infiniopCausalSoftmax": [infiniopCausalSoftmaxDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p],
     "infiniopDestroyCausalSoftmaxDescriptor": [infiniopCausalSoftmaxDescriptor_t],
+    "infiniopCreateRearrangeDescriptor": [infiniopHandle_t, POINTER(infiniopRearrangeDescriptor_t), infiniopTensorDescriptor_t, infiniopTensorDescriptor_t],
+    "infiniopRearrange": [infiniopRearrangeDescriptor_t, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroyRearrangeDescriptor": [infiniopRearrangeDescriptor_t],
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)

@@ -15,6 +15,7 @@ from .devices import DeviceEnum
 from .liboperators import (
     infiniopAddDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
+    infiniopRearrangeDescriptor_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
     infiniopSwiGLUDescriptor_t,
@@ -151,6 +152,24 @@ class CausalSoftmaxPlan(_Plan):
         return y
 
 
+class RearrangePlan(_Plan):
+    _destroy = "infiniopDestroyRearrangeDescriptor"
+
+    def __init__(self, ctx, dst, src):
+        super().__init__(ctx)
+        cts = self._describe(dst, src)
+        desc = infiniopRearrangeDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateRearrangeDescriptor(ctx.handle, ctypes.byref(desc), cts[0].descriptor, cts[1].descriptor))
+        finally:
+            self._release(cts)
+        self.desc = desc
+
+    def __call__(self, dst, src, stream=None):
+        check_error(self.lib.infiniopRearrange(self.desc, dst.data_ptr(), src.data_ptr(), stream))
+        return dst
+
+
 class Context:
     """A library handle on one GPU plus one-shot forms of the four operators."""
 
@@ -180,6 +199,10 @@ class Context:
     def rms_norm(self, y, x, w, epsilon=1e-5, stream=None):
         with RMSNormPlan(self, y, x, w, epsilon) as plan:
             return plan(y, x, w, stream)
+
+    def rearrange(self, dst, src, stream=None):
+        with RearrangePlan(self, dst, src) as plan:
+            return plan(dst, src, stream)
 
     def causal_softmax(self, y, stream=None):
         with CausalSoftmaxPlan(self, y) as plan:

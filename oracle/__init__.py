@@ -80,6 +80,9 @@ def lib():
         L.oracle_causal_softmax_check.argtypes, L.oracle_causal_softmax_check.restype = [tp, ctypes.c_int, ctypes.c_int], ctypes.c_int
         L.oracle_causal_softmax.argtypes = [u32, u64, u64, u64, i64, i64, i64, vp]
         L.oracle_causal_softmax.restype = ctypes.c_int
+        L.oracle_rearrange_check.argtypes, L.oracle_rearrange_check.restype = [tp, tp], ctypes.c_int
+        L.oracle_rearrange.argtypes = [u32, u64, vp, vp, vp, vp, vp]
+        L.oracle_rearrange.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -247,3 +250,20 @@ def causal_softmax(y, dtype):
     if rc != 0:
         raise RuntimeError(f"oracle_causal_softmax status {rc}")
     return y
+
+
+def rearrange_check(dst, src):
+    return lib().oracle_rearrange_check(dst.ref(), src.ref())
+
+
+def rearrange(dst, src):
+    """dst[...] = src[...]: numpy arrays (views) of equal shape and dtype, unit innermost strides."""
+    assert dst.shape == src.shape and dst.dtype == src.dtype
+    n, item = dst.ndim, dst.dtype.itemsize
+    shape = (ctypes.c_uint64 * n)(*dst.shape)
+    sd = (ctypes.c_int64 * n)(*[s // item for s in dst.strides])
+    ss = (ctypes.c_int64 * n)(*[s // item for s in src.strides])
+    rc = lib().oracle_rearrange(item, n, shape, sd, ss, _ptr(dst), _ptr(src))
+    if rc != 0:
+        raise RuntimeError(f"oracle_rearrange status {rc}")
+    return dst

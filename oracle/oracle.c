@@ -26,6 +26,9 @@
  *       available, a float64 softmax, rows summing to one, zeros above the
  *       diagonal.  (This operator is outside the four-operator hot path; it is
  *       the first of the operators that come next.)
+ *   oracle_rearrange                         pinned  - golden vectors written by
+ *       the compiled reference, the compiled reference itself, numpy's own
+ *       strided assignment.  (Second operator beyond the hot path.)
  *   bf16 variants of the operators           PARITY UNPINNED by the reference:
  *       no reference back end accepts bf16 for these operators.  The bf16
  *       arithmetic here is this project's extension (exact widening, the same
@@ -520,6 +523,70 @@ ORACLE_API int oracle_causal_softmax(uint32_t dt, uint64_t batch, uint64_t seq, 
                 store16(dt, row + (int64_t) j * stride_j, e);
             }
         }
+    }
+    return ST_SUCCESS;
+}
+
+/* ------------------------------------------------------------------------ *
+ * Rearrange (strided copy; second operator after the four-operator path)
+ * ------------------------------------------------------------------------ */
+
+/* Create-time checks of src/ops/rearrange/cpu/rearrange_cpu.cc:7-54 in the
+ * reference's order: equal element types; equal, non-zero rank and equal
+ * extents; unit innermost strides; for rank >= 4, dimensions 1..rank-3 must
+ * nest inside their predecessor (shape[i]*stride[i] == stride[i-1]) in both
+ * tensors. */
+ORACLE_API int oracle_rearrange_check(const oracle_tensor *dst, const oracle_tensor *src) {
+    if (dst->dt != src->dt) {
+        return ST_BAD_TENSOR_DTYPE;
+    }
+    uint64_t nd = dst->ndim;
+    if (src->ndim != nd || nd == 0) {
+        return ST_BAD_TENSOR_SHAPE;
+    }
+    for (uint64_t i = 0; i < nd; ++i) {
+        if (dst->shape[i] != src->shape[i]) {
+            return ST_BAD_TENSOR_SHAPE;
+        }
+    }
+    if (dst->strides[nd - 1] != 1 || src->strides[nd - 1] != 1) {
+        return ST_BAD_TENSOR_STRIDES;
+    }
+    if (nd >= 4) {
+        for (int64_t i = (int64_t) nd - 3; i >= 1; --i) {
+            if ((int64_t) dst->shape[i] * dst->strides[i] != dst->strides[i - 1] ||
+                (int64_t) src->shape[i] * src->strides[i] != src->strides[i - 1]) {
+                return ST_BAD_TENSOR_STRIDES;
+            }
+        }
+    }
+    return ST_SUCCESS;
+}
+
+/* dst[index] = src[index] for every index, rows of the innermost dimension
+ * moved as blocks of bytes (rearrange_cpu.cc:70-92).  Strides in elements of
+ * elem_size bytes.  Up to 16 dimensions. */
+ORACLE_API int oracle_rearrange(uint32_t elem_size, uint64_t ndim, const uint64_t *shape,
+                                const int64_t *dst_strides, const int64_t *src_strides,
+                                void *dst, const void *src) {
+    if (ndim == 0 || ndim > 16) {
+        return ST_BAD_TENSOR_SHAPE;
+    }
+    uint64_t rows = 1;
+    for (uint64_t i = 0; i + 1 < ndim; ++i) {
+        rows *= shape[i];
+    }
+    const uint64_t row_bytes = shape[ndim - 1] * elem_size;
+    for (uint64_t r = 0; r < rows; ++r) {
+        int64_t od = 0, os = 0;
+        uint64_t rest = r;
+        for (int64_t j = (int64_t) ndim - 2; j >= 0; --j) {
+            uint64_t k = rest % shape[j];
+            rest /= shape[j];
+            od += (int64_t) k * dst_strides[j];
+            os += (int64_t) k * src_strides[j];
+        }
+        memcpy((uint8_t *) dst + od * (int64_t) elem_size, (const uint8_t *) src + os * (int64_t) elem_size, row_bytes);
     }
     return ST_SUCCESS;
 }

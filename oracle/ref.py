@@ -17,6 +17,7 @@ from operators_amd.liboperators import (
     bind_prototypes,
     infiniopAddDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
+    infiniopRearrangeDescriptor_t,
     infiniopHandle_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
@@ -216,3 +217,25 @@ def causal_softmax(y, dtype):
     lib().infiniopDestroyCausalSoftmaxDescriptor(desc)
     _free(d)
     return y
+
+
+def rearrange_status(dst, src):
+    dd, ds = descriptor(*dst), descriptor(*src)
+    desc = infiniopRearrangeDescriptor_t()
+    st = lib().infiniopCreateRearrangeDescriptor(handle(), ctypes.byref(desc), dd, ds)
+    if st == 0:
+        lib().infiniopDestroyRearrangeDescriptor(desc)
+    _free(dd, ds)
+    return st
+
+
+def rearrange(dst, src, dtype):
+    dd, ds = _desc_of(dst, dtype), _desc_of(src, dtype)
+    desc = infiniopRearrangeDescriptor_t()
+    st = lib().infiniopCreateRearrangeDescriptor(handle(), ctypes.byref(desc), dd, ds)
+    assert st == 0, st
+    st = lib().infiniopRearrange(desc, dst.ctypes.data, src.ctypes.data, None)
+    assert st == 0, st
+    lib().infiniopDestroyRearrangeDescriptor(desc)
+    _free(dd, ds)
+    return dst

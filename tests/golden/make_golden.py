@@ -213,6 +213,47 @@ def causal_softmax_vectors(rng):
     return out
 
 
+REARRANGE_CASES = [
+    # (dtype, shape, src_strides or None, dst_strides or None): operatorspy/tests/rearrange.py:108-116, then more ranks and element sizes
+    ("f16", (2, 4, 32), None, (256, 64, 1)),
+    ("f16", (32, 6, 64), (64, 2560, 1), None),
+    ("f16", (4, 6, 64), (64, 2560, 1), (16384, 64, 1)),  # the reference uses 131072; shortened to keep the fixture small
+    ("f16", (1, 32, 64), (2048, 64, 1), (2048, 64, 1)),
+    ("f16", (32, 1, 64), (64, 2560, 1), (64, 64, 1)),
+    ("f16", (4, 1, 64), (64, 2560, 1), (64, 11264, 1)),
+    ("f16", (100,), None, None),
+    ("f32", (7, 33), (40, 1), (35, 1)),
+    ("u8", (5, 3, 13), (64, 16, 1), (45, 15, 1)),
+    ("f16", (2, 3, 4, 8), (3 * 64, 64, 10, 1), (3 * 40, 40, 9, 1)),
+    ("f64", (3, 2, 5), (40, 8, 1), None),
+]
+NP_OF = {"f16": np.uint16, "f32": np.float32, "u8": np.uint8, "f64": np.float64}
+
+
+def contiguous_strides(shape):
+    out, run = [], 1
+    for n in reversed(shape):
+        out.append(run)
+        run *= n
+    return tuple(reversed(out))
+
+
+def rearrange_vectors(rng):
+    out = {}
+    for i, (dt, shape, ss, sd) in enumerate(REARRANGE_CASES):
+        ss, sd = ss or contiguous_strides(shape), sd or contiguous_strides(shape)
+        item = np.dtype(NP_OF[dt]).itemsize
+        span = lambda st: 1 + sum((n - 1) * s for n, s in zip(shape, st))  # noqa: E731
+        src_buf = rng.integers(0, 200, span(ss) * item, dtype=np.uint8).view(NP_OF[dt])
+        dst_buf = rng.integers(0, 200, span(sd) * item, dtype=np.uint8).view(NP_OF[dt])
+        out[f"rearrange{i}_src"], out[f"rearrange{i}_dst_before"] = src_buf.copy(), dst_buf.copy()
+        src = np.lib.stride_tricks.as_strided(src_buf, shape, [s * item for s in ss])
+        dst = np.lib.stride_tricks.as_strided(dst_buf, shape, [s * item for s in sd])
+        ref.rearrange(dst, src, dt)
+        out[f"rearrange{i}_dst_after"] = dst_buf.copy()
+    return out
+
+
 def status_cases():
     """Create-time (and, for RMSNorm, compute-time) status codes of the reference."""
     cases = []
@@ -229,6 +270,8 @@ def status_cases():
             st = ref.rms_norm_status(*tensors, run=extra.get("run", False))
         elif op == "causal_softmax":
             st = ref.causal_softmax_status(*tensors)
+        elif op == "rearrange":
+            st = ref.rearrange_status(*tensors)
         cases.append({"op": op, "tensors": specs, "status": int(st), **extra})
 
     T = lambda dt, shape, st=None: (dt, tuple(shape), None if st is None else tuple(st))  # noqa: E731
@@ -293,6 +336,20 @@ def status_cases():
     rec("causal_softmax", [T("f32", (8, 16))])
     rec("causal_softmax", [T("bf16", (8, 16))], bf16_extension=True)
     rec("causal_softmax", [T("f16", (8, 16), (32, 2))], cpu_only_layout=True)  # accepted by the CPU back end, refused by the GPU ones
+    # rearrange (dst, src)
+    rec("rearrange", [T("f16", (4, 6, 64)), T("f16", (4, 6, 64), (64, 2560, 1))])
+    rec("rearrange", [T("f16", (64,)), T("f16", (64,))])
+    rec("rearrange", [T("f16", (4, 64)), T("f32", (4, 64))])
+    rec("rearrange", [T("f16", (4, 64)), T("f16", (4, 1, 64))])
+    rec("rearrange", [T("f16", ()), T("f16", ())])
+    rec("rearrange", [T("f16", (4, 64)), T("f16", (4, 32))])
+    rec("rearrange", [T("f16", (4, 64), (128, 2)), T("f16", (4, 64))])
+    rec("rearrange", [T("f16", (4, 64)), T("f16", (4, 64), (1, 4))])
+    rec("rearrange", [T("f16", (2, 3, 4, 8)), T("f16", (2, 3, 4, 8), (192, 64, 10, 1))])
+    rec("rearrange", [T("f16", (2, 3, 4, 8)), T("f16", (2, 3, 4, 8), (200, 64, 10, 1))])   # dim 1 does not nest in dim 0
+    rec("rearrange", [T("f16", (2, 2, 3, 4, 8)), T("f16", (2, 2, 3, 4, 8), (400, 192, 64, 10, 1))])  # dim 1 does not nest in dim 0
+    rec("rearrange", [T("bf16", (4, 64)), T("bf16", (4, 64))])
+    rec("rearrange", [T("u8", (4, 64)), T("u8", (4, 64), (100, 1))])
     return cases
 
 
@@ -305,10 +362,12 @@ def main():
     np.savez_compressed(os.path.join(HERE, "rope.npz"), **rope_vectors(rng))
     np.savez_compressed(os.path.join(HERE, "swiglu.npz"), **swiglu_vectors(rng))
     np.savez_compressed(os.path.join(HERE, "causal_softmax.npz"), **causal_softmax_vectors(rng))
+    np.savez_compressed(os.path.join(HERE, "rearrange.npz"), **rearrange_vectors(rng))
     with open(os.path.join(HERE, "status_cases.json"), "w") as f:
         json.dump({"add_cases": [list(map(list, c)) for c in ADD_CASES],
                    "rope_cases": [[list(s), None if st is None else list(st), r] for s, st, r in ROPE_CASES],
                    "swiglu_cases": [[list(s), a, b, c] for s, a, b, c in SWIGLU_CASES],
+                   "rearrange_cases": [[dt, list(sh), None if a is None else list(a), None if b is None else list(b)] for dt, sh, a, b in REARRANGE_CASES],
                    "causal_cases": [[list(s), None if st is None else list(st)] for s, st in CAUSAL_CASES],
                    "status": status_cases()}, f, indent=1)
     for name in sorted(os.listdir(HERE)):

@@ -1,0 +1,118 @@
+"""Rearrange on the GPU through the C ABI: byte-exact against the reference's
+golden vectors and the oracle, including the bytes it must not touch."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import golden, golden_json
+
+pytestmark = pytest.mark.gpu
+NP_OF = {"f16": np.uint16, "f32": np.float32, "u8": np.uint8, "f64": np.float64, "bf16": np.uint16}
+
+
+def torch_dtype(dt):
+    import torch
+
+    return {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32, "u8": torch.uint8, "f64": torch.float64}[dt]
+
+
+def contig(shape):
+    out, run = [], 1
+    for n in reversed(shape):
+        out.append(run)
+        run *= n
+    return list(reversed(out))
+
+
+def device_view(buf_np, dt, shape, strides):
+    """Upload a flat numpy buffer bit for bit and view it with the given strides."""
+    import torch
+
+    raw = torch.from_numpy(np.ascontiguousarray(buf_np).view(np.uint8).copy()).cuda()
+    typed = raw.view(torch_dtype(dt))
+    return torch.as_strided(typed, tuple(shape), tuple(strides)), raw
+
+
+def run_case(ctx, dt, shape, ss, sd, src_buf, dst_buf):
+    import torch
+
+    ss, sd = ss or contig(shape), sd or contig(shape)
+    src, _ = device_view(src_buf, dt, shape, ss)
+    dst, dst_raw = device_view(dst_buf, dt, shape, sd)
+    ctx.rearrange(dst, src)
+    torch.cuda.synchronize()
+    return dst_raw.cpu().numpy()
+
+
+def test_golden_cases(ctx):
+    g = golden("rearrange")
+    for i, (dt, shape, ss, sd) in enumerate(golden_json()["rearrange_cases"]):
+        got = run_case(ctx, dt, shape, ss, sd, g[f"rearrange{i}_src"], g[f"rearrange{i}_dst_before"])
+        assert np.array_equal(got, g[f"rearrange{i}_dst_after"].view(np.uint8)), (i, dt, shape, ss, sd)
+
+
+CASES = [
+    # dtype, shape, src strides, dst strides
+    ("f16", (2048, 8, 128), (80 * 128, 128, 1), (128, 2048 * 128, 1)),       # k heads of a fused qkv buffer -> [head, token, dim] cache
+    ("bf16", (512, 64, 128), (64 * 128, 128, 1), (128, 512 * 128, 1)),       # [token, head, dim] -> [head, token, dim]
+    ("f16", (64, 1000), (1000, 1), (1024, 1)),                               # row padding
+    ("f16", (33, 7, 5), (40, 5, 1), (35, 5, 1)),                             # odd row length: 2-byte units
+    ("u8", (9, 77), (80, 1), (77, 1)),                                       # 1-byte units
+    ("f32", (4, 3, 2, 50), (3 * 128, 128, 64, 1), (300, 100, 50, 1)),
+    ("f16", (1 << 20,), None, None),                                         # one contiguous row
+    ("f16", (3, 5, 7, 2, 16), (5 * 7 * 64, 7 * 64, 64, 32, 1), (5 * 7 * 32, 7 * 32, 32, 16, 1)),
+    ("f64", (100, 10), (16, 1), None),
+]
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_against_oracle(ctx, case):
+    dt, shape, ss, sd = CASES[case]
+    ss, sd = ss or contig(shape), sd or contig(shape)
+    item = np.dtype(NP_OF[dt]).itemsize
+    rng = np.random.default_rng(900 + case)
+    span = lambda st: 1 + sum((n - 1) * s for n, s in zip(shape, st))  # noqa: E731
+    src_buf = rng.integers(0, 256, span(ss) * item, dtype=np.uint8).view(NP_OF[dt])
+    dst_buf = rng.integers(0, 256, span(sd) * item, dtype=np.uint8).view(NP_OF[dt])
+    want_buf = dst_buf.copy()
+    src = np.lib.stride_tricks.as_strided(src_buf, shape, [s * item for s in ss])
+    dst = np.lib.stride_tricks.as_strided(want_buf, shape, [s * item for s in sd])
+    oracle.rearrange(dst, src)
+    got = run_case(ctx, dt, shape, ss, sd, src_buf, dst_buf)
+    assert np.array_equal(got, want_buf.view(np.uint8)), (dt, shape, ss, sd)
+
+
+def test_misaligned_base_pointers(ctx):
+    """Views that start 2 bytes into their buffers fall back to narrower units."""
+    import torch
+
+    rng = np.random.default_rng(950)
+    src_np = rng.integers(0, 65536, 4096 * 3 + 1, dtype=np.uint16)
+    src_all = torch.from_numpy(src_np.view(np.int16)).cuda().view(torch.float16)
+    dst_all = torch.zeros(64 * 200 + 1, dtype=torch.float16, device="cuda")
+    src = torch.as_strided(src_all[1:], (64, 128), (192, 1))
+    dst = torch.as_strided(dst_all[1:], (64, 128), (200, 1))
+    ctx.rearrange(dst, src)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(torch.int16), src.view(torch.int16))
+    assert dst_all[0] == 0 and not dst_all[1:].view(64, 200)[:, 128:].any()
+
+
+def test_status_codes_match_reference(ctx):
+    import ctypes
+
+    from operators_amd import infiniopRearrangeDescriptor_t, make_descriptor
+    from oracle.ref import LAYOUT
+
+    lib = ctx.lib
+    for case in golden_json()["status"]:
+        if case["op"] != "rearrange":
+            continue
+        descs = [make_descriptor(lib, t[1], t[2], LAYOUT[t[0]]) for t in case["tensors"]]
+        d = infiniopRearrangeDescriptor_t()
+        st = lib.infiniopCreateRearrangeDescriptor(ctx.handle, ctypes.byref(d), *descs)
+        assert st == case["status"], (case, st)
+        if st == 0:
+            assert lib.infiniopDestroyRearrangeDescriptor(d) == 0
+        for x in descs:
+            lib.infiniopDestroyTensorDescriptor(x)

@@ -288,3 +288,34 @@ def test_causal_softmax_against_float64(dt):
     assert np.all(got[:, ~keep] == 0) and np.all(got[:, keep] > 0)
     assert np.all(np.abs(got.sum(-1) - 1) < 40 * ulp)  # truncation loses up to one ulp per kept element
     assert got[:, 0, : total - seq + 1].min() > 0 and np.count_nonzero(got[:, 0]) == 3 * (total - seq + 1)
+
+
+# ---- rearrange (second operator beyond the four-operator path) ------------------------
+NP_OF = {"f16": np.uint16, "f32": np.float32, "u8": np.uint8, "f64": np.float64}
+
+
+def _views(g, i, dt, shape, ss, sd):
+    def contig(sh):
+        out, run = [], 1
+        for n in reversed(sh):
+            out.append(run)
+            run *= n
+        return list(reversed(out))
+    item = np.dtype(NP_OF[dt]).itemsize
+    ss, sd = ss or contig(shape), sd or contig(shape)
+    src_buf, dst_buf = g[f"rearrange{i}_src"].copy(), g[f"rearrange{i}_dst_before"].copy()
+    src = np.lib.stride_tricks.as_strided(src_buf, shape, [s * item for s in ss])
+    dst = np.lib.stride_tricks.as_strided(dst_buf, shape, [s * item for s in sd])
+    return src, dst, dst_buf
+
+
+def test_rearrange_golden_and_numpy():
+    g = golden("rearrange")
+    for i, (dt, shape, ss, sd) in enumerate(golden_json()["rearrange_cases"]):
+        src, dst, dst_buf = _views(g, i, dt, shape, ss, sd)
+        oracle.rearrange(dst, src)
+        assert np.array_equal(dst_buf.view(np.uint8), g[f"rearrange{i}_dst_after"].view(np.uint8)), (i, dt, shape)
+        # and numpy's own strided assignment says the same
+        src2, dst2, dst_buf2 = _views(g, i, dt, shape, ss, sd)
+        dst2[...] = src2
+        assert np.array_equal(dst_buf2.view(np.uint8), dst_buf.view(np.uint8))

@@ -32,6 +32,9 @@ def test_oracle_checks_reproduce_reference_status(i):
         st = oracle.swiglu_check(*specs, allow_bf16=False)
     elif case["op"] == "rope":
         st = oracle.rope_check(*specs, allow_bf16=False)
+    elif case["op"] == "rearrange":
+        assert oracle.rearrange_check(*specs) == case["status"], case
+        return
     elif case["op"] == "causal_softmax":
         st = oracle.causal_softmax_check(specs[0], allow_bf16=False, unit_inner=False)
         assert st == case["status"], case
@@ -74,6 +77,7 @@ CREATE = {
     "swiglu": ("infiniopCreateSwiGLUDescriptor", "infiniopDestroySwiGLUDescriptor", oa.infiniopSwiGLUDescriptor_t),
     "rope": ("infiniopCreateRoPEDescriptor", "infiniopDestroyRoPEDescriptor", oa.infiniopRoPEDescriptor_t),
     "rms_norm": ("infiniopCreateRMSNormDescriptor", "infiniopDestroyRMSNormDescriptor", oa.infiniopRMSNormDescriptor_t),
+    "rearrange": ("infiniopCreateRearrangeDescriptor", "infiniopDestroyRearrangeDescriptor", oa.infiniopRearrangeDescriptor_t),
     "causal_softmax": ("infiniopCreateCausalSoftmaxDescriptor", "infiniopDestroyCausalSoftmaxDescriptor", oa.infiniopCausalSoftmaxDescriptor_t),
 }
 
