@@ -51,7 +51,7 @@ __device__ __attribute__((noinline)) float exp_any(float d) { return expf(d); }
 // lies in the masked part re-reads the row's last kept vector, which the
 // memory pipeline merges into one request - so that the compiler can count
 // the loads in flight and wait for the current row only.
-template<typename T, int BS, int NV>
+template<typename T, int BS, int NV, bool THROUGH>
 __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
                                                           int64_t stride_b, int64_t stride_i) {
     constexpr int WAVES = BS / kWave;
@@ -146,6 +146,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
         }
         const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
         const float rcp = 1.0f / sum;
+        const StreamOut<THROUGH> out(row.ptr);// the row is the same for every lane of the workgroup
 
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -161,9 +162,9 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
 #pragma unroll
                     for (int e = 0; e < 8; ++e) o[e] = v * 8 + e < keep ? o[e] : 0.0f;
                 }
-                st16_stream(row.ptr + static_cast<uint64_t>(v) * 8, narrow8_unit_range<T>(o));
+                out.st16(v * 16, narrow8_unit_range<T>(o));
             } else if (v < nvec) {
-                st16_stream(row.ptr + static_cast<uint64_t>(v) * 8, u32x4{0, 0, 0, 0});
+                out.st16(v * 16, u32x4{0, 0, 0, 0});
             }
         }
     };
@@ -238,8 +239,16 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         causal_softmax_generic<T><<<grid, 256, 0, stream>>>(py, rows, d.seq, d.total, d.stride_b, d.stride_i);
         return;
     }
-#define CS_LAUNCH(BS, NV) \
-    causal_softmax_rows<T, BS, NV><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i)
+    const bool through = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
+#define CS_LAUNCH(BS, NV)                                                                                                          \
+    do {                                                                                                                           \
+        if (through)                                                                                                               \
+            causal_softmax_rows<T, BS, NV, true><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),                  \
+                                                                          static_cast<uint32_t>(d.total), d.stride_b, d.stride_i); \
+        else                                                                                                                       \
+            causal_softmax_rows<T, BS, NV, false><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),                 \
+                                                                           static_cast<uint32_t>(d.total), d.stride_b, d.stride_i); \
+    } while (0)
     if (nvec <= 64) CS_LAUNCH(64, 1);
     else if (nvec <= 128) CS_LAUNCH(64, 2);
     else if (nvec <= 256) CS_LAUNCH(64, 4);

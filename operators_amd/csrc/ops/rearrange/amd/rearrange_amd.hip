@@ -32,7 +32,9 @@ template<> struct Unit<1> { typedef uint8_t type; };
 // wavefront of units.  The row's offsets are found by dividing the row number
 // by the merged outer extents - once per workgroup row, on the scalar unit,
 // since the row number is uniform.
-template<int BYTES>
+// BUFST (16-byte units, large outputs): stores are written through L2 as
+// buffer stores relative to the start of the destination row (see StreamOut).
+template<int BYTES, bool BUFST>
 __global__ __launch_bounds__(kBlock) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row) {
     typedef typename Unit<BYTES>::type U;
     const uint32_t col = blockIdx.x * kBlock + threadIdx.x;
@@ -50,14 +52,20 @@ __global__ __launch_bounds__(kBlock) void rearrange_rows(uint8_t *dst, const uin
             }
         }
         const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
-        __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+        if constexpr (BUFST) {
+            StreamOut<true>(dst + od).st16(col * 16, v);
+        } else {
+            __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+        }
     }
 }
 
 // Short rows: one lane per unit over the flat (row, unit) space, one unit per
 // lane and one workgroup per 256 units.  Idx is 32-bit when the unit count
-// allows, which makes the divisions cheap.
-template<int BYTES, typename Idx>
+// allows, which makes the divisions cheap.  BUFST (16-byte units only): the
+// whole destination lies within 4 GiB of its base and no stride is negative,
+// so stores go out as buffer stores relative to the base (see StreamOut).
+template<int BYTES, typename Idx, bool BUFST>
 __global__ __launch_bounds__(kBlock) void rearrange_flat(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t total_units, Idx units_per_row) {
     typedef typename Unit<BYTES>::type U;
     const uint64_t idx64 = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
@@ -78,7 +86,11 @@ __global__ __launch_bounds__(kBlock) void rearrange_flat(uint8_t *dst, const uin
         }
     }
     const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
-    __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+    if constexpr (BUFST) {
+        StreamOut<true>(dst).st16(static_cast<uint32_t>(od) + static_cast<uint32_t>(col) * 16, v);
+    } else {
+        __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+    }
 }
 
 template<int BYTES>
@@ -86,9 +98,21 @@ bool launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
     auto *pd = static_cast<uint8_t *>(dst);
     auto *ps = static_cast<const uint8_t *>(src);
     const uint64_t upr = desc.row_bytes / BYTES;
+    const bool large = desc.rows * desc.row_bytes >= kWriteThroughBytes;// worth writing through L2
+    // where the destination ends, in bytes from its base, when no stride is negative
+    bool forward = true;
+    uint64_t dst_span = desc.row_bytes;
+    for (int k = 0; k < d.ndim; ++k) {
+        forward = forward && d.dst_stride[k] >= 0;
+        dst_span += (d.shape[k] - 1) * static_cast<uint64_t>(d.dst_stride[k] >= 0 ? d.dst_stride[k] : 0);
+    }
     if (upr >= kWave && upr < (1ull << 31)) {
         const dim3 grid(static_cast<unsigned>(ceil_div(upr, kBlock)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
-        rearrange_rows<BYTES><<<grid, kBlock, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+        if (BYTES == 16 && large && desc.row_bytes < (1ull << 32)) {
+            rearrange_rows<BYTES, BYTES == 16><<<grid, kBlock, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+        } else {
+            rearrange_rows<BYTES, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+        }
     } else {// short rows, or a single row too long for 32-bit column numbers
         const uint64_t total = desc.rows * upr;
         const uint64_t blocks = ceil_div(total, kBlock);
@@ -96,9 +120,13 @@ bool launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
             return false;
         }
         if (total < (1ull << 32)) {
-            rearrange_flat<BYTES, uint32_t><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr));
+            if (BYTES == 16 && large && forward && dst_span < (1ull << 32)) {
+                rearrange_flat<BYTES, uint32_t, BYTES == 16><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr));
+            } else {
+                rearrange_flat<BYTES, uint32_t, false><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr));
+            }
         } else {
-            rearrange_flat<BYTES, uint64_t><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, upr);
+            rearrange_flat<BYTES, uint64_t, false><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, upr);
         }
     }
     return true;

@@ -76,7 +76,7 @@ enum WeightHome { kWGlobal = 0, kWLds = 1 };
 // (and their value replaced by zero) rather than branched around: with
 // straight-line loads the compiler can count how many are still in flight and
 // wait for the current row only, not for the prefetched one.
-template<typename T, typename W, int BS, int NV, int WHOME, bool EXACT>
+template<typename T, typename W, int BS, int NV, int WHOME, bool EXACT, bool THROUGH>
 __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w,
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps) {
     constexpr int WAVES = BS / kWave;
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
         }
         const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
 
-        uint16_t *yr = y + static_cast<int64_t>(r) * stride_y;
+        const StreamOut<THROUGH> yr(y + static_cast<int64_t>(r) * stride_y);// a row is far shorter than 4 GiB
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = k * BS + threadIdx.x;
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
                 }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
-                st16_stream(yr + static_cast<uint64_t>(v) * 8, narrow8<T>(f));
+                yr.st16(v * 16, narrow8<T>(f));
             }
         }
     };
@@ -251,14 +251,20 @@ void launch_rms_norm(const RMSNormAmdDescriptor &desc, void *y, const void *x, c
         home = kWGlobal;// one row per workgroup: staging would only add a pass
     }
 
-#define RMS_LAUNCH_HOME(BS, NV, HOME, LDS)                                                                              \
+    const bool through = n * d * sizeof(uint16_t) >= kWriteThroughBytes;
+#define RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, EXACT)                                                                      \
     do {                                                                                                                \
-        if (nvec == static_cast<uint64_t>(BS) * NV)                                                                     \
-            rms_norm_rows<T, W, BS, NV, HOME, true><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(                  \
+        if (through)                                                                                                    \
+            rms_norm_rows<T, W, BS, NV, HOME, EXACT, true><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(           \
                 py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon);                    \
         else                                                                                                            \
-            rms_norm_rows<T, W, BS, NV, HOME, false><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(                 \
+            rms_norm_rows<T, W, BS, NV, HOME, EXACT, false><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(          \
                 py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon);                    \
+    } while (0)
+#define RMS_LAUNCH_HOME(BS, NV, HOME, LDS)                                                                              \
+    do {                                                                                                                \
+        if (nvec == static_cast<uint64_t>(BS) * NV) RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, true);                          \
+        else RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, false);                                                                \
     } while (0)
 #define RMS_LAUNCH(BS, NV)                                                                                              \
     do {                                                                                                                \
@@ -276,6 +282,7 @@ void launch_rms_norm(const RMSNormAmdDescriptor &desc, void *y, const void *x, c
     else RMS_LAUNCH(1024, 8);
 #undef RMS_LAUNCH
 #undef RMS_LAUNCH_HOME
+#undef RMS_LAUNCH_EXACT
 }
 
 template<typename T>

@@ -29,12 +29,30 @@ using namespace amd;
 constexpr int kBlock = 256;
 constexpr int kHeadsPerLane = 4;// 2 and 4 measure within 2 % of each other on MI355X; 1 and 8 are slower
 
+// The token of the wavefront's first lane, as a wavefront-uniform value: lanes
+// are numbered in item order, so it is the smallest token the wavefront
+// touches, and the base address of the wavefront's buffer stores.
+template<typename Idx>
+__device__ __forceinline__ Idx first_lane(Idx v) {
+    if constexpr (sizeof(Idx) == 4) {
+        return static_cast<Idx>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
+    } else {
+        const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(v))));
+        const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(v >> 32))));
+        return static_cast<Idx>((static_cast<uint64_t>(hi) << 32) | lo);
+    }
+}
+
 // One lane = one 8-element column group `cv` of up to HPT heads of one token.
 // Work items are numbered (token, head group g, cv) with cv fastest, so the
 // lanes of a wavefront cover consecutive 16-byte pieces of consecutive heads.
 // Lane (g, cv) rotates heads g, g+G, g+2G, ... (G = number of head groups):
 // at every step the wavefront's accesses are again to neighbouring heads.
-template<typename T, typename Idx, int HPT>
+// BUFST: results are written through L2 by buffer stores relative to the
+// wavefront's first token (see StreamOut); the host selects it for large
+// outputs when strides are non-negative and the 64 tokens a wavefront can span
+// fit a 32-bit byte offset.
+template<typename T, typename Idx, int HPT, bool BUFST>
 __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
                                                    uint64_t total_items, Idx items_per_token, Idx vecs_per_head, Idx groups,
                                                    uint32_t heads, uint32_t head_dim, int64_t stride_token, int64_t stride_head) {
@@ -47,6 +65,9 @@ __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *
     const Idx cv = rem - g * vecs_per_head;
 
     uint16_t *base = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(cv) * 8;
+    const Idx token0 = BUFST ? first_lane(token) : token;
+    const StreamOut<true> out(t + static_cast<int64_t>(token0) * stride_token);
+    const uint32_t off = static_cast<uint32_t>(token - token0) * static_cast<uint32_t>(stride_token) * 2 + static_cast<uint32_t>(cv) * 16;
 
     u32x4 tv[HPT];
 #pragma unroll
@@ -75,7 +96,11 @@ __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *
                 r[k] = ac - bs;
                 r[k + 1] = as + bc;
             }
-            st16_stream(base + static_cast<int64_t>(h) * stride_head, narrow8<T>(r));
+            if constexpr (BUFST) {
+                out.st16(off + h * static_cast<uint32_t>(stride_head) * 2, narrow8<T>(r));
+            } else {
+                st16_stream(base + static_cast<int64_t>(h) * stride_head, narrow8<T>(r));
+            }
         }
     }
 }
@@ -91,11 +116,13 @@ struct RopeTile {
     u32x4 tv[HPT];
     f32x4 s_lo, s_hi, c_lo, c_hi;
     uint16_t *base;
+    uint16_t *out_base;// wavefront-uniform: the first lane's token
+    uint32_t off;      // this lane's byte offset from out_base, head 0
     uint32_t g;
     bool live;
 };
 
-template<typename T, typename Idx, int HPT>
+template<typename T, typename Idx, int HPT, bool BUFST>
 __global__ __launch_bounds__(kBlock) void rope_vec_loop(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
                                                         uint64_t total_items, Idx items_per_token, Idx vecs_per_head, Idx groups,
                                                         uint32_t heads, uint32_t head_dim, int64_t stride_token, int64_t stride_head) {
@@ -110,6 +137,11 @@ __global__ __launch_bounds__(kBlock) void rope_vec_loop(uint16_t *t, const uint6
         const Idx cv = rem - g * vecs_per_head;
         r.g = static_cast<uint32_t>(g);
         r.base = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(cv) * 8;
+        if constexpr (BUFST) {
+            const Idx token0 = first_lane(token);
+            r.out_base = t + static_cast<int64_t>(token0) * stride_token;
+            r.off = static_cast<uint32_t>(token - token0) * static_cast<uint32_t>(stride_token) * 2 + static_cast<uint32_t>(cv) * 16;
+        }
 #pragma unroll
         for (int i = 0; i < HPT; ++i) {
             uint32_t h = r.g + i * static_cast<uint32_t>(groups);
@@ -123,6 +155,7 @@ __global__ __launch_bounds__(kBlock) void rope_vec_loop(uint16_t *t, const uint6
     auto rotate = [&](const RopeTile<T, HPT> &r) {
         const float sn[8] = {r.s_lo.x, r.s_lo.y, r.s_lo.z, r.s_lo.w, r.s_hi.x, r.s_hi.y, r.s_hi.z, r.s_hi.w};
         const float cs[8] = {r.c_lo.x, r.c_lo.y, r.c_lo.z, r.c_lo.w, r.c_hi.x, r.c_hi.y, r.c_hi.z, r.c_hi.w};
+        const StreamOut<true> out(BUFST ? r.out_base : t);
 #pragma unroll
         for (int i = 0; i < HPT; ++i) {
             const uint32_t h = r.g + i * static_cast<uint32_t>(groups);
@@ -137,7 +170,13 @@ __global__ __launch_bounds__(kBlock) void rope_vec_loop(uint16_t *t, const uint6
                 o[k + 1] = as + bc;
             }
             const u32x4 packed = narrow8<T>(o);
-            if (r.live && h < heads) st16_stream(r.base + static_cast<int64_t>(h) * stride_head, packed);
+            if (r.live && h < heads) {
+                if constexpr (BUFST) {
+                    out.st16(r.off + h * static_cast<uint32_t>(stride_head) * 2, packed);
+                } else {
+                    st16_stream(r.base + static_cast<int64_t>(h) * stride_head, packed);
+                }
+            }
         }
     };
 
@@ -193,6 +232,12 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
     const uint64_t ipt = groups * vph;
     const uint64_t total = d.tokens * ipt;
     const unsigned grid = static_cast<unsigned>(ceil_div(total, kBlock));
+    // Large outputs are written through L2 with buffer stores, which address
+    // 32 bits from the first token of a wavefront (it spans at most 64 tokens).
+    const bool bufst = d.tokens * d.heads * d.head_dim * sizeof(uint16_t) >= kWriteThroughBytes &&
+                       d.stride_token >= 0 && d.stride_head >= 0 &&
+                       static_cast<uint64_t>(d.stride_token) < (1ull << 23) &&
+                       d.heads * static_cast<uint64_t>(d.stride_head) < (1ull << 30) && d.head_dim < (1ull << 24);
     // Enough tiles to keep every compute unit looping: the prefetching form.
     // Measured on MI355X (256 compute units): q [8192,64,128] bf16, 8192 tiles,
     // 47.0 us looping with 2 workgroups per unit against 48.5 us one tile per
@@ -203,23 +248,35 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
         const uint64_t per_cu = grid >= 16u * static_cast<unsigned>(d.cu_count) ? 2 : 4;
         const uint64_t cap = static_cast<uint64_t>(d.cu_count) * per_cu;
         const unsigned lgrid = static_cast<unsigned>(grid < cap ? grid : cap);
-#define ROPE_LAUNCH_LOOP(HPT)                                                                                                       \
-    rope_vec_loop<T, Idx, HPT><<<lgrid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph),   \
-                                                             static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),              \
-                                                             static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
-        if (hpt == 4) ROPE_LAUNCH_LOOP(4);
-        else if (hpt == 2) ROPE_LAUNCH_LOOP(2);
-        else ROPE_LAUNCH_LOOP(1);
+#define ROPE_LAUNCH_LOOP(HPT, B)                                                                                                    \
+    rope_vec_loop<T, Idx, HPT, B><<<lgrid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph), \
+                                                                static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),           \
+                                                                static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
+        if (bufst) {
+            if (hpt == 4) ROPE_LAUNCH_LOOP(4, true);
+            else if (hpt == 2) ROPE_LAUNCH_LOOP(2, true);
+            else ROPE_LAUNCH_LOOP(1, true);
+        } else {
+            if (hpt == 4) ROPE_LAUNCH_LOOP(4, false);
+            else if (hpt == 2) ROPE_LAUNCH_LOOP(2, false);
+            else ROPE_LAUNCH_LOOP(1, false);
+        }
 #undef ROPE_LAUNCH_LOOP
         return;
     }
-#define ROPE_LAUNCH(HPT)                                                                                                   \
-    rope_vec<T, Idx, HPT><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph), \
-                                                       static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),            \
-                                                       static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
-    if (hpt == 4) ROPE_LAUNCH(4);
-    else if (hpt == 2) ROPE_LAUNCH(2);
-    else ROPE_LAUNCH(1);
+#define ROPE_LAUNCH(HPT, B)                                                                                                   \
+    rope_vec<T, Idx, HPT, B><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph), \
+                                                          static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),           \
+                                                          static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
+    if (bufst) {
+        if (hpt == 4) ROPE_LAUNCH(4, true);
+        else if (hpt == 2) ROPE_LAUNCH(2, true);
+        else ROPE_LAUNCH(1, true);
+    } else {
+        if (hpt == 4) ROPE_LAUNCH(4, false);
+        else if (hpt == 2) ROPE_LAUNCH(2, false);
+        else ROPE_LAUNCH(1, false);
+    }
 #undef ROPE_LAUNCH
 }
 

@@ -62,6 +62,9 @@ CASES = [
     ("f16", (1 << 20,), None, None),                                         # one contiguous row
     ("f16", (3, 5, 7, 2, 16), (5 * 7 * 64, 7 * 64, 64, 32, 1), (5 * 7 * 32, 7 * 32, 32, 16, 1)),
     ("f64", (100, 10), (16, 1), None),
+    # 128 MiB outputs: large enough for the write-through store path of both kernels
+    ("bf16", (8192, 64, 128), (80 * 128, 128, 1), (128, 8192 * 128, 1)),     # q heads -> [head, token, dim], 256-byte rows
+    ("f16", (4096, 16384), (16384, 1), (16392, 1)),                          # long rows into a padded destination
 ]
 
 
