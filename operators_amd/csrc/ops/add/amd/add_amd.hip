@@ -7,8 +7,8 @@
 //
 // The operation moves 3 bytes per byte of output and computes almost nothing,
 // so everything here is about keeping HBM busy: 16 bytes per lane per access,
-// several independent accesses in flight per lane, non-temporal hints on data
-// that is touched once.
+// memory walked in address order, non-temporal hints on data that is touched
+// once.
 #include "../../../devices/amd/kernel_amd.h"
 #include "add_amd.h"
 
@@ -16,14 +16,15 @@ namespace {
 
 using namespace amd;
 
-// Launch shape of the flat kernel, chosen by measurement on MI355X at
-// [8192, 4096] fp16 and [8192, 8192] bf16: 256 lanes, 4 accesses per lane per
-// operand, at most 32 workgroups per compute unit looping over tiles gives
-// 77-81 % of the 8 TB/s peak; 1 or 2 accesses per lane, 512 or 1024 lanes, or
-// one workgroup per tile are all within 2 % of it or slower.
-constexpr int kBlock = 256;  // lanes per workgroup
-constexpr int kUnroll = 4;   // independent 16-byte accesses per lane per operand
-constexpr int kFlatPerCu = 32;
+// Launch shape of the flat kernel, chosen by measurement on MI355X with a
+// stand-alone c = a + b over 3 x 128 MiB: workgroups of one wavefront with one
+// 16-byte access per lane per operand, one workgroup per KiB of output, take
+// 61.4 us; 128 lanes 61.6; 256 lanes 63.1-63.7; 2 or 4 accesses per lane
+// 62.7-65.8; workgroups that loop over tiles (16-64 per compute unit)
+// 65.4-69.6.  The broadcast kernels keep 256 lanes: with an operand that is
+// re-read through the caches, [8192, 4096] fp16 plus a [4096] row takes 25.4 us
+// that way and 32.2 us with single-wavefront workgroups.
+constexpr int kBlock = 256;// lanes per workgroup of the broadcast and element-wise kernels
 
 // ---- per-type arithmetic on one 128-bit word ---------------------------------
 template<typename T>
@@ -62,43 +63,17 @@ struct Add32 {
 };
 
 // ---- no broadcasting: c[i] = a[i] + b[i] over a flat range -------------------
-// Each workgroup walks tiles of kBlock*kUnroll vectors; inside a tile lane l
-// takes vectors l, l+kBlock, ... so every access instruction of a wavefront
-// covers 1 KiB of consecutive memory.  All loads of a tile are issued before
-// the first add.
+// One wavefront per workgroup, one vector per lane, one workgroup per KiB: the
+// dispatcher hands out consecutive KiBs in order and every wavefront gives its
+// slot back the moment it is done.  (The loop only runs more than once for
+// ranges beyond 2^31 workgroups.)
 template<typename Op>
-__global__ __launch_bounds__(kBlock) void add_flat_vec(u32x4 *c, const u32x4 *a, const u32x4 *b, uint64_t nvec) {
-    constexpr uint64_t kTile = static_cast<uint64_t>(kBlock) * kUnroll;
-    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kTile;
-    for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kTile; base < nvec; base += step) {
-        u32x4 va[kUnroll], vb[kUnroll];
-        if (base + kTile <= nvec) {
-#pragma unroll
-            for (int k = 0; k < kUnroll; ++k) {
-                const uint64_t i = base + k * kBlock + threadIdx.x;
-                va[k] = ld16_stream(a + i);
-                vb[k] = ld16_stream(b + i);
-            }
-#pragma unroll
-            for (int k = 0; k < kUnroll; ++k) {
-                const uint64_t i = base + k * kBlock + threadIdx.x;
-                st16_stream(c + i, Op::vec(va[k], vb[k]));
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < kUnroll; ++k) {
-                const uint64_t i = base + k * kBlock + threadIdx.x;
-                if (i < nvec) {
-                    va[k] = ld16_stream(a + i);
-                    vb[k] = ld16_stream(b + i);
-                }
-            }
-#pragma unroll
-            for (int k = 0; k < kUnroll; ++k) {
-                const uint64_t i = base + k * kBlock + threadIdx.x;
-                if (i < nvec) st16_stream(c + i, Op::vec(va[k], vb[k]));
-            }
-        }
+__global__ __launch_bounds__(kWave) void add_flat_vec(u32x4 *c, const u32x4 *a, const u32x4 *b, uint64_t nvec) {
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * kWave;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kWave + threadIdx.x; i < nvec; i += step) {
+        const u32x4 va = ld16_stream(a + i);
+        const u32x4 vb = ld16_stream(b + i);
+        st16_stream(c + i, Op::vec(va, vb));
     }
 }
 
@@ -215,7 +190,8 @@ __global__ __launch_bounds__(kBlock) void add_bcast_scalar(typename Op::scalar *
 inline unsigned grid_for(uint64_t work_items, uint64_t per_block, int cu_count, int blocks_per_cu) {
     const uint64_t want = ceil_div(work_items, per_block);
     const uint64_t cap = blocks_per_cu > 0 ? static_cast<uint64_t>(cu_count) * blocks_per_cu : want;
-    const uint64_t g = want < cap ? want : cap;
+    uint64_t g = want < cap ? want : cap;
+    g = g < 0x7FFFFFFFull ? g : 0x7FFFFFFFull;// the kernels stride over whatever one launch cannot index
     return static_cast<unsigned>(g == 0 ? 1 : g);
 }
 
@@ -230,8 +206,8 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         if (aligned16(c) && aligned16(a) && aligned16(b)) {
             const uint64_t nvec = n / Op::kPerVec;
             if (nvec > 0) {
-                const unsigned grid = grid_for(nvec, static_cast<uint64_t>(kBlock) * kUnroll, cus, kFlatPerCu);
-                add_flat_vec<Op><<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const u32x4 *>(a),
+                const unsigned grid = grid_for(nvec, kWave, cus, 0);
+                add_flat_vec<Op><<<grid, kWave, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const u32x4 *>(a),
                                                               static_cast<const u32x4 *>(b), nvec);
             }
             done = nvec * Op::kPerVec;

@@ -226,12 +226,15 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
     // Rows of up to 4096 elements are taken by single wavefronts (no barrier, no
-    // LDS; 32 such workgroups per compute unit), longer ones by 256-1024 lanes
-    // (8 per unit).  Measured on MI355X at [32, 4096, 4096] fp16: 317 us with
-    // one row per wavefront against 338-360 us with 128, 256 or 512 lanes per
-    // row; a plain kernel that reads half of every 8 KiB row and writes all of
-    // it - the traffic of this operator without any arithmetic - needs 284 us.
-    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * (nvec <= 512 ? 32 : 8);
+    // LDS), longer ones by 256-1024 lanes (8 workgroups per compute unit).
+    // Measured on MI355X at [32, 4096, 4096] fp16: one row per wavefront is
+    // 6-13 % faster than 128, 256 or 512 lanes per row.  The grid of the
+    // single-wavefront form is several times what the chip holds at once
+    // (16 such wavefronts per compute unit), so the dispatcher evens out the
+    // triangular load while each workgroup still prefetches across its few
+    // rows: 32 workgroups per unit 314 us, 64 288, 96 281, 128 277, 256 278,
+    // one workgroup per row 293.
+    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * (nvec <= 512 ? 128 : 8);
     const unsigned grid = static_cast<unsigned>(rows < cap ? rows : cap);
 
     const bool vec_ok = d.total % 8 == 0 && nvec <= 4096 && d.seq < (1ull << 31) && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);
