@@ -244,7 +244,11 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
     // workgroup; [4096,32,128] fp16, 2048 tiles, 14.1 us (4 per unit) against
     // 16.8 us; k [8192,8,128], 1024 tiles, is faster one tile per workgroup
     // (9.7 against 10.5 us) and stays on rope_vec.  Workgroups of 64 or 128
-    // lanes, one tile each, measure the same as 256 for all three shapes.
+    // lanes, one tile each, measure the same as 256 for all three shapes, and
+    // so does a 2-D grid with the token in blockIdx.y (position and table base
+    // then come through scalar loads): 47.3 us for q.  With table loads and
+    // arithmetic removed the looping form takes 44.7 us for q, so they cost
+    // 1.7 us; an out-of-place copy of the same strided rows takes 41.9 us.
     if (grid >= 8u * static_cast<unsigned>(d.cu_count)) {
         const uint64_t per_cu = grid >= 16u * static_cast<unsigned>(d.cu_count) ? 2 : 4;
         const uint64_t cap = static_cast<uint64_t>(d.cu_count) * per_cu;
