@@ -18,7 +18,12 @@ object: `value` is algorithmic bytes moved per second over the whole chain;
 `roofline` describes the dominant kernel (SwiGLU) timed on its own with events
 on the launch stream; `cpu_baseline` is the CPU oracle timed on this host on a
 bounded sample of the same workload; `ops` lists every operator/configuration
-with its own time, bandwidth and fraction of the 8 TB/s peak.
+with its own time, bandwidth and fraction of the 8 TB/s peak: per row one cold
+first call (buffers never touched before; includes one-time code loading where
+the kernel has not run yet in the process), then at least 20 warm-up calls and
+5 runs of at least 40 calls each between two events, rotating over buffer
+sets; `us_per_call` is the median run, `us_min`/`us_max` the fastest and
+slowest.
 """
 import argparse
 import json
@@ -34,7 +39,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 # HBM bytes per launch of the dominant kernel at the default workload
 # (swiglu bf16 [8192, 28672] from a fused [8192, 57344] buffer), measured with
 # rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each scaled by what the same
-# counter reads for a plain 128 MiB device copy (1.99959 and 1.00000); the runs
+# counter reads for a plain 128 MiB device copy (1.99960 and 1.00000); the runs
 # are summarised in profiles/c5_kernels_hbm_traffic_pmc.txt.  Algorithmic bytes
 # for the same launch: 1 409 286 144.
 MEASURED_TRAFFIC_SWIGLU_8192 = 1409141585
@@ -203,14 +208,34 @@ def sets_needed(touched_bytes, minimum):
     return max(minimum, min(MAX_SETS, -(-ROTATE_BYTES // max(1, touched_bytes))))
 
 
-def op_entry(name, config, sets, steps, warmup):
+def op_entry(name, config, sets, steps, warmup, repeats):
+    """One row of the per-operator table: a cold first call, then `repeats`
+    timed runs of `steps` calls each (rotating over the buffer sets) after
+    `warmup` untimed calls; the row reports the median run."""
+    import torch
+
+    stream = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record(stream)
+    sets[-1](stream.cuda_stream)  # first call on these buffers: nothing of them is in any cache
+    e1.record(stream)
+    torch.cuda.synchronize()
+    cold_us = e0.elapsed_time(e1) * 1e3
+
     steps = max(steps, 2 * len(sets))
-    wall, ev = time_rotating([[s] for s in sets], steps, warmup)
-    per_call = ev / steps
+    runs = []
+    for rep in range(repeats):
+        _, ev = time_rotating([[s] for s in sets], steps, warmup if rep == 0 else 0)
+        runs.append(ev / steps)
+    runs.sort()
+    per_call = runs[len(runs) // 2]
     nbytes = sets[0].nbytes
     gbps = nbytes / per_call / 1e9
-    return {"op": name, "config": config, "us_per_call": round(per_call * 1e6, 3), "bytes": nbytes,
-            "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4), "buffer_sets": len(sets), "calls": steps}
+    return {"op": name, "config": config, "us_per_call": round(per_call * 1e6, 3), "us_min": round(runs[0] * 1e6, 3),
+            "us_max": round(runs[-1] * 1e6, 3), "cold_first_call_us": round(cold_us, 1), "bytes": nbytes,
+            "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4), "buffer_sets": len(sets),
+            "calls_per_run": steps, "runs": repeats, "warmup_calls": warmup}
 
 
 def ops_table(ctx, args, gen):
@@ -265,7 +290,12 @@ def ops_table(ctx, args, gen):
         if args.only and args.only not in label:
             continue
         sets = build()
-        rows.append(op_entry(sets[0].name, label, sets, args.steps, args.warmup))
+        # the table proper: 20 warm-up calls, 5 runs of >= 40 calls, median; a single
+        # named row (profiling) runs exactly what was asked for, once
+        if args.only:
+            rows.append(op_entry(sets[0].name, label, sets, args.steps, args.warmup, 1))
+        else:
+            rows.append(op_entry(sets[0].name, label, sets, max(args.steps, 40), max(args.warmup, 20), 5))
         del sets
         torch.cuda.empty_cache()
     return rows
@@ -345,6 +375,17 @@ def cpu_per_op(T):
     gu5 = codes((T, 57344), "bf16")
     o5 = np.empty((T, 28672), np.uint16)
     run("C5 swiglu", "bf16", lambda: oracle.swiglu(gu5[:, 28672:], gu5[:, :28672], "bf16", c=o5), None)
+    del gu5, o5
+    # the two operators beyond the four-operator path
+    q6 = codes((T, 80, 128), "bf16")
+    d6 = np.empty((64, T, 128), np.uint16)
+    run("N2 rearrange", "f16", lambda: oracle.rearrange(d6.transpose(1, 0, 2), q6[:, :64, :]), lambda: ref.rearrange(d6.transpose(1, 0, 2), q6[:, :64, :], "f16"))
+    del q6, d6
+    # causal softmax: 2 of the 32 [4096, 4096] matrices, scaled to the whole batch (every matrix costs the same)
+    y7 = codes((2, 4096, 4096), "f16")
+    run("N1 causal_softmax", "f16", lambda: oracle.causal_softmax(y7, "f16"), lambda: ref.causal_softmax(y7, "f16"))
+    out["N1 causal_softmax"]["cpu_us_per_call"] = round(out["N1 causal_softmax"]["cpu_us_per_call"] * 16, 1)
+    out["N1 causal_softmax"]["cpu_sample"] = "2 of 32 matrices, x16"
     return out
 
 
