@@ -144,6 +144,20 @@ def make_rearrange(ctx, tokens, heads, dtype, gen, name):
     return Launch(name, ctx.lib.infiniopRearrange, (plan.desc, dst.data_ptr(), src.data_ptr()), 2 * src.numel() * src.element_size(), (plan, qkv, cache))
 
 
+def make_add_rms_norm(ctx, n, d, dtype, w_dtype, gen, name):
+    """The fused residual form: c = a + b, y = RMSNorm(c) * w; c updates the residual a in place."""
+    import torch
+
+    from operators_amd.ops import AddRMSNormPlan
+
+    a, b = _randn((n, d), dtype, gen), _randn((n, d), dtype, gen)
+    w = (torch.rand(d, device="cuda", dtype=torch.float32, generator=gen) + 0.5).to(w_dtype)
+    y = torch.empty_like(a)
+    plan = AddRMSNormPlan(ctx, y, a, a, b, w, 1e-5)
+    nbytes = 4 * n * d * a.element_size() + w.numel() * w.element_size()
+    return Launch(name, ctx.lib.infiniopAddRMSNorm, (plan.desc, None, 0, y.data_ptr(), a.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr()), nbytes, (plan, a, b, w, y))
+
+
 def make_add(ctx, n, d, dtype, broadcast, gen, name):
     import torch
 
@@ -274,6 +288,7 @@ def ops_table(ctx, args, gen):
         f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(sets_needed(6 * T * 8192, nset))],
         # beyond the four-operator path: attention scores of 32 heads, 4096 x 4096, in place
         f"N2 rearrange bf16 [{T},64,128] of [{T},80,128] -> [64,{T},128]": lambda: [make_rearrange(ctx, T, 64, bf16, gen, "rearrange") for _ in range(sets_needed(4 * T * 64 * 128, nset))],
+        f"F1 add_rms_norm bf16 [{T},8192] w f32 (fused Add + RMSNorm)": lambda: [make_add_rms_norm(ctx, T, 8192, bf16, torch.float32, gen, "add_rms_norm") for _ in range(sets_needed(6 * T * 8192, nset))],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:

@@ -3,7 +3,9 @@
  *
  * The library implements ONE device of the InfiniOperators operator library,
  * `DevAmdGpu` (AMD Instinct MI355X, gfx950), for the four memory-bound LLM-layer
- * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax and Rearrange.  The entry points below have the
+ * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax, Rearrange and
+ * a fused AddRMSNorm (the one operator here that the reference does not have).
+ * The entry points below have the
  * names, argument order, argument meaning and status codes of the reference
  * library, so that a caller written against the reference (its ctypes harness,
  * its composite operators, any C client) binds to this library unchanged and
@@ -14,7 +16,7 @@
  *   1. infiniopCreateHandle(&handle, DevAmdGpu, device_id)
  *   2. infiniopCreate<Op>Descriptor(handle, &desc, tensor descriptors...)
  *        all shape/stride/dtype checking happens here, once
- *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax; always 0)
+ *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, AddRMSNorm; always 0)
  *   4. infiniop<Op>(desc, ..., data pointers..., stream)
  *        enqueues on `stream` (a hipStream_t, NULL = the null stream) and
  *        returns without synchronising
@@ -263,5 +265,36 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRearrange(
     infiniopRearrangeDescriptor_t desc, void *dst, void const *src, void *stream);
 /* replaces include/ops/rearrange/rearrange.h:19 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyRearrangeDescriptor(infiniopRearrangeDescriptor_t desc);
+
+/* ======================================================================== *
+ * AddRMSNorm (fused residual form; no counterpart in the reference, whose
+ * callers issue infiniopAdd and then infiniopRMSNorm on the sum):
+ *     c[i][j] = a[i][j] + b[i][j]                       rounded as Add rounds
+ *     y[i][j] = c[i][j] * w[j] / sqrt(mean_j(c[i][j]^2) + epsilon)
+ * in one pass over memory.  y and c are bit for bit what infiniopAdd followed
+ * by infiniopRMSNorm of this library produce.  y, c, a, b: 2-D [n, d], one
+ * element type (F16 or BF16), unit inner strides, free row strides; w: 1-D
+ * [d], F16, BF16 or F32.  c may be a or b; y must not overlap the others.
+ * ======================================================================== */
+typedef struct AddRMSNormDescriptor {
+    Device device;
+} AddRMSNormDescriptor;
+typedef AddRMSNormDescriptor *infiniopAddRMSNormDescriptor_t;
+
+/* no counterpart in the reference; argument order follows include/ops/rms_norm/rms_norm.h:13-19
+ * with the Add operands (include/ops/add/add.h:13-17) between y and w */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateAddRMSNormDescriptor(
+    infiniopHandle_t handle, infiniopAddRMSNormDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t y_desc, infiniopTensorDescriptor_t c_desc,
+    infiniopTensorDescriptor_t a_desc, infiniopTensorDescriptor_t b_desc,
+    infiniopTensorDescriptor_t w_desc, float epsilon);
+/* no counterpart in the reference (pattern of include/ops/rms_norm/rms_norm.h:21) - always 0 bytes */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetAddRMSNormWorkspaceSize(infiniopAddRMSNormDescriptor_t desc, uint64_t *size);
+/* no counterpart in the reference (pattern of include/ops/rms_norm/rms_norm.h:23-24) */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopAddRMSNorm(
+    infiniopAddRMSNormDescriptor_t desc, void *workspace, uint64_t workspace_size,
+    void *y, void *c, void const *a, void const *b, void const *w, void *stream);
+/* no counterpart in the reference (pattern of include/ops/rms_norm/rms_norm.h:26) */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyAddRMSNormDescriptor(infiniopAddRMSNormDescriptor_t desc);
 
 #endif /* INFINIOP_AMD_INFINIOP_H */

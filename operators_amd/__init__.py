@@ -11,6 +11,7 @@ from .devices import DeviceEnum  # noqa: F401
 from .liboperators import (  # noqa: F401
     CTensor,
     infiniopAddDescriptor_t,
+    infiniopAddRMSNormDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
     infiniopHandle_t,
     infiniopRearrangeDescriptor_t,

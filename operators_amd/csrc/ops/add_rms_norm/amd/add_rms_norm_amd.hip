@@ -1,0 +1,36 @@
+// Stage 4 of the fused Add + RMSNorm: RMSNorm's kernels in their residual form
+// (rms_norm_kernels.h).  Each row of a and b is read once; the sum is rounded
+// as Add rounds it, written to c, and normalised from registers, so the pair
+// moves 4 bytes per byte of y instead of the 5 that Add followed by RMSNorm
+// moves.  y and c are bit for bit what those two calls produce.
+//
+// c may be a or b (the residual stream updated in place); y must not overlap
+// any of the others, and rows must not overlap each other.
+#include "add_rms_norm_amd.h"
+#include "../../rms_norm/amd/rms_norm_kernels.h"
+
+using namespace rms_norm_kernels;
+
+infiniopStatus_t amdAddRMSNorm(AddRMSNormAmdDescriptor_t desc, void *, uint64_t, void *y, void *c, void const *a,
+                               void const *b, void const *w, void *stream) {
+    if (desc->elem != amd::Elem::F16 && desc->elem != amd::Elem::BF16) {
+        return STATUS_BAD_TENSOR_DTYPE;
+    }
+    if (desc->n == 0 || desc->d == 0) {
+        return STATUS_SUCCESS;
+    }
+    if (y == nullptr || c == nullptr || a == nullptr || b == nullptr || w == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const RowsShape shape{desc->cu_count, desc->lds_per_block, desc->n, desc->d, desc->stride_y, desc->stride_a, desc->epsilon};
+    const Residual<true> res{static_cast<uint16_t *>(c), static_cast<const uint16_t *>(b), desc->stride_c, desc->stride_b};
+    const bool ok = desc->elem == amd::Elem::F16 ? launch_by_weight<amd::F16Ref, true>(desc->w_elem, shape, y, a, w, res, s)
+                                                 : launch_by_weight<amd::BF16Rne, true>(desc->w_elem, shape, y, a, w, res, s);
+    if (!ok) {
+        return STATUS_BAD_TENSOR_DTYPE;
+    }
+    AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+    return STATUS_SUCCESS;
+}

@@ -1,0 +1,379 @@
+// Device code of RMSNorm on gfx950, shared by the plain operator and the fused
+// residual form (Add + RMSNorm in one pass).  Include from .hip files only.
+//
+// Arithmetic contract (reference src/ops/rms_norm/cpu/rms_norm_cpu.cc:46-86):
+//     ss   = sum_j x[j]^2                      fp32
+//     k    = (ss / d + eps) ^ -1/2             fp32 mean, double power
+//     y[j] = narrow( (k * x[j]) * w[j] )
+// The reference adds the squares left to right and carries the two products
+// in double before narrowing; here the sum is a tree over lanes and waves and
+// the products are fp32.  Both differences are below one fp32 ulp of y and
+// show up, after narrowing to 16 bits, as a last-bit difference on roughly one
+// element in 10^4.  fp16 narrows by the reference's truncation, bf16
+// (extension) rounds to nearest even.
+//
+// Data movement is the whole cost: x is read once and kept in registers
+// between the reduction and the scaling pass, y is written once, and the
+// weight row - re-used by every row - is staged once per workgroup in LDS as
+// fp32 when a workgroup serves more than one row.
+#ifndef INFINIOP_AMD_RMS_NORM_KERNELS_H
+#define INFINIOP_AMD_RMS_NORM_KERNELS_H
+
+#include "../../../devices/amd/common_amd.h"
+#include "../../../devices/amd/kernel_amd.h"
+
+namespace rms_norm_kernels {
+
+using namespace amd;
+
+// ---- weight row access ----------------------------------------------------------
+struct WF32 {
+    typedef float scalar;
+    __device__ static __forceinline__ void load8(const void *w, uint32_t vec, float (&g)[8]) {
+        const float *p = static_cast<const float *>(w) + static_cast<uint64_t>(vec) * 8;
+        const f32x4 a = ld16f(p), b = ld16f(p + 4);
+        g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
+        g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
+    }
+    __device__ static __forceinline__ float one(const void *w, uint64_t j) { return static_cast<const float *>(w)[j]; }
+};
+template<typename T>
+struct W16 {
+    typedef uint16_t scalar;
+    __device__ static __forceinline__ void load8(const void *w, uint32_t vec, float (&g)[8]) {
+        widen8<T>(ld16(static_cast<const uint16_t *>(w) + static_cast<uint64_t>(vec) * 8), g);
+    }
+    __device__ static __forceinline__ float one(const void *w, uint64_t j) {
+        return T::one(static_cast<const uint16_t *>(w)[j]);
+    }
+};
+
+__device__ __forceinline__ float inv_rms(float sum_sq, uint64_t d, float eps) {
+    const float mean_eps = sum_sq / static_cast<float>(d) + eps;
+    return static_cast<float>(1.0 / sqrt(static_cast<double>(mean_eps)));
+}
+
+// ---- rows that fit in registers -----------------------------------------------
+// One workgroup of BS lanes per row at a time; lane l owns vectors l, l+BS, ...
+// (NV of them, 8 elements each), so d <= 8*BS*NV.  Workgroups stride over rows
+// and fetch the next row's x before reducing the current one, so a load is
+// always in flight while the reduction, the barrier and the stores happen.
+//
+// Where the weight row lives while a workgroup works through its rows:
+//   kWGlobal: re-read from memory for every row (one row per workgroup, or a
+//             row too long for LDS)
+//   kWLds   : staged once in LDS as fp32
+// Measured at [8192, 8192] bf16 with fp32 weights: 45.7 us with the weights in
+// LDS, 47.0-50.6 us when every row re-reads them through L2 (one workgroup per
+// row, or 8-16 looping workgroups per compute unit); keeping each lane's 8*NV
+// weights in registers instead of LDS is no faster than LDS.  Giving every
+// wavefront a row of its own (16 vectors per lane, DPP-only reduction, no
+// barrier, weights shared in LDS by the 4 wavefronts of a workgroup) takes
+// 50.3-53.4 us against 44.6 us for one row per 256 lanes.
+//
+// LDS layout of the staged weight row: the 8 floats of vector v are split into
+// two 16-byte halves stored at lo[v] and hi[v] (hi = lo + nvec).  A wavefront
+// reading lo[v..v+63] or hi[v..v+63] then touches 64 consecutive 16-byte words
+// - no two lanes on the same bank in the same phase - where the natural
+// 32-byte-per-lane layout would be a two-way conflict.
+enum WeightHome { kWGlobal = 0, kWLds = 1 };
+
+// EXACT means d == 8*BS*NV: every lane owns NV whole vectors and no access is
+// predicated.  Otherwise loads of absent vectors are redirected to vector 0
+// (and their value replaced by zero) rather than branched around: with
+// straight-line loads the compiler can count how many are still in flight and
+// wait for the current row only, not for the prefetched one.
+//
+// ADD is the fused residual form: x is one of two addends, res carries the
+// other (b) and where their sum goes (c).  The sum is rounded to the element
+// type exactly as the Add operator rounds it, stored, and that rounded row is
+// what gets normalised - the results are those of Add followed by RMSNorm,
+// with the sum read from registers instead of from memory.
+template<bool ADD>
+struct Residual {};
+template<>
+struct Residual<true> {
+    uint16_t *c;
+    const uint16_t *b;
+    int64_t stride_c, stride_b;
+};
+
+template<typename T, typename W, int BS, int NV, int WHOME, bool EXACT, bool THROUGH, bool ADD>
+__global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w,
+                                                     uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
+                                                     Residual<ADD> res) {
+    constexpr int WAVES = BS / kWave;
+    __shared__ float red[2 * WAVES];
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
+    f32x4 *w_lo = reinterpret_cast<f32x4 *>(dyn_lds);
+    const uint32_t nvec = d / 8;
+    f32x4 *w_hi = w_lo + nvec;
+
+    constexpr int NB = ADD ? NV : 1;// registers for the second addend only in the fused form
+    auto load_row = [&](uint64_t row, u32x4(&dst)[NV], u32x4(&dst_b)[NB]) {
+        const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            dst[k] = ld16_stream(xr + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
+        }
+        if constexpr (ADD) {
+            const uint16_t *br = res.b + static_cast<int64_t>(row) * res.stride_b;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                dst_b[k] = ld16_stream(br + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
+            }
+        }
+    };
+
+    uint64_t row = blockIdx.x;
+    if (row >= n) return;
+    u32x4 xv[NV], xn[NV], bv[NB], bn[NB];
+    load_row(row, xv, bv);// in flight while the weights are fetched below
+
+    if constexpr (WHOME == kWLds) {
+        // all of this lane's weight loads are issued before the first is
+        // consumed: one memory latency for the staging, not one per vector
+        float g[NV][8];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            W::load8(w, EXACT || v < nvec ? v : 0, g[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            if (EXACT || v < nvec) {
+                w_lo[v] = f32x4{g[k][0], g[k][1], g[k][2], g[k][3]};
+                w_hi[v] = f32x4{g[k][4], g[k][5], g[k][6], g[k][7]};
+            }
+        }
+        __syncthreads();
+    }
+
+    // One row: reduce, scale by the weights, store.
+    auto finish_row = [&](uint64_t r, u32x4(&cur)[NV], const u32x4(&cur_b)[NB], int phase) {
+        if constexpr (ADD) {// cur += cur_b, rounded as Add rounds, and out to c
+            const StreamOut<THROUGH> cr(res.c + static_cast<int64_t>(r) * res.stride_c);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                float p[8], q[8];
+                widen8<T>(cur[k], p);
+                widen8<T>(cur_b[k], q);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) p[i] += q[i];
+                cur[k] = narrow8<T>(p);
+                if (EXACT || v < nvec) cr.st16(v * 16, cur[k]);
+            }
+        }
+        float part = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            float f[8];
+            widen8<T>(cur[k], f);
+            if constexpr (!EXACT) {
+                if (k * BS + threadIdx.x >= nvec) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) f[i] = 0.0f;
+                }
+            }
+            // pairwise inside the vector, then onto the running partial
+            const float s01 = f[0] * f[0] + f[1] * f[1], s23 = f[2] * f[2] + f[3] * f[3];
+            const float s45 = f[4] * f[4] + f[5] * f[5], s67 = f[6] * f[6] + f[7] * f[7];
+            part += (s01 + s23) + (s45 + s67);
+        }
+        const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
+
+        const StreamOut<THROUGH> yr(y + static_cast<int64_t>(r) * stride_y);// a row is far shorter than 4 GiB
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            if (EXACT || v < nvec) {
+                float f[8], g[8];
+                widen8<T>(cur[k], f);
+                if constexpr (WHOME == kWLds) {
+                    const f32x4 a = w_lo[v], b = w_hi[v];
+                    g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
+                    g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
+                } else {
+                    W::load8(w, v, g);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
+                yr.st16(v * 16, narrow8<T>(f));
+            }
+        }
+    };
+
+    // Steady state: the next row's loads are issued, unconditionally, before
+    // the current row is reduced.  Two register sets take turns (no copies, so
+    // the wait for a prefetched row comes only when that row is reduced) and a
+    // row's loads are never issued unless this workgroup owns that row.
+    const uint64_t hop = gridDim.x;
+    while (true) {
+        if (row + hop >= n) {
+            finish_row(row, xv, bv, 0);
+            break;
+        }
+        load_row(row + hop, xn, bn);
+        finish_row(row, xv, bv, 0);
+        row += hop;
+        if (row + hop >= n) {
+            finish_row(row, xn, bn, 1);
+            break;
+        }
+        load_row(row + hop, xv, bv);
+        finish_row(row, xn, bn, 1);
+        row += hop;
+    }
+}
+
+// ---- any row length, any alignment ----------------------------------------------
+// Two passes over the row with element accesses; the second pass re-reads x,
+// which the first pass left in cache for rows of ordinary length.
+template<typename T, typename W, bool ADD>
+__global__ __launch_bounds__(256) void rms_norm_generic(uint16_t *y, const uint16_t *x, const void *w,
+                                                         uint64_t n, uint64_t d, int64_t stride_y, int64_t stride_x, float eps,
+                                                         Residual<ADD> res) {
+    constexpr int BS = 256, WAVES = BS / kWave;
+    __shared__ float red[2 * WAVES];
+    int phase = 0;
+    for (uint64_t row = blockIdx.x; row < n; row += gridDim.x, phase ^= 1) {
+        const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
+        uint16_t *yr = y + static_cast<int64_t>(row) * stride_y;
+        float part = 0.0f;
+        if constexpr (ADD) {// first pass forms and stores the sum; the second pass reads it back from c
+            const uint16_t *br = res.b + static_cast<int64_t>(row) * res.stride_b;
+            uint16_t *cr = res.c + static_cast<int64_t>(row) * res.stride_c;
+            for (uint64_t j = threadIdx.x; j < d; j += BS) {
+                const uint16_t sum = T::narrow1(T::one(xr[j]) + T::one(br[j]));
+                cr[j] = sum;
+                const float f = T::one(sum);
+                part += f * f;
+            }
+            xr = cr;
+        } else {
+            for (uint64_t j = threadIdx.x; j < d; j += BS) {
+                const float f = T::one(xr[j]);
+                part += f * f;
+            }
+        }
+        const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
+        for (uint64_t j = threadIdx.x; j < d; j += BS) {
+            yr[j] = T::narrow1((k_row * T::one(xr[j])) * W::one(w, j));
+        }
+        // y may alias x (and c may alias a or b): every lane re-reads only elements it wrote itself.
+    }
+}
+
+// ---- launch -----------------------------------------------------------------------
+// What a launch needs to know about the operator instance.
+struct RowsShape {
+    int cu_count;
+    int lds_per_block;
+    uint64_t n, d;
+    int64_t stride_y, stride_x;
+    float epsilon;
+};
+
+template<typename T, typename W, bool ADD>
+void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *w, const Residual<ADD> &res, hipStream_t stream) {
+    auto *py = static_cast<uint16_t *>(y);
+    auto *px = static_cast<const uint16_t *>(x);
+    const uint64_t n = desc.n, d = desc.d;
+    const uint64_t nvec = d / 8;
+
+    bool vec_ok = d % 8 == 0 && nvec <= 8192 && desc.stride_x % 8 == 0 && desc.stride_y % 8 == 0 &&
+                  aligned16(x) && aligned16(y) && aligned16(w);
+    if constexpr (ADD) {
+        vec_ok = vec_ok && res.stride_b % 8 == 0 && res.stride_c % 8 == 0 && aligned16(res.b) && aligned16(res.c);
+    }
+    if (!vec_ok) {
+        const uint64_t cap = static_cast<uint64_t>(desc.cu_count) * 8;
+        rms_norm_generic<T, W, ADD><<<static_cast<unsigned>(n < cap ? n : cap), 256, 0, stream>>>(
+            py, px, w, n, d, desc.stride_y, desc.stride_x, desc.epsilon, res);
+        return;
+    }
+
+    // A workgroup that serves several rows fetches the weights once: into LDS
+    // as fp32 when the row leaves room for at least two workgroups per compute
+    // unit, else it re-reads them from memory like a one-row workgroup does.
+    const uint64_t lds_bytes = d * sizeof(float);
+    const uint64_t lds_limit = static_cast<uint64_t>(desc.lds_per_block) - 1024;
+    // With the next row always in flight, one workgroup per compute unit already
+    // reaches the bandwidth this access pattern allows (measured at [8192, 8192]
+    // bf16: 1, 2, 3 and 4 per unit all give 73.3-74.0 % of peak); 2 keeps some
+    // slack while staging the weights only 512 times.  Shorter rows put fewer
+    // bytes in flight per workgroup, so they get proportionally more of them.
+    uint64_t per_cu = ceil_div(32 * 1024, d * sizeof(uint16_t));
+    per_cu = per_cu < 2 ? 2 : (per_cu > 16 ? 16 : per_cu);
+    int home = kWLds;
+    if (lds_bytes <= lds_limit && lds_bytes <= 64 * 1024) {
+        const uint64_t fit = (160 * 1024) / (lds_bytes + 256);// 160 KiB of LDS per compute unit
+        per_cu = fit < per_cu ? fit : per_cu;
+    } else {
+        home = kWGlobal;
+    }
+    uint64_t grid = static_cast<uint64_t>(desc.cu_count) * per_cu;
+    if (n <= grid) {
+        grid = n;
+        home = kWGlobal;// one row per workgroup: staging would only add a pass
+    }
+
+    const bool through = n * d * sizeof(uint16_t) >= kWriteThroughBytes;
+#define RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, EXACT)                                                                      \
+    do {                                                                                                                \
+        if (through)                                                                                                    \
+            rms_norm_rows<T, W, BS, NV, HOME, EXACT, true, ADD><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(      \
+                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res);                \
+        else                                                                                                            \
+            rms_norm_rows<T, W, BS, NV, HOME, EXACT, false, ADD><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(     \
+                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res);                \
+    } while (0)
+#define RMS_LAUNCH_HOME(BS, NV, HOME, LDS)                                                                              \
+    do {                                                                                                                \
+        if (nvec == static_cast<uint64_t>(BS) * NV) RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, true);                          \
+        else RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, false);                                                                \
+    } while (0)
+#define RMS_LAUNCH(BS, NV)                                                                                              \
+    do {                                                                                                                \
+        if (home == kWLds) RMS_LAUNCH_HOME(BS, NV, kWLds, lds_bytes);                                                   \
+        else RMS_LAUNCH_HOME(BS, NV, kWGlobal, 0);                                                                      \
+    } while (0)
+
+    if (nvec <= 64) RMS_LAUNCH(64, 1);
+    else if (nvec <= 128) RMS_LAUNCH(128, 1);
+    else if (nvec <= 256) RMS_LAUNCH(256, 1);
+    else if (nvec <= 512) RMS_LAUNCH(256, 2);
+    else if (nvec <= 1024) RMS_LAUNCH(256, 4);// d = 8192: 512x2 measures the same, 1024x1 is 8 % slower
+    else if (nvec <= 2048) RMS_LAUNCH(512, 4);
+    else if (nvec <= 4096) RMS_LAUNCH(1024, 4);
+    else RMS_LAUNCH(1024, 8);
+#undef RMS_LAUNCH
+#undef RMS_LAUNCH_HOME
+#undef RMS_LAUNCH_EXACT
+}
+
+// Weight element type -> kernel family.  False when the type is not supported.
+template<typename T, bool ADD>
+bool launch_by_weight(amd::Elem w_elem, const RowsShape &desc, void *y, const void *x, const void *w, const Residual<ADD> &res, hipStream_t s) {
+    switch (w_elem) {
+        case amd::Elem::F32:
+            launch_rms_norm<T, WF32, ADD>(desc, y, x, w, res, s);
+            return true;
+        case amd::Elem::F16:
+            launch_rms_norm<T, W16<amd::F16Ref>, ADD>(desc, y, x, w, res, s);
+            return true;
+        case amd::Elem::BF16:
+            launch_rms_norm<T, W16<amd::BF16Rne>, ADD>(desc, y, x, w, res, s);
+            return true;
+        default:
+            return false;
+    }
+}
+
+}// namespace rms_norm_kernels
+
+#endif

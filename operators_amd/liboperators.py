@@ -65,12 +65,17 @@ class RearrangeDescriptor(_OpDescriptor):
     pass
 
 
+class AddRMSNormDescriptor(_OpDescriptor):
+    pass
+
+
 infiniopAddDescriptor_t = POINTER(AddDescriptor)
 infiniopRMSNormDescriptor_t = POINTER(RMSNormDescriptor)
 infiniopRoPEDescriptor_t = POINTER(RoPEDescriptor)
 infiniopSwiGLUDescriptor_t = POINTER(SwiGLUDescriptor)
 infiniopCausalSoftmaxDescriptor_t = POINTER(CausalSoftmaxDescriptor)
 infiniopRearrangeDescriptor_t = POINTER(RearrangeDescriptor)
+infiniopAddRMSNormDescriptor_t = POINTER(AddRMSNormDescriptor)
 
 
 class CTensor:
@@ -115,15 +120,26 @@ _PROTOTYPES = {
     "infiniopCreateRearrangeDescriptor": [infiniopHandle_t, POINTER(infiniopRearrangeDescriptor_t), infiniopTensorDescriptor_t, infiniopTensorDescriptor_t],
     "infiniopRearrange": [infiniopRearrangeDescriptor_t, c_void_p, c_void_p, c_void_p],
     "infiniopDestroyRearrangeDescriptor": [infiniopRearrangeDescriptor_t],
+    "infiniopCreateAddRMSNormDescriptor": [infiniopHandle_t, POINTER(infiniopAddRMSNormDescriptor_t)] + [infiniopTensorDescriptor_t] * 5 + [c_float],
+    "infiniopGetAddRMSNormWorkspaceSize": [infiniopAddRMSNormDescriptor_t, POINTER(c_uint64)],
+    "infiniopAddRMSNorm": [infiniopAddRMSNormDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroyAddRMSNormDescriptor": [infiniopAddRMSNormDescriptor_t],
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
 
 
-def bind_prototypes(lib):
+# Entry points of this library that the reference does not have.
+EXTENSION_SYMBOLS = tuple(n for n in _PROTOTYPES if "AddRMSNorm" in n)
+
+
+def bind_prototypes(lib, extensions=True):
     """Attach argument and result types for every entry point.  Works on any
-    library exporting the same C ABI (this one, or a build of the reference)."""
+    library exporting the same C ABI: this one, or (with extensions=False) a
+    build of the reference, which lacks the fused operator."""
     for name, argtypes in _PROTOTYPES.items():
+        if not extensions and name in EXTENSION_SYMBOLS:
+            continue
         fn = getattr(lib, name)  # AttributeError names the missing symbol
         fn.argtypes = argtypes
         fn.restype = c_int32

@@ -16,6 +16,7 @@ from .liboperators import (
     infiniopAddDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
     infiniopRearrangeDescriptor_t,
+    infiniopAddRMSNormDescriptor_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
     infiniopSwiGLUDescriptor_t,
@@ -109,6 +110,29 @@ class RMSNormPlan(_Plan):
         return y
 
 
+class AddRMSNormPlan(_Plan):
+    """c = a + b; y = RMSNorm(c) * w in one pass (the reference issues Add, then RMSNorm)."""
+
+    _destroy = "infiniopDestroyAddRMSNormDescriptor"
+
+    def __init__(self, ctx, y, c, a, b, w, epsilon):
+        super().__init__(ctx)
+        cts = self._describe(y, c, a, b, w)
+        desc = infiniopAddRMSNormDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateAddRMSNormDescriptor(ctx.handle, ctypes.byref(desc), *[ct.descriptor for ct in cts], epsilon))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetAddRMSNormWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value
+
+    def __call__(self, y, c, a, b, w, stream=None):
+        check_error(self.lib.infiniopAddRMSNorm(self.desc, None, self.workspace_size, y.data_ptr(), c.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr(), stream))
+        return y, c
+
+
 class RoPEPlan(_Plan):
     _destroy = "infiniopDestroyRoPEDescriptor"
 
@@ -199,6 +223,10 @@ class Context:
     def rms_norm(self, y, x, w, epsilon=1e-5, stream=None):
         with RMSNormPlan(self, y, x, w, epsilon) as plan:
             return plan(y, x, w, stream)
+
+    def add_rms_norm(self, y, c, a, b, w, epsilon=1e-5, stream=None):
+        with AddRMSNormPlan(self, y, c, a, b, w, epsilon) as plan:
+            return plan(y, c, a, b, w, stream)
 
     def rearrange(self, dst, src, stream=None):
         with RearrangePlan(self, dst, src) as plan:

@@ -202,6 +202,16 @@ def rms_norm(x, w, eps, dtype, w_dtype, y=None):
     return y
 
 
+def add_rms_norm(a, b, w, eps, dtype, w_dtype):
+    """The reference's two calls behind the fused operator: c = a + b
+    (src/ops/add/cpu/add_cpu.cc:72-89), then y = RMSNorm(c) * w
+    (src/ops/rms_norm/cpu/rms_norm_cpu.cc:46-86).  a, b: contiguous [n, d]
+    storage arrays.  Returns (c, y)."""
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    c = add(a, b, a.shape, dtype)
+    return c, rms_norm(c, w, eps, dtype, w_dtype)
+
+
 def rope_check(t, pos, sin_t, cos_t, allow_bf16=False):
     return lib().oracle_rope_check(t.ref(), pos.ref(), sin_t.ref(), cos_t.ref(), int(allow_bf16))
 

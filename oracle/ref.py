@@ -40,7 +40,7 @@ def available():
 def lib():
     global _lib, _handle
     if _lib is None:
-        L = bind_prototypes(ctypes.CDLL(LIB_PATH))
+        L = bind_prototypes(ctypes.CDLL(LIB_PATH), extensions=False)
         # the reference also exports its scalar conversions as C++ symbols
         L._Z10f16_to_f32t.argtypes, L._Z10f16_to_f32t.restype = [ctypes.c_uint16], ctypes.c_float
         L._Z10f32_to_f16f.argtypes, L._Z10f32_to_f16f.restype = [ctypes.c_float], ctypes.c_uint16

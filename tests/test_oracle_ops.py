@@ -141,6 +141,29 @@ def test_rms_norm_bf16_extension_matches_float64_formula():
     assert np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-30)  # half a bf16 ulp, with slack for fp32 steps
 
 
+# ---- fused Add + RMSNorm: the reference's two calls in sequence ------------------------
+@needs_ref
+def test_add_rms_norm_is_the_reference_add_then_rms_norm():
+    rng = np.random.default_rng(17)
+    for n, d in [(16, 2048), (5, 333)]:
+        a = oracle.encode(rng.standard_normal((n, d)).astype(np.float32) * 3, "f16")
+        b = oracle.encode(rng.standard_normal((n, d)).astype(np.float32) * 3, "f16")
+        w = oracle.encode(rng.uniform(0.5, 1.5, d).astype(np.float32), "f32")
+        c, y = oracle.add_rms_norm(a, b, w, 1e-5, "f16", "f32")
+        rc = ref.add(a, b, (n, d), "f16")
+        assert np.array_equal(c, rc) and np.array_equal(y, ref.rms_norm(rc, w, 1e-5, "f16", "f32"))
+
+
+def test_add_rms_norm_normalises_the_rounded_sum():
+    """The norm is taken over the 16-bit sum, not over the exact one: a + b with
+    a = 1, b = 2^-12 rounds to 1 in fp16, so y must equal RMSNorm of a row of ones."""
+    a = oracle.encode(np.ones((1, 64), np.float32), "f16")
+    b = oracle.encode(np.full((1, 64), 2.0 ** -12, np.float32), "f16")
+    w = np.ones(64, np.float32)
+    c, y = oracle.add_rms_norm(a, b, w, 0.0, "f16", "f32")
+    assert np.all(c == a) and np.array_equal(y, oracle.rms_norm(a, w, 0.0, "f16", "f32"))
+
+
 # ---- RoPE ---------------------------------------------------------------------------
 def test_rope_golden():
     g = golden("rope")

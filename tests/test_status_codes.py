@@ -118,6 +118,48 @@ def test_library_host_validation_reproduces_reference_status(fake_handle, i):
         lib.infiniopDestroyTensorDescriptor(x)
 
 
+FUSED_CASES = [
+    # (y, c, a, b, w) as (dtype, shape, strides) -> create status; the fused Add + RMSNorm has no reference
+    # counterpart, so the expectations are RMSNorm's and Add's own rules (shape 4, strides 5, type at compute time)
+    ([("f16", (4, 64), None)] * 4 + [("f32", (64,), None)], 0),
+    ([("f16", (4, 64), (128, 1))] * 4 + [("f16", (64,), None)], 0),
+    ([("f16", (4, 64), None)] * 3 + [("f16", (4, 32), None), ("f32", (64,), None)], 4),
+    ([("f16", (4, 64), None)] * 4 + [("f32", (32,), None)], 4),
+    ([("f16", (4, 64), None)] * 2 + [("f16", (64,), None), ("f16", (4, 64), None), ("f32", (64,), None)], 4),
+    ([("f16", (4, 64), None)] * 3 + [("f16", (4, 64), (128, 2)), ("f32", (64,), None)], 5),
+    ([("f16", (4, 64), None)] * 4 + [("f32", (64,), (2,))], 5),
+]
+
+
+@pytest.mark.parametrize("i", range(len(FUSED_CASES)))
+def test_fused_add_rms_norm_host_validation(fake_handle, i):
+    tensors, want = FUSED_CASES[i]
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    descs = [oa.make_descriptor(lib, t[1], t[2], LAYOUT[t[0]]) for t in tensors]
+    d = oa.infiniopAddRMSNormDescriptor_t()
+    st = lib.infiniopCreateAddRMSNormDescriptor(handle, ctypes.byref(d), *descs, ctypes.c_float(1e-5))
+    assert st == want, (tensors, st)
+    if st == 0:
+        size = ctypes.c_uint64(7)
+        assert lib.infiniopGetAddRMSNormWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
+        assert lib.infiniopDestroyAddRMSNormDescriptor(d) == 0
+    for x in descs:
+        lib.infiniopDestroyTensorDescriptor(x)
+
+
+def test_fused_add_rms_norm_refuses_mixed_types_at_compute_time(fake_handle):
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    descs = [oa.make_descriptor(lib, (4, 64), None, oa.F16 if k != 2 else oa.F32) for k in range(4)] + [oa.make_descriptor(lib, (64,), None, oa.F32)]
+    d = oa.infiniopAddRMSNormDescriptor_t()
+    assert lib.infiniopCreateAddRMSNormDescriptor(handle, ctypes.byref(d), *descs, ctypes.c_float(1e-5)) == 0
+    assert lib.infiniopAddRMSNorm(d, None, 0, None, None, None, None, None, None) == 3  # answered before anything touches a device
+    assert lib.infiniopDestroyAddRMSNormDescriptor(d) == 0
+    for x in descs:
+        lib.infiniopDestroyTensorDescriptor(x)
+
+
 def test_descriptor_starts_with_device_number(fake_handle):
     lib = oa.open_lib()
     handle, _keep = fake_handle
