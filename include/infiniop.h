@@ -267,6 +267,59 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRearrange(
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyRearrangeDescriptor(infiniopRearrangeDescriptor_t desc);
 
 /* ======================================================================== *
+ * Matmul:  c = alpha * a @ b + beta * c; operands 2-D [rows, cols] or 3-D
+ * [batch, rows, cols] with one of the two matrix strides equal to 1 (row- or
+ * column-major), a and b with c's batch count or 1.  F16, F32 (reference) and
+ * BF16 (extension), one type for all three; accumulation in fp32.  A plain
+ * library GEMM (rocBLAS), as the reference's GPU back end uses cuBLAS.
+ * ======================================================================== */
+typedef struct MatmulDescriptor {
+    Device device;
+} MatmulDescriptor;
+typedef MatmulDescriptor *infiniopMatmulDescriptor_t;
+
+/* replaces include/ops/matmul/matmul.h:13-19 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateMatmulDescriptor(
+    infiniopHandle_t handle, infiniopMatmulDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t c_desc, float alpha,
+    infiniopTensorDescriptor_t a_desc, infiniopTensorDescriptor_t b_desc, float beta);
+/* replaces include/ops/matmul/matmul.h:21 - always 0 bytes */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetMatmulWorkspaceSize(infiniopMatmulDescriptor_t desc, uint64_t *size);
+/* replaces include/ops/matmul/matmul.h:23-29 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopMatmul(
+    infiniopMatmulDescriptor_t desc, void *workspace, uint64_t workspace_size,
+    void *c, void const *a, void const *b, void *stream);
+/* replaces include/ops/matmul/matmul.h:31 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyMatmulDescriptor(infiniopMatmulDescriptor_t desc);
+
+/* ======================================================================== *
+ * MLP:  y = alpha * SwiGLU(x @ w12) @ w3 (+ y when residual != 0), where
+ * x @ w12 is [tokens, 2*di] with the gate in columns 0..di-1 and the up
+ * projection in columns di..2*di-1.  x, y: 2-D with unit inner stride; w12
+ * [d, 2*di], w3 [di, d].  The caller provides the workspace (the [tokens,
+ * 2*di] and [tokens, di] intermediates).  A composite of Matmul and SwiGLU.
+ * ======================================================================== */
+typedef struct MLPDescriptor {
+    Device device;
+} MLPDescriptor;
+typedef MLPDescriptor *infiniopMLPDescriptor_t;
+
+/* replaces include/ops/mlp/mlp.h:15-22 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateMLPDescriptor(
+    infiniopHandle_t handle, infiniopMLPDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t y_desc, infiniopTensorDescriptor_t x_desc,
+    infiniopTensorDescriptor_t w12_desc, infiniopTensorDescriptor_t w3_desc,
+    float alpha, char residual);
+/* replaces include/ops/mlp/mlp.h:24 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetMLPWorkspaceSize(infiniopMLPDescriptor_t desc, uint64_t *size);
+/* replaces include/ops/mlp/mlp.h:26-33 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopMLP(
+    infiniopMLPDescriptor_t desc, void *workspace, uint64_t workspace_size,
+    void *y, void const *x, void const *w12, void const *w3, void *stream);
+/* replaces include/ops/mlp/mlp.h:35 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyMLPDescriptor(infiniopMLPDescriptor_t desc);
+
+/* ======================================================================== *
  * AddRMSNorm (fused residual form; no counterpart in the reference, whose
  * callers issue infiniopAdd and then infiniopRMSNorm on the sum):
  *     c[i][j] = a[i][j] + b[i][j]                       rounded as Add rounds

@@ -14,6 +14,8 @@ from .liboperators import (  # noqa: F401
     infiniopAddRMSNormDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
     infiniopHandle_t,
+    infiniopMatmulDescriptor_t,
+    infiniopMLPDescriptor_t,
     infiniopRearrangeDescriptor_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,

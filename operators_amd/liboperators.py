@@ -8,7 +8,7 @@ raises.
 """
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_float, c_int, c_int32, c_int64, c_uint64, c_void_p
+from ctypes import POINTER, Structure, c_char, c_float, c_int, c_int32, c_int64, c_uint64, c_void_p
 
 from .data_layout import DataLayout
 
@@ -69,6 +69,14 @@ class AddRMSNormDescriptor(_OpDescriptor):
     pass
 
 
+class MatmulDescriptor(_OpDescriptor):
+    pass
+
+
+class MLPDescriptor(_OpDescriptor):
+    pass
+
+
 infiniopAddDescriptor_t = POINTER(AddDescriptor)
 infiniopRMSNormDescriptor_t = POINTER(RMSNormDescriptor)
 infiniopRoPEDescriptor_t = POINTER(RoPEDescriptor)
@@ -76,6 +84,8 @@ infiniopSwiGLUDescriptor_t = POINTER(SwiGLUDescriptor)
 infiniopCausalSoftmaxDescriptor_t = POINTER(CausalSoftmaxDescriptor)
 infiniopRearrangeDescriptor_t = POINTER(RearrangeDescriptor)
 infiniopAddRMSNormDescriptor_t = POINTER(AddRMSNormDescriptor)
+infiniopMatmulDescriptor_t = POINTER(MatmulDescriptor)
+infiniopMLPDescriptor_t = POINTER(MLPDescriptor)
 
 
 class CTensor:
@@ -120,6 +130,15 @@ _PROTOTYPES = {
     "infiniopCreateRearrangeDescriptor": [infiniopHandle_t, POINTER(infiniopRearrangeDescriptor_t), infiniopTensorDescriptor_t, infiniopTensorDescriptor_t],
     "infiniopRearrange": [infiniopRearrangeDescriptor_t, c_void_p, c_void_p, c_void_p],
     "infiniopDestroyRearrangeDescriptor": [infiniopRearrangeDescriptor_t],
+    "infiniopCreateMatmulDescriptor": [infiniopHandle_t, POINTER(infiniopMatmulDescriptor_t), infiniopTensorDescriptor_t, c_float,
+                                       infiniopTensorDescriptor_t, infiniopTensorDescriptor_t, c_float],
+    "infiniopGetMatmulWorkspaceSize": [infiniopMatmulDescriptor_t, POINTER(c_uint64)],
+    "infiniopMatmul": [infiniopMatmulDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroyMatmulDescriptor": [infiniopMatmulDescriptor_t],
+    "infiniopCreateMLPDescriptor": [infiniopHandle_t, POINTER(infiniopMLPDescriptor_t)] + [infiniopTensorDescriptor_t] * 4 + [c_float, c_char],
+    "infiniopGetMLPWorkspaceSize": [infiniopMLPDescriptor_t, POINTER(c_uint64)],
+    "infiniopMLP": [infiniopMLPDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "infiniopDestroyMLPDescriptor": [infiniopMLPDescriptor_t],
     "infiniopCreateAddRMSNormDescriptor": [infiniopHandle_t, POINTER(infiniopAddRMSNormDescriptor_t)] + [infiniopTensorDescriptor_t] * 5 + [c_float],
     "infiniopGetAddRMSNormWorkspaceSize": [infiniopAddRMSNormDescriptor_t, POINTER(c_uint64)],
     "infiniopAddRMSNorm": [infiniopAddRMSNormDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],

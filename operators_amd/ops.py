@@ -17,6 +17,8 @@ from .liboperators import (
     infiniopCausalSoftmaxDescriptor_t,
     infiniopRearrangeDescriptor_t,
     infiniopAddRMSNormDescriptor_t,
+    infiniopMatmulDescriptor_t,
+    infiniopMLPDescriptor_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
     infiniopSwiGLUDescriptor_t,
@@ -133,6 +135,58 @@ class AddRMSNormPlan(_Plan):
         return y, c
 
 
+class MatmulPlan(_Plan):
+    """c = alpha * a @ b + beta * c (2-D or batched 3-D, row- or column-major operands)."""
+
+    _destroy = "infiniopDestroyMatmulDescriptor"
+
+    def __init__(self, ctx, c, a, b, alpha=1.0, beta=0.0):
+        super().__init__(ctx)
+        cts = self._describe(c, a, b)
+        desc = infiniopMatmulDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateMatmulDescriptor(ctx.handle, ctypes.byref(desc), cts[0].descriptor, alpha,
+                                                                cts[1].descriptor, cts[2].descriptor, beta))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetMatmulWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value
+
+    def __call__(self, c, a, b, stream=None):
+        check_error(self.lib.infiniopMatmul(self.desc, None, self.workspace_size, c.data_ptr(), a.data_ptr(), b.data_ptr(), stream))
+        return c
+
+
+class MLPPlan(_Plan):
+    """y = alpha * SwiGLU(x @ w12) @ w3 (+ y); owns the workspace the composite asks for."""
+
+    _destroy = "infiniopDestroyMLPDescriptor"
+
+    def __init__(self, ctx, y, x, w12, w3, alpha=1.0, residual=False):
+        import torch
+
+        super().__init__(ctx)
+        cts = self._describe(y, x, w12, w3)
+        desc = infiniopMLPDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateMLPDescriptor(ctx.handle, ctypes.byref(desc), *[ct.descriptor for ct in cts], alpha,
+                                                             ctypes.c_char(b"\x01" if residual else b"\x00")))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetMLPWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value
+        self.workspace = torch.empty(max(1, size.value), dtype=torch.uint8, device=x.device)
+
+    def __call__(self, y, x, w12, w3, stream=None):
+        check_error(self.lib.infiniopMLP(self.desc, self.workspace.data_ptr(), self.workspace_size, y.data_ptr(), x.data_ptr(),
+                                         w12.data_ptr(), w3.data_ptr(), stream))
+        return y
+
+
 class RoPEPlan(_Plan):
     _destroy = "infiniopDestroyRoPEDescriptor"
 
@@ -227,6 +281,18 @@ class Context:
     def add_rms_norm(self, y, c, a, b, w, epsilon=1e-5, stream=None):
         with AddRMSNormPlan(self, y, c, a, b, w, epsilon) as plan:
             return plan(y, c, a, b, w, stream)
+
+    def matmul(self, c, a, b, alpha=1.0, beta=0.0, stream=None):
+        with MatmulPlan(self, c, a, b, alpha, beta) as plan:
+            return plan(c, a, b, stream)
+
+    def mlp(self, y, x, w12, w3, alpha=1.0, residual=False, stream=None):
+        import torch
+
+        with MLPPlan(self, y, x, w12, w3, alpha, residual) as plan:
+            out = plan(y, x, w12, w3, stream)
+            torch.cuda.synchronize()  # the plan's workspace must outlive the work queued on it
+            return out
 
     def rearrange(self, dst, src, stream=None):
         with RearrangePlan(self, dst, src) as plan:

@@ -212,6 +212,45 @@ def add_rms_norm(a, b, w, eps, dtype, w_dtype):
     return c, rms_norm(c, w, eps, dtype, w_dtype)
 
 
+def _matrix(x):
+    """(batch, batch stride, row stride, col stride) of a 2-D or 3-D storage array, in elements."""
+    st = [s // x.itemsize for s in x.strides]
+    if x.ndim == 2:
+        return 1, 0, st[0], st[1]
+    assert x.ndim == 3
+    return x.shape[0], (0 if x.shape[0] == 1 else st[0]), st[1], st[2]
+
+
+def matmul(c, a, b, alpha, beta, dtype):
+    """In place on c: c = alpha * a @ b + beta * c (src/ops/matmul/cpu/matmul_cpu.cc:47-82).
+    2-D or batched 3-D storage arrays with any strides; a and b may have one
+    matrix for all of c's batches."""
+    cb, csb, crs, ccs = _matrix(c)
+    ab, asb, ars, acs = _matrix(a)
+    bb, bsb, brs, bcs = _matrix(b)
+    m, n, k = c.shape[-2], c.shape[-1], a.shape[-1]
+    assert a.shape[-2] == m and b.shape[-1] == n and b.shape[-2] == k and ab in (1, cb) and bb in (1, cb)
+    f = lib().oracle_matmul
+    f.argtypes = [ctypes.c_uint32] + [ctypes.c_uint64] * 4 + [ctypes.c_int64] * 9 + [ctypes.c_float] * 2 + [ctypes.c_void_p] * 3
+    st = f(DT[dtype], cb, m, n, k, csb, crs, ccs, asb if ab > 1 else 0, ars, acs, bsb if bb > 1 else 0, brs, bcs,
+           alpha, beta, _ptr(c), _ptr(a), _ptr(b))
+    if st != 0:
+        raise RuntimeError(f"oracle_matmul status {st}")
+    return c
+
+
+def mlp(y, x, w12, w3, alpha, residual, dtype):
+    """In place on y: the reference's composite (src/ops/mlp/operator.cc:22-122) -
+    gate_up = x @ w12 rounded to the storage type, hidden = swiglu(up = second
+    half, gate = first half), y = alpha * hidden @ w3 (+ y when residual)."""
+    n, two_di = x.shape[0], w12.shape[1]
+    di = two_di // 2
+    gate_up = np.zeros((n, two_di), NP_DTYPE[dtype])
+    matmul(gate_up, x, w12, 1.0, 0.0, dtype)
+    hidden = swiglu(gate_up[:, di:], gate_up[:, :di], dtype)
+    return matmul(y, hidden, w3, alpha, 1.0 if residual else 0.0, dtype)
+
+
 def rope_check(t, pos, sin_t, cos_t, allow_bf16=False):
     return lib().oracle_rope_check(t.ref(), pos.ref(), sin_t.ref(), cos_t.ref(), int(allow_bf16))
 

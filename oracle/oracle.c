@@ -29,6 +29,12 @@
  *   oracle_rearrange                         pinned  - golden vectors written by
  *       the compiled reference, the compiled reference itself, numpy's own
  *       strided assignment.  (Second operator beyond the hot path.)
+ *   oracle_matmul (fp16, fp32)               pinned  - the compiled reference
+ *       itself bit for bit (its own test shapes, row- and column-major
+ *       operands, batches, beta != 0), a float64 product, identity and
+ *       permutation matrices.  The MLP is the reference's composition of
+ *       matmul, swiglu and matmul (src/ops/mlp/operator.cc:22-122), checked
+ *       against the compiled reference's MLP bit for bit.
  *   bf16 variants of the operators           PARITY UNPINNED by the reference:
  *       no reference back end accepts bf16 for these operators.  The bf16
  *       arithmetic here is this project's extension (exact widening, the same
@@ -587,6 +593,58 @@ ORACLE_API int oracle_rearrange(uint32_t elem_size, uint64_t ndim, const uint64_
             os += (int64_t) k * src_strides[j];
         }
         memcpy((uint8_t *) dst + od * (int64_t) elem_size, (const uint8_t *) src + os * (int64_t) elem_size, row_bytes);
+    }
+    return ST_SUCCESS;
+}
+
+/* ------------------------------------------------------------------------ *
+ * Matmul (third operator beyond the four-operator path, with the MLP that is
+ * built on it)
+ * ------------------------------------------------------------------------ */
+
+/* c = alpha * a @ b + beta * c, src/ops/matmul/cpu/matmul_cpu.cc:47-82: per
+ * output element a running fp32 sum over k of widened products, in index
+ * order; then f32_to_f16(alpha * sum) when beta == 0 (c is not read), else
+ * f32_to_f16(beta * c + alpha * sum).  fp32 data: beta * c + alpha * sum
+ * always.  Each operand: `batch` matrices `*_sb` elements apart (0 when the
+ * operand has one matrix for every batch), element (i, j) at i * rs + j * cs.
+ * The reference's transposition trick (blas.h:100-106) changes the order in
+ * which outputs are visited, not what is computed for any of them. */
+ORACLE_API int oracle_matmul(uint32_t dt, uint64_t batch, uint64_t m, uint64_t n, uint64_t k,
+                             int64_t c_sb, int64_t c_rs, int64_t c_cs,
+                             int64_t a_sb, int64_t a_rs, int64_t a_cs,
+                             int64_t b_sb, int64_t b_rs, int64_t b_cs,
+                             float alpha, float beta, void *c, const void *a, const void *b) {
+    if (dt != DT_F16 && dt != DT_F32 && dt != DT_BF16) {
+        return ST_BAD_TENSOR_DTYPE;
+    }
+    for (uint64_t i = 0; i < batch; ++i) {
+        for (uint64_t r = 0; r < m; ++r) {
+            for (uint64_t q = 0; q < n; ++q) {
+                const int64_t oc = (int64_t) i * c_sb + (int64_t) r * c_rs + (int64_t) q * c_cs;
+                float sum = 0;
+                for (uint64_t t = 0; t < k; ++t) {
+                    const int64_t oa = (int64_t) i * a_sb + (int64_t) r * a_rs + (int64_t) t * a_cs;
+                    const int64_t ob = (int64_t) i * b_sb + (int64_t) t * b_rs + (int64_t) q * b_cs;
+                    if (dt == DT_F32) {
+                        sum += ((const float *) a)[oa] * ((const float *) b)[ob];
+                    } else {
+                        sum += load16(dt, (const uint16_t *) a + oa) * load16(dt, (const uint16_t *) b + ob);
+                    }
+                }
+                if (dt == DT_F32) {
+                    float *pc = (float *) c + oc;
+                    *pc = beta * (*pc) + alpha * sum;
+                } else {
+                    uint16_t *pc = (uint16_t *) c + oc;
+                    if (beta == 0) {
+                        store16(dt, pc, alpha * sum);
+                    } else {
+                        store16(dt, pc, beta * load16(dt, pc) + alpha * sum);
+                    }
+                }
+            }
+        }
     }
     return ST_SUCCESS;
 }

@@ -239,3 +239,49 @@ def rearrange(dst, src, dtype):
     lib().infiniopDestroyRearrangeDescriptor(desc)
     _free(dd, ds)
     return dst
+
+
+def matmul(c, a, b, alpha, beta, dtype):
+    """In place on c, through the reference's own CPU back end."""
+    from operators_amd.liboperators import infiniopMatmulDescriptor_t
+
+    dc, da, db = _desc_of(c, dtype), _desc_of(a, dtype), _desc_of(b, dtype)
+    desc = infiniopMatmulDescriptor_t()
+    st = lib().infiniopCreateMatmulDescriptor(handle(), ctypes.byref(desc), dc, alpha, da, db, beta)
+    assert st == 0, st
+    st = lib().infiniopMatmul(desc, None, 0, c.ctypes.data, a.ctypes.data, b.ctypes.data, None)
+    assert st == 0, st
+    lib().infiniopDestroyMatmulDescriptor(desc)
+    _free(dc, da, db)
+    return c
+
+
+def matmul_status(c, a, b):
+    """Create-time status for (dtype, shape, strides) triples."""
+    from operators_amd.liboperators import infiniopMatmulDescriptor_t
+
+    dc, da, db = (descriptor(*s) for s in (c, a, b))
+    desc = infiniopMatmulDescriptor_t()
+    st = lib().infiniopCreateMatmulDescriptor(handle(), ctypes.byref(desc), dc, 1.0, da, db, 0.0)
+    if st == 0:
+        lib().infiniopDestroyMatmulDescriptor(desc)
+    _free(dc, da, db)
+    return st
+
+
+def mlp(y, x, w12, w3, alpha, residual, dtype):
+    """In place on y, through the reference's own composite and CPU back end."""
+    from operators_amd.liboperators import infiniopMLPDescriptor_t
+
+    ds = [_desc_of(t, dtype) for t in (y, x, w12, w3)]
+    desc = infiniopMLPDescriptor_t()
+    st = lib().infiniopCreateMLPDescriptor(handle(), ctypes.byref(desc), *ds, alpha, ctypes.c_char(b"\x01" if residual else b"\x00"))
+    assert st == 0, st
+    size = ctypes.c_uint64(0)
+    assert lib().infiniopGetMLPWorkspaceSize(desc, ctypes.byref(size)) == 0
+    ws = np.zeros(max(1, size.value), np.uint8)
+    st = lib().infiniopMLP(desc, ws.ctypes.data, size.value, y.ctypes.data, x.ctypes.data, w12.ctypes.data, w3.ctypes.data, None)
+    assert st == 0, st
+    lib().infiniopDestroyMLPDescriptor(desc)
+    _free(*ds)
+    return y

@@ -1,0 +1,154 @@
+"""Matmul and the MLP composite on the GPU through the C ABI.
+
+The product is a library GEMM with fp32 accumulation and round-to-nearest
+output; the reference's CPU path accumulates in fp32 in index order and
+truncates.  Bar: the reference's own test tolerance, rtol 1e-2
+(operatorspy/tests/matmul.py:127), applied as
+    |gpu - ref| <= 1e-2 * |ref| + slack,
+where slack is what the two summation orders may differ by,
+4 * k * 2^-24 * sum|a||b|; and, tighter, both results within rounding of the
+float64 product."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import strided_like, to_codes, to_torch
+
+pytestmark = pytest.mark.gpu
+ULP = {"f16": 2.0 ** -10, "bf16": 2.0 ** -7, "f32": 2.0 ** -23}
+
+
+def as_f64(x, dt):
+    return (x if dt == "f32" else oracle.decode(x, dt)).astype(np.float64)
+
+
+def make(shape, dt, rng, positive):
+    v = rng.random(shape, dtype=np.float32) if positive else rng.standard_normal(shape).astype(np.float32)
+    return v if dt == "f32" else oracle.encode(v, dt)
+
+
+def device(x, dt, strides=None):
+    if strides is None:
+        return to_torch(x, dt)
+    return strided_like(x, x.shape, strides, dt)[0]
+
+
+def check(got, ref, exact, mag, k, dt, what):
+    g, r = as_f64(got, dt), as_f64(ref, dt)
+    order_slack = 4 * k * 2.0 ** -24 * mag
+    assert np.all(np.abs(g - r) <= 1e-2 * np.abs(r) + order_slack + 1e-30), what
+    # each within rounding (gpu: nearest, half an ulp; reference: truncation, one ulp) of the float64 product
+    assert np.all(np.abs(g - exact) <= 0.5 * ULP[dt] * np.abs(exact) + order_slack + 1e-30), what + " (gpu vs float64)"
+    assert np.all(np.abs(r - exact) <= 1.0 * ULP[dt] * np.abs(exact) + order_slack + 1e-30), what + " (oracle vs float64)"
+
+
+REFERENCE_CASES = [
+    # alpha, beta, a_shape, b_shape, c_shape, a_stride, b_stride, c_stride   (operatorspy/tests/matmul.py:297-306)
+    (1.0, 0.0, (1, 2048), (2048, 2048), (1, 2048), None, None, None),
+    (1.0, 0.0, (2, 4, 2048), (2, 2048, 2048), (2, 4, 2048), None, None, None),
+    (1.0, 0.0, (1, 2048), (2048, 2048), (1, 2048), (4096, 1), (4096, 1), (4096, 1)),
+    (1.0, 1.0, (6, 2048), (2048, 2560), (6, 2560), (2048, 1), (1, 2048), (2560, 1)),
+    (1.0 / 8.0, 0.0, (4, 8 * 6, 64), (4, 64, 6), (4, 8 * 6, 6), None, None, None),
+]
+MORE_CASES = [
+    (0.5, -1.5, (33, 100), (100, 17), (33, 17), (1, 33), (1, 100), (1, 33)),          # everything column-major
+    (1.0, 0.0, (40, 72), (72, 56), (40, 56), (1, 40), (56, 1), (56, 1)),               # a column-major, b and c row-major
+    (2.0, 1.0, (3, 16, 32), (32, 24), (3, 16, 24), None, None, None),                  # one b for every batch
+    (1.0, 0.0, (5, 8, 64), (5, 64, 8), (5, 8, 8), (1024, 64, 1), (1024, 1, 64), None), # padded batch strides
+    (1.0, 0.0, (128, 256), (256, 512), (128, 512), None, None, None),
+]
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32", "bf16"])
+@pytest.mark.parametrize("case", range(len(REFERENCE_CASES) + len(MORE_CASES)))
+def test_against_oracle(ctx, dt, case):
+    import torch
+
+    alpha, beta, a_shape, b_shape, c_shape, a_st, b_st, c_st = (REFERENCE_CASES + MORE_CASES)[case]
+    rng = np.random.default_rng(1000 + case)
+    positive = case < len(REFERENCE_CASES)  # the reference's test draws from [0, 1)
+    a, b = make(a_shape, dt, rng, positive), make(b_shape, dt, rng, positive)
+    c0 = make(c_shape, dt, rng, positive)
+    ta, tb, tc = device(a, dt, a_st), device(b, dt, b_st), device(c0, dt, c_st)
+    ctx.matmul(tc, ta, tb, alpha, beta)
+    torch.cuda.synchronize()
+    got = tc.cpu().numpy() if dt == "f32" else to_codes(tc)
+    ref = oracle.matmul(c0.copy(), a, b, alpha, beta, dt)
+    fa, fb, fc = as_f64(a, dt), as_f64(b, dt), as_f64(c0, dt)
+    exact = alpha * np.matmul(fa, fb) + beta * fc
+    mag = abs(alpha) * np.matmul(np.abs(fa), np.abs(fb)) + abs(beta) * np.abs(fc)
+    check(got, ref, exact, mag, a_shape[-1], dt, f"case {case} {dt}")
+
+
+def test_identity_and_permutation_are_exact(ctx):
+    """a @ I = a and a @ P = a with its columns permuted: no rounding anywhere."""
+    import torch
+
+    rng = np.random.default_rng(7)
+    a = oracle.encode(rng.standard_normal((48, 64)).astype(np.float32), "f16")
+    perm = rng.permutation(64)
+    p = np.zeros((64, 64), np.float32)
+    p[perm, np.arange(64)] = 1
+    for mat, want in ((np.eye(64, dtype=np.float32), a), (p, a[:, perm])):
+        tc = torch.zeros((48, 64), dtype=torch.float16, device="cuda")
+        ctx.matmul(tc, to_torch(a, "f16"), to_torch(oracle.encode(mat, "f16"), "f16"))
+        torch.cuda.synchronize()
+        assert np.array_equal(to_codes(tc), want)
+
+
+def test_status_codes(ctx):
+    import torch
+
+    from operators_amd import InfiniopError
+    from operators_amd.ops import MatmulPlan
+
+    z = lambda *s, dtype=torch.float16: torch.zeros(s, dtype=dtype, device="cuda")  # noqa: E731
+    MatmulPlan(ctx, z(4, 6), z(4, 5), z(5, 6)).close()
+    bad = [
+        ((z(4, 6), z(4, 5), z(7, 6)), 4),                      # inner extents differ (the reference ends the process here)
+        ((z(2, 2, 4, 6), z(4, 5), z(5, 6)), 4),                # rank 4
+        ((z(4, 12)[:, ::2], z(8, 5)[::2], z(5, 6)), 5),        # c with neither stride 1
+        ((z(3, 4, 6), z(2, 4, 5), z(5, 6)), 2),                # batch of a is neither c's nor 1
+        ((z(4, 6, dtype=torch.int32), z(4, 5, dtype=torch.int32), z(5, 6, dtype=torch.int32)), 3),
+    ]
+    for tensors, code in bad:
+        with pytest.raises(InfiniopError) as err:
+            MatmulPlan(ctx, *tensors)
+        assert err.value.status == code, (err.value.status, code)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("residual", [False, True])
+def test_mlp_against_oracle(ctx, dt, residual):
+    """tokens 64, d 256, di 384: the reference's composite, stage by stage."""
+    import torch
+
+    rng = np.random.default_rng(31)
+    n, d, di = 64, 256, 384
+    x = oracle.encode(rng.standard_normal((n, d)).astype(np.float32), dt)
+    w12 = oracle.encode(rng.standard_normal((d, 2 * di)).astype(np.float32) * d ** -0.5, dt)
+    w3 = oracle.encode(rng.standard_normal((di, d)).astype(np.float32) * di ** -0.5, dt)
+    y0 = oracle.encode(rng.standard_normal((n, d)).astype(np.float32), dt)
+    want = oracle.mlp(y0.copy(), x, w12, w3, 0.5, residual, dt)
+    ty = to_torch(y0, dt)
+    ctx.mlp(ty, to_torch(x, dt), to_torch(w12, dt), to_torch(w3, dt), 0.5, residual)
+    torch.cuda.synchronize()
+    g, r = as_f64(to_codes(ty), dt), as_f64(want, dt)
+    # rounding of the two intermediates differs (nearest vs truncation): a few ulps of the values that enter the second product
+    tol = 1e-2 * np.abs(r) + 8 * ULP[dt] * np.sqrt(di) * 0.5
+    assert np.all(np.abs(g - r) <= tol), float(np.max(np.abs(g - r) - tol))
+
+
+def test_mlp_workspace_contract(ctx):
+    import torch
+
+    from operators_amd.ops import MLPPlan
+
+    f16 = torch.float16
+    y, x = torch.zeros((8, 64), dtype=f16, device="cuda"), torch.zeros((8, 64), dtype=f16, device="cuda")
+    w12, w3 = torch.zeros((64, 256), dtype=f16, device="cuda"), torch.zeros((128, 64), dtype=f16, device="cuda")
+    with MLPPlan(ctx, y, x, w12, w3) as plan:
+        assert plan.workspace_size == 8 * 256 * 2 + 8 * 128 * 2
+        st = ctx.lib.infiniopMLP(plan.desc, plan.workspace.data_ptr(), plan.workspace_size - 1, y.data_ptr(), x.data_ptr(),
+                                 w12.data_ptr(), w3.data_ptr(), None)
+        assert st == 6  # a short workspace: STATUS_MEMORY_NOT_ALLOCATED, as in the reference

@@ -342,3 +342,96 @@ def test_rearrange_golden_and_numpy():
         src2, dst2, dst_buf2 = _views(g, i, dt, shape, ss, sd)
         dst2[...] = src2
         assert np.array_equal(dst_buf2.view(np.uint8), dst_buf.view(np.uint8))
+
+
+# ---- matmul and the MLP composite (third step beyond the four-operator path) ------------
+MATMUL_CASES = [
+    # alpha, beta, a, b, c shapes, a, b, c strides: the reference's own test list (operatorspy/tests/matmul.py:297-306) ...
+    (1.0, 0.0, (1, 2048), (2048, 2048), (1, 2048), None, None, None),
+    (1.0, 0.0, (2, 4, 2048), (2, 2048, 2048), (2, 4, 2048), None, None, None),
+    (1.0, 0.0, (1, 2048), (2048, 2048), (1, 2048), (4096, 1), (4096, 1), (4096, 1)),
+    (1.0, 1.0, (6, 2048), (2048, 2560), (6, 2560), (2048, 1), (1, 2048), (2560, 1)),
+    (1.0 / 8.0, 0.0, (4, 8 * 6, 64), (4, 64, 6), (4, 8 * 6, 6), None, None, None),
+    # ... and layouts it does not cover
+    (0.5, -1.5, (33, 100), (100, 17), (33, 17), (1, 33), (1, 100), (1, 33)),
+    (2.0, 1.0, (3, 16, 32), (32, 24), (3, 16, 24), None, None, None),
+]
+
+
+def _strided(x, strides):
+    if strides is None:
+        return x
+    span = 1 + sum((n - 1) * s for n, s in zip(x.shape, strides))
+    buf = np.zeros(span, x.dtype)
+    view = np.lib.stride_tricks.as_strided(buf, x.shape, [s * x.itemsize for s in strides])
+    view[...] = x
+    return view
+
+
+@needs_ref
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("case", range(len(MATMUL_CASES)))
+def test_matmul_vs_compiled_reference(dt, case):
+    alpha, beta, a_shape, b_shape, c_shape, a_st, b_st, c_st = MATMUL_CASES[case]
+    rng = np.random.default_rng(300 + case)
+    mk = (lambda s: rng.standard_normal(s).astype(np.float32)) if dt == "f32" else (lambda s: oracle.encode(rng.standard_normal(s).astype(np.float32), dt))
+    a, b, c = _strided(mk(a_shape), a_st), _strided(mk(b_shape), b_st), mk(c_shape)
+    c1, c2 = _strided(c.copy(), c_st), _strided(c.copy(), c_st)
+    oracle.matmul(c1, a, b, alpha, beta, dt)
+    ref.matmul(c2, a, b, alpha, beta, dt)
+    assert np.array_equal(c1.view(np.uint8) if c_st is None else np.ascontiguousarray(c1).view(np.uint8),
+                          c2.view(np.uint8) if c_st is None else np.ascontiguousarray(c2).view(np.uint8))
+
+
+def test_matmul_against_float64_and_exact_cases():
+    rng = np.random.default_rng(41)
+    a = oracle.encode(rng.standard_normal((20, 300)).astype(np.float32), "f16")
+    b = oracle.encode(rng.standard_normal((300, 30)).astype(np.float32), "f16")
+    c0 = oracle.encode(rng.standard_normal((20, 30)).astype(np.float32), "f16")
+    fa, fb, fc = (oracle.decode(t, "f16").astype(np.float64) for t in (a, b, c0))
+    got = oracle.decode(oracle.matmul(c0.copy(), a, b, 0.25, 2.0, "f16"), "f16").astype(np.float64)
+    exact = 0.25 * fa @ fb + 2.0 * fc
+    mag = 0.25 * np.abs(fa) @ np.abs(fb) + 2.0 * np.abs(fc)
+    assert np.all(np.abs(got - exact) <= 2.0 ** -10 * np.abs(exact) + 300 * 2.0 ** -23 * mag)
+    assert np.all(np.abs(got) <= np.abs(exact) + 300 * 2.0 ** -23 * mag)  # truncation never rounds away from zero
+    # a transposed operand (column-major b) gives the same bits as its row-major copy
+    bt = np.ascontiguousarray(b.T).T
+    assert np.array_equal(oracle.matmul(c0.copy(), a, bt, 0.25, 2.0, "f16"), oracle.matmul(c0.copy(), a, b, 0.25, 2.0, "f16"))
+    # identity and permutation matrices: exact
+    eye = oracle.encode(np.eye(300, dtype=np.float32), "f16")
+    out = oracle.matmul(np.zeros((20, 300), np.uint16), a, eye, 1.0, 0.0, "f16")
+    assert np.array_equal(out, a)
+    # beta == 0 never reads c: NaNs in c do not reach the result
+    nan_c = np.full((20, 30), 0x7E00, np.uint16)
+    assert np.array_equal(oracle.matmul(nan_c, a, b, 1.0, 0.0, "f16"), oracle.matmul(np.zeros((20, 30), np.uint16), a, b, 1.0, 0.0, "f16"))
+
+
+@needs_ref
+@pytest.mark.parametrize("residual", [False, True])
+def test_mlp_vs_compiled_reference(residual):
+    rng = np.random.default_rng(43)
+    n, d, di = 9, 64, 96
+    x = oracle.encode(rng.standard_normal((n, d)).astype(np.float32), "f16")
+    w12 = oracle.encode(rng.standard_normal((d, 2 * di)).astype(np.float32) * 0.1, "f16")
+    w3 = oracle.encode(rng.standard_normal((di, d)).astype(np.float32) * 0.1, "f16")
+    y = oracle.encode(rng.standard_normal((n, d)).astype(np.float32), "f16")
+    assert np.array_equal(oracle.mlp(y.copy(), x, w12, w3, 0.7, residual, "f16"), ref.mlp(y.copy(), x, w12, w3, 0.7, residual, "f16"))
+
+
+MATMUL_STATUS = [
+    # (c, a, b) as (dtype, shape, strides) -> create status
+    ((("f16", (4, 6), None), ("f16", (4, 5), None), ("f16", (5, 6), None)), 0),
+    ((("f32", (2, 4, 6), None), ("f32", (2, 4, 5), None), ("f32", (5, 6), None)), 0),
+    ((("f16", (2, 2, 4, 6), None), ("f16", (4, 5), None), ("f16", (5, 6), None)), 4),
+    ((("f16", (4, 6), (12, 2)), ("f16", (4, 5), None), ("f16", (5, 6), None)), 5),
+    ((("f16", (3, 4, 6), None), ("f16", (2, 4, 5), None), ("f16", (5, 6), None)), 2),
+    ((("u8", (4, 6), None), ("u8", (4, 5), None), ("u8", (5, 6), None)), 3),
+]
+
+
+@needs_ref
+@pytest.mark.parametrize("i", range(len(MATMUL_STATUS)))
+def test_matmul_status_table_is_the_reference_s(i):
+    tensors, want = MATMUL_STATUS[i]
+    assert ref.matmul_status(*tensors) == want
+

@@ -160,6 +160,57 @@ def test_fused_add_rms_norm_refuses_mixed_types_at_compute_time(fake_handle):
         lib.infiniopDestroyTensorDescriptor(x)
 
 
+MATMUL_CASES = [
+    # (c, a, b) as (dtype, shape, strides) -> create status; the table the reference's own back end is held to
+    # in test_oracle_ops.py, plus what this back end answers where the reference ends the process (mismatched extents)
+    ((("f16", (4, 6), None), ("f16", (4, 5), None), ("f16", (5, 6), None)), 0),
+    ((("f32", (2, 4, 6), None), ("f32", (2, 4, 5), None), ("f32", (5, 6), None)), 0),
+    ((("f16", (4, 6), (1, 4)), ("f16", (4, 5), (1, 4)), ("f16", (5, 6), (1, 5))), 0),
+    ((("f16", (2, 2, 4, 6), None), ("f16", (4, 5), None), ("f16", (5, 6), None)), 4),
+    ((("f16", (4, 6), (12, 2)), ("f16", (4, 5), None), ("f16", (5, 6), None)), 5),
+    ((("f16", (3, 4, 6), None), ("f16", (2, 4, 5), None), ("f16", (5, 6), None)), 2),
+    ((("u8", (4, 6), None), ("u8", (4, 5), None), ("u8", (5, 6), None)), 3),
+    ((("f16", (4, 6), None), ("f16", (4, 5), None), ("f16", (7, 6), None)), 4),
+]
+
+
+@pytest.mark.parametrize("i", range(len(MATMUL_CASES)))
+def test_matmul_host_validation(fake_handle, i):
+    tensors, want = MATMUL_CASES[i]
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    descs = [oa.make_descriptor(lib, t[1], t[2], LAYOUT[t[0]]) for t in tensors]
+    d = oa.infiniopMatmulDescriptor_t()
+    st = lib.infiniopCreateMatmulDescriptor(handle, ctypes.byref(d), descs[0], ctypes.c_float(1.0), descs[1], descs[2], ctypes.c_float(0.0))
+    assert st == want, (tensors, st)
+    if st == 0:
+        size = ctypes.c_uint64(7)
+        assert lib.infiniopGetMatmulWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
+        assert lib.infiniopDestroyMatmulDescriptor(d) == 0
+    for x in descs:
+        lib.infiniopDestroyTensorDescriptor(x)
+
+
+def test_mlp_host_validation_and_workspace_size(fake_handle):
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+    mk = lambda shape, strides=None: oa.make_descriptor(lib, shape, strides, oa.F16)  # noqa: E731
+    y, x, w12, w3 = mk((8, 64)), mk((8, 64)), mk((64, 256)), mk((128, 64))
+    d = oa.infiniopMLPDescriptor_t()
+    assert lib.infiniopCreateMLPDescriptor(handle, ctypes.byref(d), y, x, w12, w3, ctypes.c_float(1.0), ctypes.c_char(b"\x00")) == 0
+    size = ctypes.c_uint64(0)
+    assert lib.infiniopGetMLPWorkspaceSize(d, ctypes.byref(size)) == 0
+    assert size.value == 8 * 256 * 2 + 8 * 128 * 2  # the two intermediates; the reference reserves the same (mlp/operator.cc:62-65)
+    assert lib.infiniopMLP(d, None, 0, None, None, None, None, None) == 6  # short workspace
+    assert lib.infiniopDestroyMLPDescriptor(d) == 0
+    bad_x = mk((8, 64), (128, 2))
+    assert lib.infiniopCreateMLPDescriptor(handle, ctypes.byref(d), y, bad_x, w12, w3, ctypes.c_float(1.0), ctypes.c_char(b"\x00")) == 5
+    w3_bad = mk((100, 64))
+    assert lib.infiniopCreateMLPDescriptor(handle, ctypes.byref(d), y, x, w12, w3_bad, ctypes.c_float(1.0), ctypes.c_char(b"\x00")) == 4
+    for t in (y, x, w12, w3, bad_x, w3_bad):
+        lib.infiniopDestroyTensorDescriptor(t)
+
+
 def test_descriptor_starts_with_device_number(fake_handle):
     lib = oa.open_lib()
     handle, _keep = fake_handle
