@@ -35,6 +35,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+MFMA_PEAK_TFLOPS_16BIT = 2500.0  # MI355X published dense bf16 / fp16 matrix peak
 
 # HBM bytes per launch of the dominant kernel at the default workload
 # (swiglu bf16 [8192, 28672] from a fused [8192, 57344] buffer), measured with
@@ -64,8 +65,9 @@ def parse():
 class Launch:
     """One prepared stage-4 call: bound function + arguments, and its algorithmic bytes."""
 
-    def __init__(self, name, fn, args, nbytes, keep):
+    def __init__(self, name, fn, args, nbytes, keep, flops=None):
         self.name, self.fn, self.args, self.nbytes, self.keep = name, fn, args, nbytes, keep
+        self.flops = flops  # set for the GEMM-bound rows (Matmul, MLP): priced against the MFMA peak, not HBM
 
     def __call__(self, stream):
         st = self.fn(*self.args, stream)
@@ -158,6 +160,37 @@ def make_add_rms_norm(ctx, n, d, dtype, w_dtype, gen, name):
     return Launch(name, ctx.lib.infiniopAddRMSNorm, (plan.desc, None, 0, y.data_ptr(), a.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr()), nbytes, (plan, a, b, w, y))
 
 
+def make_mlp(ctx, tokens, d, di, dtype, gen, name):
+    """The reference's MLP composite: x @ w12 -> SwiGLU on the fused gate/up halves -> @ w3, added onto y."""
+    import torch
+
+    from operators_amd.ops import MLPPlan
+
+    x = _randn((tokens, d), dtype, gen)
+    y = _randn((tokens, d), dtype, gen)
+    w12 = (torch.randn((d, 2 * di), device="cuda", dtype=torch.float32, generator=gen) * d ** -0.5).to(dtype)
+    w3 = (torch.randn((di, d), device="cuda", dtype=torch.float32, generator=gen) * di ** -0.5).to(dtype)
+    plan = MLPPlan(ctx, y, x, w12, w3, 1.0, True)
+    es = x.element_size()
+    nbytes = (x.numel() + 2 * y.numel() + w12.numel() + w3.numel()) * es + 2 * (tokens * 2 * di + tokens * di) * es
+    flops = 2 * tokens * d * 2 * di + 2 * tokens * di * d
+    args = (plan.desc, plan.workspace.data_ptr(), plan.workspace_size, y.data_ptr(), x.data_ptr(), w12.data_ptr(), w3.data_ptr())
+    return Launch(name, ctx.lib.infiniopMLP, args, nbytes, (plan, x, y, w12, w3), flops)
+
+
+def make_matmul(ctx, m, k, n, dtype, gen, name):
+    import torch
+
+    from operators_amd.ops import MatmulPlan
+
+    a = _randn((m, k), dtype, gen)
+    b = (torch.randn((k, n), device="cuda", dtype=torch.float32, generator=gen) * k ** -0.5).to(dtype)
+    c = torch.empty((m, n), dtype=dtype, device="cuda")
+    plan = MatmulPlan(ctx, c, a, b)
+    nbytes = (a.numel() + b.numel() + c.numel()) * a.element_size()
+    return Launch(name, ctx.lib.infiniopMatmul, (plan.desc, None, 0, c.data_ptr(), a.data_ptr(), b.data_ptr()), nbytes, (plan, a, b, c), 2 * m * k * n)
+
+
 def make_add(ctx, n, d, dtype, broadcast, gen, name):
     import torch
 
@@ -246,10 +279,15 @@ def op_entry(name, config, sets, steps, warmup, repeats):
     per_call = runs[len(runs) // 2]
     nbytes = sets[0].nbytes
     gbps = nbytes / per_call / 1e9
-    return {"op": name, "config": config, "us_per_call": round(per_call * 1e6, 3), "us_min": round(runs[0] * 1e6, 3),
-            "us_max": round(runs[-1] * 1e6, 3), "cold_first_call_us": round(cold_us, 1), "bytes": nbytes,
-            "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4), "buffer_sets": len(sets),
-            "calls_per_run": steps, "runs": repeats, "warmup_calls": warmup}
+    row = {"op": name, "config": config, "us_per_call": round(per_call * 1e6, 3), "us_min": round(runs[0] * 1e6, 3),
+           "us_max": round(runs[-1] * 1e6, 3), "cold_first_call_us": round(cold_us, 1), "bytes": nbytes,
+           "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4), "buffer_sets": len(sets),
+           "calls_per_run": steps, "runs": repeats, "warmup_calls": warmup}
+    if sets[0].flops:
+        tflops = sets[0].flops / per_call / 1e12
+        row.update({"bound": "mfma", "flops": sets[0].flops, "tflop_per_s": round(tflops, 1),
+                    "frac_of_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS_16BIT, 4)})
+    return row
 
 
 def ops_table(ctx, args, gen):
@@ -289,6 +327,9 @@ def ops_table(ctx, args, gen):
         # beyond the four-operator path: attention scores of 32 heads, 4096 x 4096, in place
         f"N2 rearrange bf16 [{T},64,128] of [{T},80,128] -> [64,{T},128]": lambda: [make_rearrange(ctx, T, 64, bf16, gen, "rearrange") for _ in range(sets_needed(4 * T * 64 * 128, nset))],
         f"F1 add_rms_norm bf16 [{T},8192] w f32 (fused Add + RMSNorm)": lambda: [make_add_rms_norm(ctx, T, 8192, bf16, torch.float32, gen, "add_rms_norm") for _ in range(sets_needed(6 * T * 8192, nset))],
+        # GEMM-bound rows (a library GEMM; priced against the MFMA peak): the gate/up projection and the whole MLP of a Llama-70B layer
+        f"M1 matmul bf16 [{T},8192] x [8192,57344]": lambda: [make_matmul(ctx, T, 8192, 57344, bf16, gen, "matmul") for _ in range(2)],
+        f"M2 mlp bf16 tokens {T}, d 8192, di 28672 (matmul + swiglu + matmul, residual)": lambda: [make_mlp(ctx, T, 8192, 28672, bf16, gen, "mlp") for _ in range(2)],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
@@ -396,6 +437,14 @@ def cpu_per_op(T):
     d6 = np.empty((64, T, 128), np.uint16)
     run("N2 rearrange", "f16", lambda: oracle.rearrange(d6.transpose(1, 0, 2), q6[:, :64, :]), lambda: ref.rearrange(d6.transpose(1, 0, 2), q6[:, :64, :], "f16"))
     del q6, d6
+    # matmul: 4 rows of a against 896 of b's 57344 columns, scaled to the whole product (the reference's loop
+    # nest costs the same for every output element)
+    a8, b8 = codes((4, 8192), "f16"), np.zeros((8192, 57344), np.uint16)[:, :896]  # b's real row stride; only these columns are touched
+    c8 = np.zeros((4, 896), np.uint16)
+    run("M1 matmul", "f16", lambda: oracle.matmul(c8, a8, b8, 1.0, 0.0, "f16"), lambda: ref.matmul(c8, a8, b8, 1.0, 0.0, "f16"))
+    out["M1 matmul"]["cpu_us_per_call"] = round(out["M1 matmul"]["cpu_us_per_call"] * (T / 4) * 64, 1)
+    out["M1 matmul"]["cpu_sample"] = f"4 of {T} rows x 896 of 57344 columns, fp16, x{int(T / 4 * 64)}"
+    del a8, b8, c8
     # causal softmax: 2 of the 32 [4096, 4096] matrices, scaled to the whole batch (every matrix costs the same)
     y7 = codes((2, 4096, 4096), "f16")
     run("N1 causal_softmax", "f16", lambda: oracle.causal_softmax(y7, "f16"), lambda: ref.causal_softmax(y7, "f16"))
