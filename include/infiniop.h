@@ -3,8 +3,9 @@
  *
  * The library implements ONE device of the InfiniOperators operator library,
  * `DevAmdGpu` (AMD Instinct MI355X, gfx950), for the four memory-bound LLM-layer
- * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax, Rearrange and
- * a fused AddRMSNorm (the one operator here that the reference does not have).
+ * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax, Rearrange,
+ * Matmul, the MLP composite and a fused AddRMSNorm (the one operator here that
+ * the reference does not have).
  * The entry points below have the
  * names, argument order, argument meaning and status codes of the reference
  * library, so that a caller written against the reference (its ctypes harness,
@@ -16,7 +17,7 @@
  *   1. infiniopCreateHandle(&handle, DevAmdGpu, device_id)
  *   2. infiniopCreate<Op>Descriptor(handle, &desc, tensor descriptors...)
  *        all shape/stride/dtype checking happens here, once
- *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, AddRMSNorm; always 0)
+ *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, Matmul, AddRMSNorm: always 0; MLP: its two intermediates)
  *   4. infiniop<Op>(desc, ..., data pointers..., stream)
  *        enqueues on `stream` (a hipStream_t, NULL = the null stream) and
  *        returns without synchronising
