@@ -4,7 +4,7 @@
  * The library implements ONE device of the InfiniOperators operator library,
  * `DevAmdGpu` (AMD Instinct MI355X, gfx950), for the four memory-bound LLM-layer
  * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax, Rearrange,
- * Matmul, the MLP composite and a fused AddRMSNorm (the one operator here that
+ * Matmul, the MLP and Attention composites and a fused AddRMSNorm (the one operator here that
  * the reference does not have).
  * The entry points below have the
  * names, argument order, argument meaning and status codes of the reference
@@ -17,7 +17,7 @@
  *   1. infiniopCreateHandle(&handle, DevAmdGpu, device_id)
  *   2. infiniopCreate<Op>Descriptor(handle, &desc, tensor descriptors...)
  *        all shape/stride/dtype checking happens here, once
- *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, Matmul, AddRMSNorm: always 0; MLP: its two intermediates)
+ *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, Matmul, AddRMSNorm: always 0; MLP, Attention: their intermediates)
  *   4. infiniop<Op>(desc, ..., data pointers..., stream)
  *        enqueues on `stream` (a hipStream_t, NULL = the null stream) and
  *        returns without synchronising
@@ -319,6 +319,35 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopMLP(
     void *y, void const *x, void const *w12, void const *w3, void *stream);
 /* replaces include/ops/mlp/mlp.h:35 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyMLPDescriptor(infiniopMLPDescriptor_t desc);
+
+/* ======================================================================== *
+ * Attention with a KV cache: k and v are written into their caches at row
+ * `pos`, then out = softmax_causal(q @ K^T / sqrt(head_dim)) @ V over the
+ * caches up to row pos + seq.  q [n_q_head, seq, head_dim]; k, v [n_kv_head,
+ * seq, head_dim]; caches [n_kv_head, capacity, head_dim]; unit innermost
+ * strides, the others free; out [seq, n_q_head, head_dim] contiguous.  A
+ * composite of Rearrange, Matmul and CausalSoftmax; the caller provides the
+ * workspace.
+ * ======================================================================== */
+typedef struct AttentionDescriptor {
+    Device device;
+} AttentionDescriptor;
+typedef AttentionDescriptor *infiniopAttentionDescriptor_t;
+
+/* replaces include/ops/attention/attention.h:15-23 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateAttentionDescriptor(
+    infiniopHandle_t handle, infiniopAttentionDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t out_desc, infiniopTensorDescriptor_t q_desc,
+    infiniopTensorDescriptor_t k_desc, infiniopTensorDescriptor_t v_desc,
+    infiniopTensorDescriptor_t k_cache_desc, infiniopTensorDescriptor_t v_cache_desc, uint64_t pos);
+/* replaces include/ops/attention/attention.h:25 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetAttentionWorkspaceSize(infiniopAttentionDescriptor_t desc, uint64_t *size);
+/* replaces include/ops/attention/attention.h:27-36 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopAttention(
+    infiniopAttentionDescriptor_t desc, void *workspace, uint64_t workspace_size,
+    void *out, void const *q, void const *k, void const *v, void *k_cache, void *v_cache, void *stream);
+/* replaces include/ops/attention/attention.h:38 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyAttentionDescriptor(infiniopAttentionDescriptor_t desc);
 
 /* ======================================================================== *
  * AddRMSNorm (fused residual form; no counterpart in the reference, whose

@@ -12,6 +12,7 @@ from .liboperators import (  # noqa: F401
     CTensor,
     infiniopAddDescriptor_t,
     infiniopAddRMSNormDescriptor_t,
+    infiniopAttentionDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
     infiniopHandle_t,
     infiniopMatmulDescriptor_t,

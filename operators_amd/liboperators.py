@@ -77,6 +77,10 @@ class MLPDescriptor(_OpDescriptor):
     pass
 
 
+class AttentionDescriptor(_OpDescriptor):
+    pass
+
+
 infiniopAddDescriptor_t = POINTER(AddDescriptor)
 infiniopRMSNormDescriptor_t = POINTER(RMSNormDescriptor)
 infiniopRoPEDescriptor_t = POINTER(RoPEDescriptor)
@@ -86,6 +90,7 @@ infiniopRearrangeDescriptor_t = POINTER(RearrangeDescriptor)
 infiniopAddRMSNormDescriptor_t = POINTER(AddRMSNormDescriptor)
 infiniopMatmulDescriptor_t = POINTER(MatmulDescriptor)
 infiniopMLPDescriptor_t = POINTER(MLPDescriptor)
+infiniopAttentionDescriptor_t = POINTER(AttentionDescriptor)
 
 
 class CTensor:
@@ -139,6 +144,10 @@ _PROTOTYPES = {
     "infiniopGetMLPWorkspaceSize": [infiniopMLPDescriptor_t, POINTER(c_uint64)],
     "infiniopMLP": [infiniopMLPDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "infiniopDestroyMLPDescriptor": [infiniopMLPDescriptor_t],
+    "infiniopCreateAttentionDescriptor": [infiniopHandle_t, POINTER(infiniopAttentionDescriptor_t)] + [infiniopTensorDescriptor_t] * 6 + [c_uint64],
+    "infiniopGetAttentionWorkspaceSize": [infiniopAttentionDescriptor_t, POINTER(c_uint64)],
+    "infiniopAttention": [infiniopAttentionDescriptor_t, c_void_p, c_uint64] + [c_void_p] * 7,
+    "infiniopDestroyAttentionDescriptor": [infiniopAttentionDescriptor_t],
     "infiniopCreateAddRMSNormDescriptor": [infiniopHandle_t, POINTER(infiniopAddRMSNormDescriptor_t)] + [infiniopTensorDescriptor_t] * 5 + [c_float],
     "infiniopGetAddRMSNormWorkspaceSize": [infiniopAddRMSNormDescriptor_t, POINTER(c_uint64)],
     "infiniopAddRMSNorm": [infiniopAddRMSNormDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],

@@ -17,6 +17,7 @@ from .liboperators import (
     infiniopCausalSoftmaxDescriptor_t,
     infiniopRearrangeDescriptor_t,
     infiniopAddRMSNormDescriptor_t,
+    infiniopAttentionDescriptor_t,
     infiniopMatmulDescriptor_t,
     infiniopMLPDescriptor_t,
     infiniopRMSNormDescriptor_t,
@@ -187,6 +188,33 @@ class MLPPlan(_Plan):
         return y
 
 
+class AttentionPlan(_Plan):
+    """k, v -> caches at `pos`; out = softmax_causal(q K^T / sqrt(d)) V; owns the workspace."""
+
+    _destroy = "infiniopDestroyAttentionDescriptor"
+
+    def __init__(self, ctx, out, q, k, v, k_cache, v_cache, pos):
+        import torch
+
+        super().__init__(ctx)
+        cts = self._describe(out, q, k, v, k_cache, v_cache)
+        desc = infiniopAttentionDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateAttentionDescriptor(ctx.handle, ctypes.byref(desc), *[ct.descriptor for ct in cts], pos))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetAttentionWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value
+        self.workspace = torch.empty(max(1, size.value), dtype=torch.uint8, device=q.device)
+
+    def __call__(self, out, q, k, v, k_cache, v_cache, stream=None):
+        check_error(self.lib.infiniopAttention(self.desc, self.workspace.data_ptr(), self.workspace_size, out.data_ptr(), q.data_ptr(),
+                                               k.data_ptr(), v.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), stream))
+        return out
+
+
 class RoPEPlan(_Plan):
     _destroy = "infiniopDestroyRoPEDescriptor"
 
@@ -293,6 +321,14 @@ class Context:
             out = plan(y, x, w12, w3, stream)
             torch.cuda.synchronize()  # the plan's workspace must outlive the work queued on it
             return out
+
+    def attention(self, out, q, k, v, k_cache, v_cache, pos, stream=None):
+        import torch
+
+        with AttentionPlan(self, out, q, k, v, k_cache, v_cache, pos) as plan:
+            res = plan(out, q, k, v, k_cache, v_cache, stream)
+            torch.cuda.synchronize()  # the plan's workspace must outlive the work queued on it
+            return res
 
     def rearrange(self, dst, src, stream=None):
         with RearrangePlan(self, dst, src) as plan:

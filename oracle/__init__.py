@@ -251,6 +251,28 @@ def mlp(y, x, w12, w3, alpha, residual, dtype):
     return matmul(y, hidden, w3, alpha, 1.0 if residual else 0.0, dtype)
 
 
+def attention(out, q, k, v, k_cache, v_cache, pos, dtype):
+    """In place on out and on the caches: the reference's composite
+    (src/ops/attention/operator.cc:31-320) - rearrange k, v into the caches at
+    row pos; scores = q @ K^T / sqrt(head_dim) per K/V head over its group of
+    query heads, rounded to the storage type; causal softmax in place; scores
+    @ V, rounded; head-major result transposed into out [seq, heads, dim]."""
+    heads, seq, hd = q.shape
+    kv_heads, total = k.shape[0], pos + seq
+    group = heads // kv_heads
+    rearrange(k_cache[:, pos:total, :], k)
+    rearrange(v_cache[:, pos:total, :], v)
+    packed = np.zeros((heads, seq, hd), NP_DTYPE[dtype])
+    rearrange(packed, q)
+    scores = np.zeros((kv_heads, group * seq, total), NP_DTYPE[dtype])
+    matmul(scores, packed.reshape(kv_heads, group * seq, hd), k_cache[:, :total, :].transpose(0, 2, 1), 1 / np.sqrt(hd), 0.0, dtype)
+    causal_softmax(scores.reshape(heads, seq, total), dtype)
+    result = np.zeros((kv_heads, group * seq, hd), NP_DTYPE[dtype])
+    matmul(result, scores, v_cache[:, :total, :], 1.0, 0.0, dtype)
+    rearrange(out, result.reshape(heads, seq, hd).transpose(1, 0, 2))
+    return out
+
+
 def rope_check(t, pos, sin_t, cos_t, allow_bf16=False):
     return lib().oracle_rope_check(t.ref(), pos.ref(), sin_t.ref(), cos_t.ref(), int(allow_bf16))
 

@@ -285,3 +285,22 @@ def mlp(y, x, w12, w3, alpha, residual, dtype):
     lib().infiniopDestroyMLPDescriptor(desc)
     _free(*ds)
     return y
+
+
+def attention(out, q, k, v, k_cache, v_cache, pos, dtype):
+    """In place on out and the caches, through the reference's own composite and CPU back end."""
+    from operators_amd.liboperators import infiniopAttentionDescriptor_t
+
+    ds = [_desc_of(t, dtype) for t in (out, q, k, v, k_cache, v_cache)]
+    desc = infiniopAttentionDescriptor_t()
+    st = lib().infiniopCreateAttentionDescriptor(handle(), ctypes.byref(desc), *ds, pos)
+    assert st == 0, st
+    size = ctypes.c_uint64(0)
+    assert lib().infiniopGetAttentionWorkspaceSize(desc, ctypes.byref(size)) == 0
+    ws = np.zeros(max(1, size.value), np.uint8)
+    st = lib().infiniopAttention(desc, ws.ctypes.data, size.value, out.ctypes.data, q.ctypes.data, k.ctypes.data, v.ctypes.data,
+                                 k_cache.ctypes.data, v_cache.ctypes.data, None)
+    assert st == 0, st
+    lib().infiniopDestroyAttentionDescriptor(desc)
+    _free(*ds)
+    return out

@@ -435,3 +435,27 @@ def test_matmul_status_table_is_the_reference_s(i):
     tensors, want = MATMUL_STATUS[i]
     assert ref.matmul_status(*tensors) == want
 
+
+ATTENTION_CASES = [
+    # n_q_head, n_kv_head, seq, head_dim, pos, capacity, q/k/v strides, cache strides (operatorspy/tests/attention.py:310-358)
+    (32, 4, 5, 64, 0, 2048, (64, 2560, 1), (64, 11264, 1)),
+    (32, 4, 1, 64, 3, 2048, (64, 2560, 1), (64, 11264, 1)),
+    (8, 4, 2, 16, 1, 8, None, None),
+]
+
+
+@needs_ref
+@pytest.mark.parametrize("case", range(len(ATTENTION_CASES)))
+def test_attention_vs_compiled_reference(case):
+    """The oracle's composition of rearrange, matmul and causal softmax is the reference's infiniopAttention."""
+    heads, kv_heads, seq, hd, pos, cap, qkv_st, cache_st = ATTENTION_CASES[case]
+    rng = np.random.default_rng(600 + case)
+    enc = lambda s: oracle.encode(rng.standard_normal(s).astype(np.float32), "f16")  # noqa: E731
+    q, k, v = (_strided(enc(s), qkv_st) for s in ((heads, seq, hd), (kv_heads, seq, hd), (kv_heads, seq, hd)))
+    kc, vc = enc((kv_heads, cap, hd)), enc((kv_heads, cap, hd))
+    kc1, vc1, kc2, vc2 = (_strided(t.copy(), cache_st) for t in (kc, vc, kc, vc))
+    o1 = oracle.attention(np.zeros((seq, heads, hd), np.uint16), q, k, v, kc1, vc1, pos, "f16")
+    o2 = ref.attention(np.zeros((seq, heads, hd), np.uint16), q, k, v, kc2, vc2, pos, "f16")
+    assert np.array_equal(o1, o2)
+    assert np.array_equal(np.ascontiguousarray(kc1), np.ascontiguousarray(kc2)) and np.array_equal(np.ascontiguousarray(vc1), np.ascontiguousarray(vc2))
+
