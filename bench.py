@@ -178,6 +178,28 @@ def make_mlp(ctx, tokens, d, di, dtype, gen, name):
     return Launch(name, ctx.lib.infiniopMLP, args, nbytes, (plan, x, y, w12, w3), flops)
 
 
+def make_attention(ctx, heads, kv_heads, seq, hd, dtype, gen, name):
+    """Prefill attention at position 0: q, k, v are views of one fused qkv buffer [seq, heads + 2*kv_heads, hd]."""
+    import torch
+
+    from operators_amd.ops import AttentionPlan
+
+    qkv = _randn((seq, heads + 2 * kv_heads, hd), dtype, gen)
+    q = qkv[:, :heads, :].permute(1, 0, 2)
+    k = qkv[:, heads:heads + kv_heads, :].permute(1, 0, 2)
+    v = qkv[:, heads + kv_heads:, :].permute(1, 0, 2)
+    k_cache = torch.zeros((kv_heads, seq, hd), dtype=dtype, device="cuda")
+    v_cache = torch.zeros((kv_heads, seq, hd), dtype=dtype, device="cuda")
+    out = torch.empty((seq, heads, hd), dtype=dtype, device="cuda")
+    plan = AttentionPlan(ctx, out, q, k, v, k_cache, v_cache, 0)
+    es = qkv.element_size()
+    nbytes = (qkv.numel() + out.numel() + 2 * k_cache.numel()) * es  # what a fused kernel would have to move
+    flops = 2 * 2 * heads * seq * seq * hd  # both products, full (unmasked) squares as the composite computes them
+    args = (plan.desc, plan.workspace.data_ptr(), plan.workspace_size, out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            k_cache.data_ptr(), v_cache.data_ptr())
+    return Launch(name, ctx.lib.infiniopAttention, args, nbytes, (plan, qkv, k_cache, v_cache, out), flops)
+
+
 def make_matmul(ctx, m, k, n, dtype, gen, name):
     import torch
 
@@ -330,6 +352,7 @@ def ops_table(ctx, args, gen):
         # GEMM-bound rows (a library GEMM; priced against the MFMA peak): the gate/up projection and the whole MLP of a Llama-70B layer
         f"M1 matmul bf16 [{T},8192] x [8192,57344]": lambda: [make_matmul(ctx, T, 8192, 57344, bf16, gen, "matmul") for _ in range(2)],
         f"M2 mlp bf16 tokens {T}, d 8192, di 28672 (matmul + swiglu + matmul, residual)": lambda: [make_mlp(ctx, T, 8192, 28672, bf16, gen, "mlp") for _ in range(2)],
+        "A1 attention bf16 prefill: 64 q heads, 8 kv heads, seq 4096, head_dim 128 (2 rearranges + matmul + causal softmax + matmul + rearrange)": lambda: [make_attention(ctx, 64, 8, 4096, 128, bf16, gen, "attention") for _ in range(2)],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
