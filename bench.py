@@ -43,7 +43,7 @@ MFMA_PEAK_TFLOPS_16BIT = 2500.0  # MI355X published dense bf16 / fp16 matrix pea
 # counter reads for a plain 128 MiB device copy (1.99960 and 1.00000); the runs
 # are summarised in profiles/c5_kernels_hbm_traffic_pmc.txt.  Algorithmic bytes
 # for the same launch: 1 409 286 144.
-MEASURED_TRAFFIC_SWIGLU_8192 = 1409141585
+MEASURED_TRAFFIC_SWIGLU_8192 = 1409140152
 
 
 def parse():
