@@ -1,0 +1,64 @@
+"""The five launches of the prefill chain recorded into a HIP graph and
+replayed: stage 4 of every operator only enqueues kernels on the caller's
+stream (no allocation, no memset, no synchronisation), so a capture holds
+exactly those kernels.  Every replay, with eager work and synchronisations in
+between, must reproduce the eager results bit for bit."""
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_chain_replays_from_a_hip_graph(ctx):
+    import torch
+
+    from operators_amd.ops import AddPlan, RMSNormPlan, RoPEPlan, SwiGLUPlan, sin_cos_table
+
+    tokens, bf16 = 512, torch.bfloat16
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    rnd = lambda *s: torch.randn(s, device="cuda", dtype=torch.float32, generator=gen).to(bf16)  # noqa: E731
+    x, w = rnd(tokens, 8192), torch.rand(8192, device="cuda", generator=gen) + 0.5
+    qkv0 = rnd(tokens, 80, 128)
+    gate_up, a, b = rnd(tokens, 2 * 4096), rnd(tokens, 8192), rnd(tokens, 8192)
+    pos = torch.arange(tokens, device="cuda", dtype=torch.int64).view(torch.uint64)
+    sin_t, cos_t = sin_cos_table(tokens, 128, 5e5, device="cuda")
+
+    y, qkv = torch.empty_like(x), qkv0.clone()
+    h, c = torch.empty((tokens, 4096), dtype=bf16, device="cuda"), torch.empty_like(a)
+    q, k = qkv[:, :64, :], qkv[:, 64:72, :]
+    plans = [RMSNormPlan(ctx, y, x, w, 1e-5), RoPEPlan(ctx, q, pos, sin_t, cos_t), RoPEPlan(ctx, k, pos, sin_t, cos_t),
+             SwiGLUPlan(ctx, h, gate_up[:, 4096:], gate_up[:, :4096]), AddPlan(ctx, c, a, b)]
+
+    def chain(stream):
+        plans[0](y, x, w, stream)
+        plans[1](q, pos, sin_t, cos_t, stream)
+        plans[2](k, pos, sin_t, cos_t, stream)
+        plans[3](h, gate_up[:, 4096:], gate_up[:, :4096], stream)
+        plans[4](c, a, b, stream)
+
+    # eager results (RoPE works in place: start every run from the same qkv)
+    chain(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (y, qkv, h, c)]
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        qkv.copy_(qkv0)
+        with torch.cuda.graph(graph, stream=side):
+            chain(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    for replay in range(4):
+        for t in (y, h, c):
+            t.zero_()  # eager work between replays, and proof that the replay rewrites the outputs
+        qkv.copy_(qkv0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref, name in zip((y, qkv, h, c), want, ("rms_norm", "rope", "swiglu", "add")):
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), (replay, name)
+    for p in plans:
+        p.close()
