@@ -203,6 +203,86 @@ __global__ __launch_bounds__(kBlock) void rope_vec_loop(uint16_t *t, const uint6
     }
 }
 
+// One token per tile: when a token's work items fill a workgroup exactly
+// (heads / HPT * head_dim / 8 == kBlock), a lane's head group and column group
+// never change, the token is the same for the whole workgroup, and its
+// position and table rows are found with scalar loads and scalar arithmetic.
+// Nothing is predicated.  Workgroups loop over tokens with the next token's
+// loads in flight, as rope_vec_loop does.
+template<typename T, int HPT>
+struct RopeTokenTile {
+    u32x4 tv[HPT];
+    f32x4 s_lo, s_hi, c_lo, c_hi;
+    uint16_t *base;// the token's row: wavefront-uniform
+};
+
+template<typename T, int HPT, bool BUFST>
+__global__ __launch_bounds__(kBlock) void rope_token_loop(uint16_t *__restrict__ t, const uint64_t *__restrict__ pos,
+                                                          const float *__restrict__ sin_t, const float *__restrict__ cos_t,
+                                                          uint64_t tokens, uint32_t vecs_per_head, uint32_t groups, uint32_t head_dim,
+                                                          int64_t stride_token, int64_t stride_head) {
+    const uint32_t g = threadIdx.x / vecs_per_head;
+    const uint32_t cv = threadIdx.x - g * vecs_per_head;
+    int64_t lane_off[HPT];// elements from the token's row to this lane's vector of head g + i * groups
+#pragma unroll
+    for (int i = 0; i < HPT; ++i) lane_off[i] = static_cast<int64_t>(g + i * groups) * stride_head + static_cast<int64_t>(cv) * 8;
+
+    auto fetch = [&](uint64_t token, RopeTokenTile<T, HPT> &r) {
+        r.base = t + static_cast<int64_t>(token) * stride_token;
+#pragma unroll
+        for (int i = 0; i < HPT; ++i) r.tv[i] = ld16_stream(r.base + lane_off[i]);
+        const uint64_t row = pos[token] * head_dim;
+        const float *sp = sin_t + row + cv * 8, *cp = cos_t + row + cv * 8;
+        r.s_lo = ld16f(sp), r.s_hi = ld16f(sp + 4);
+        r.c_lo = ld16f(cp), r.c_hi = ld16f(cp + 4);
+    };
+    auto rotate = [&](const RopeTokenTile<T, HPT> &r) {
+        const float sn[8] = {r.s_lo.x, r.s_lo.y, r.s_lo.z, r.s_lo.w, r.s_hi.x, r.s_hi.y, r.s_hi.z, r.s_hi.w};
+        const float cs[8] = {r.c_lo.x, r.c_lo.y, r.c_lo.z, r.c_lo.w, r.c_hi.x, r.c_hi.y, r.c_hi.z, r.c_hi.w};
+        const StreamOut<true> out(r.base);
+#pragma unroll
+        for (int i = 0; i < HPT; ++i) {
+            float f[8], o[8];
+            widen8<T>(r.tv[i], f);
+#pragma unroll
+            for (int k = 0; k < 8; k += 2) {
+                const float a = f[k], b = f[k + 1];
+                const float ac = a * cs[k], bs = b * sn[k];
+                const float as = a * sn[k + 1], bc = b * cs[k + 1];
+                o[k] = ac - bs;
+                o[k + 1] = as + bc;
+            }
+            if constexpr (BUFST) {
+                out.st16(static_cast<uint32_t>(lane_off[i]) * 2, narrow8<T>(o));
+            } else {
+                st16_stream(r.base + lane_off[i], narrow8<T>(o));
+            }
+        }
+    };
+
+    uint64_t token = blockIdx.x;
+    if (token >= tokens) return;
+    const uint64_t hop = gridDim.x;
+    RopeTokenTile<T, HPT> a, b;
+    fetch(token, a);
+    while (true) {
+        if (token + hop >= tokens) {
+            rotate(a);
+            break;
+        }
+        fetch(token + hop, b);
+        rotate(a);
+        token += hop;
+        if (token + hop >= tokens) {
+            rotate(b);
+            break;
+        }
+        fetch(token + hop, a);
+        rotate(b);
+        token += hop;
+    }
+}
+
 // Any even head_dim, any strides and alignment: one lane per pair.
 template<typename T>
 __global__ __launch_bounds__(kBlock) void rope_pairs(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
@@ -249,6 +329,28 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
     // then come through scalar loads): 47.3 us for q.  With table loads and
     // arithmetic removed the looping form takes 44.7 us for q, so they cost
     // 1.7 us; an out-of-place copy of the same strided rows takes 41.9 us.
+    // A token per tile, when some number of heads per lane makes a token fill a
+    // workgroup exactly and there are tokens enough to loop over.  Measured on
+    // MI355X: q [8192,64,128] bf16 45.1 us with 2 workgroups per compute unit
+    // (46.3 with 4, 45.9 with 8) against 46.4 us for rope_vec_loop, whose lanes
+    // recompute token, head group and column for every tile; [4096,32,128]
+    // fp16 (2 heads per lane) 14.1 us either way.
+    if (sizeof(Idx) == 4 && d.tokens >= 8ull * d.cu_count) {
+        int h2 = 0;
+        for (int cand : {4, 2, 8, 1}) {
+            if (h2 == 0 && d.heads % cand == 0 && (d.heads / cand) * vph == kBlock) h2 = cand;
+        }
+        if (h2 != 0) {
+            const uint64_t cap2 = static_cast<uint64_t>(d.cu_count) * 2;
+            const unsigned g2 = static_cast<unsigned>(d.tokens < cap2 ? d.tokens : cap2);
+            const bool b2 = bufst && d.heads * static_cast<uint64_t>(d.stride_head) < (1ull << 30);
+#define ROPE_TL(HPT, B) rope_token_loop<T, HPT, B><<<g2, kBlock, 0, stream>>>(t, pos, sn, cs, d.tokens, static_cast<uint32_t>(vph), static_cast<uint32_t>(d.heads / HPT), static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
+            if (b2) { if (h2 == 4) ROPE_TL(4, true); else if (h2 == 2) ROPE_TL(2, true); else if (h2 == 8) ROPE_TL(8, true); else ROPE_TL(1, true); }
+            else { if (h2 == 4) ROPE_TL(4, false); else if (h2 == 2) ROPE_TL(2, false); else if (h2 == 8) ROPE_TL(8, false); else ROPE_TL(1, false); }
+#undef ROPE_TL
+            return;
+        }
+    }
     if (grid >= 8u * static_cast<unsigned>(d.cu_count)) {
         const uint64_t per_cu = grid >= 16u * static_cast<unsigned>(d.cu_count) ? 2 : 4;
         const uint64_t cap = static_cast<uint64_t>(d.cu_count) * per_cu;
