@@ -22,8 +22,10 @@ using namespace amd;
 // 61.4 us; 128 lanes 61.6; 256 lanes 63.1-63.7; 2 or 4 accesses per lane
 // 62.7-65.8; workgroups that loop over tiles (16-64 per compute unit)
 // 65.4-69.6.  The broadcast kernels keep 256 lanes: with an operand that is
-// re-read through the caches, [8192, 4096] fp16 plus a [4096] row takes 25.4 us
-// that way and 32.2 us with single-wavefront workgroups.
+// re-read through the caches, [8192, 4096] fp16 plus a [4096] row takes 24.4 us
+// that way and 31-32 us as a 2-D grid of single-wavefront workgroups (only 8
+// of them per row; the same workgroups numbered along one grid axis, with the
+// row found by division, take 24.1 us - not worth a second kernel shape).
 constexpr int kBlock = 256;// lanes per workgroup of the broadcast and element-wise kernels
 
 // ---- per-type arithmetic on one 128-bit word ---------------------------------
