@@ -42,10 +42,10 @@ template<> struct Unit<1> { typedef uint8_t type; };
 // since the row number is uniform.
 // BUFST (16-byte units, large outputs): stores are written through L2 as
 // buffer stores relative to the start of the destination row (see StreamOut).
-template<int BYTES, bool BUFST>
-__global__ __launch_bounds__(Lanes<BYTES>::value) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row) {
+template<int BYTES, bool BUFST, int LANES>
+__global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row) {
     typedef typename Unit<BYTES>::type U;
-    const uint32_t col = blockIdx.x * Lanes<BYTES>::value + threadIdx.x;
+    const uint32_t col = blockIdx.x * LANES + threadIdx.x;
     if (col >= units_per_row) return;
     for (uint64_t r = blockIdx.y; r < rows; r += gridDim.y) {
         int64_t od = 0, os = 0;
@@ -116,11 +116,20 @@ bool launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         dst_span += (d.shape[k] - 1) * static_cast<uint64_t>(d.dst_stride[k] >= 0 ? d.dst_stride[k] : 0);
     }
     if (upr >= kWave && upr < (1ull << 31)) {
-        const dim3 grid(static_cast<unsigned>(ceil_div(upr, kBlock)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
-        if (BYTES == 16 && large && desc.row_bytes < (1ull << 32)) {
-            rearrange_rows<BYTES, BYTES == 16><<<grid, kBlock, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+        // A 2-D grid of single-wavefront workgroups needs at least 16 of them per
+        // row.  Measured on MI355X with 128 MiB of fp16 rows: 16 KiB rows 41.3 us
+        // with 64 lanes and 42.1 us with 256; 8 KiB rows (8 wavefronts each) 57.5
+        // against 42.1 us, 2 KiB rows 61.0 against 46.3 us.
+        const bool wave_rows = kBlock == kWave && upr >= 16 * kWave;
+        const int lanes = wave_rows ? kWave : 256;
+        const dim3 grid(static_cast<unsigned>(ceil_div(upr, lanes)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
+        const bool bufst = BYTES == 16 && large && desc.row_bytes < (1ull << 32);
+        if (wave_rows) {
+            if (bufst) rearrange_rows<BYTES, BYTES == 16, kWave><<<grid, kWave, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+            else rearrange_rows<BYTES, false, kWave><<<grid, kWave, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
         } else {
-            rearrange_rows<BYTES, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+            if (bufst) rearrange_rows<BYTES, BYTES == 16, 256><<<grid, 256, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+            else rearrange_rows<BYTES, false, 256><<<grid, 256, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
         }
     } else {// short rows, or a single row too long for 32-bit column numbers
         const uint64_t total = desc.rows * upr;
