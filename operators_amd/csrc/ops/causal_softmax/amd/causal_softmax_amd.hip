@@ -226,7 +226,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
     // Rows of up to 4096 elements are taken by single wavefronts (no barrier, no
-    // LDS), longer ones by 256-1024 lanes (8 workgroups per compute unit).
+    // LDS), longer ones by 256-1024 lanes.
     // Measured on MI355X at [32, 4096, 4096] fp16: one row per wavefront is
     // 6-13 % faster than 128, 256 or 512 lanes per row.  The grid of the
     // single-wavefront form is several times what the chip holds at once
@@ -234,7 +234,16 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     // triangular load while each workgroup still prefetches across its few
     // rows: 32 workgroups per unit 314 us, 64 288, 96 281, 128 277, 256 278,
     // one workgroup per row 293.
-    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * (nvec <= 512 ? 128 : 8);
+    // Both forms get a grid several times what is resident.  Short rows: 128
+    // workgroups per unit at 4096 elements, 512 for 2048 and shorter
+    // ([128, 2048, 2048]: 274 us with 512, 302 with 128).  Long rows: 64 per
+    // unit ([8, 8192, 8192]: 272 us against 300 with 8; [2, 16384, 16384]: 268
+    // against 289).
+    uint64_t per_cu = 64;
+    if (nvec <= 512) {
+        per_cu = nvec > 256 ? 128 : 512;
+    }
+    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * per_cu;
     const unsigned grid = static_cast<unsigned>(rows < cap ? rows : cap);
 
     const bool vec_ok = d.total % 8 == 0 && nvec <= 4096 && d.seq < (1ull << 31) && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);

@@ -337,7 +337,7 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
     // fp16 (2 heads per lane) 14.1 us either way.
     if (sizeof(Idx) == 4 && d.tokens >= 8ull * d.cu_count) {
         int h2 = 0;
-        for (int cand : {4, 2, 8, 1}) {
+        for (int cand : {4, 2, 8}) {// not 1: a lane that rotates one head loads four table vectors for it ([32768,32,64]: 62 us against 47)
             if (h2 == 0 && d.heads % cand == 0 && (d.heads / cand) * vph == kBlock) h2 = cand;
         }
         if (h2 != 0) {
@@ -345,8 +345,8 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
             const unsigned g2 = static_cast<unsigned>(d.tokens < cap2 ? d.tokens : cap2);
             const bool b2 = bufst && d.heads * static_cast<uint64_t>(d.stride_head) < (1ull << 30);
 #define ROPE_TL(HPT, B) rope_token_loop<T, HPT, B><<<g2, kBlock, 0, stream>>>(t, pos, sn, cs, d.tokens, static_cast<uint32_t>(vph), static_cast<uint32_t>(d.heads / HPT), static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
-            if (b2) { if (h2 == 4) ROPE_TL(4, true); else if (h2 == 2) ROPE_TL(2, true); else if (h2 == 8) ROPE_TL(8, true); else ROPE_TL(1, true); }
-            else { if (h2 == 4) ROPE_TL(4, false); else if (h2 == 2) ROPE_TL(2, false); else if (h2 == 8) ROPE_TL(8, false); else ROPE_TL(1, false); }
+            if (b2) { if (h2 == 4) ROPE_TL(4, true); else if (h2 == 2) ROPE_TL(2, true); else ROPE_TL(8, true); }
+            else { if (h2 == 4) ROPE_TL(4, false); else if (h2 == 2) ROPE_TL(2, false); else ROPE_TL(8, false); }
 #undef ROPE_TL
             return;
         }
