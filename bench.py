@@ -26,6 +26,7 @@ sets; `us_per_call` is the median run, `us_min`/`us_max` the fastest and
 slowest.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -130,6 +131,20 @@ def make_causal_softmax(ctx, heads, seq, total, dtype, gen, name):
     kept = seq * (total - seq) + seq * (seq + 1) // 2  # elements read per matrix; every element is written
     nbytes = heads * (kept + seq * total) * y.element_size()
     return Launch(name, ctx.lib.infiniopCausalSoftmax, (plan.desc, None, 0, y.data_ptr()), nbytes, (plan, y))
+
+
+def make_random_sample(ctx, voc, topk, gen, name):
+    """One draw from `voc` fp16 logits ~ N(0, 3): top-p 0.9, top-k `topk`, temperature 0.8 (greedy when topk is 1)."""
+    import torch
+
+    from operators_amd.ops import RandomSamplePlan
+
+    logits = (_randn((voc,), torch.float32, gen) * 3).to(torch.float16)
+    result = torch.zeros(1, dtype=torch.int64, device="cuda").view(torch.uint64)
+    plan = RandomSamplePlan(ctx, result, logits)
+    f = ctypes.c_float
+    args = (plan.desc, None, 0, result.data_ptr(), logits.data_ptr(), f(0.37), f(0.9 if topk > 1 else 0.0), topk, f(0.8))
+    return Launch(name, ctx.lib.infiniopRandomSample, args, voc * 2 + 8, (plan, logits, result))
 
 
 def make_rearrange(ctx, tokens, heads, dtype, gen, name):
@@ -353,6 +368,10 @@ def ops_table(ctx, args, gen):
         f"M1 matmul bf16 [{T},8192] x [8192,57344]": lambda: [make_matmul(ctx, T, 8192, 57344, bf16, gen, "matmul") for _ in range(2)],
         f"M2 mlp bf16 tokens {T}, d 8192, di 28672 (matmul + swiglu + matmul, residual)": lambda: [make_mlp(ctx, T, 8192, 28672, bf16, gen, "mlp") for _ in range(2)],
         "A1 attention bf16 prefill: 64 q heads, 8 kv heads, seq 4096, head_dim 128 (2 rearranges + matmul + causal softmax + matmul + rearrange)": lambda: [make_attention(ctx, 64, 8, 4096, 128, bf16, gen, "attention") for _ in range(2)],
+        # sampling: one workgroup, latency-bound (64-300 KB of logits); the bandwidth columns say nothing here
+        "S1 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample") for _ in range(MAX_SETS)],
+        "S2 random_sample f16 voc 32000, greedy": lambda: [make_random_sample(ctx, 32000, 1, gen, "random_sample") for _ in range(MAX_SETS)],
+        "S3 random_sample f16 voc 151936, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 50, gen, "random_sample") for _ in range(MAX_SETS)],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
@@ -473,6 +492,11 @@ def cpu_per_op(T):
     run("N1 causal_softmax", "f16", lambda: oracle.causal_softmax(y7, "f16"), lambda: ref.causal_softmax(y7, "f16"))
     out["N1 causal_softmax"]["cpu_us_per_call"] = round(out["N1 causal_softmax"]["cpu_us_per_call"] * 16, 1)
     out["N1 causal_softmax"]["cpu_sample"] = "2 of 32 matrices, x16"
+    del y7
+    l9 = (rng.standard_normal(151936, dtype=np.float32) * 3).astype(np.float16).view(np.uint16)
+    run("S1 random_sample", "f16", lambda: oracle.random_sample(l9[:32000], 0.37, 0.9, 50, 0.8), lambda: ref.random_sample(l9[:32000], 0.37, 0.9, 50, 0.8))
+    run("S2 random_sample", "f16", lambda: oracle.random_sample(l9[:32000], 0.37, 0.0, 1, 0.8), lambda: ref.random_sample(l9[:32000], 0.37, 0.0, 1, 0.8))
+    run("S3 random_sample", "f16", lambda: oracle.random_sample(l9, 0.37, 0.9, 50, 0.8), lambda: ref.random_sample(l9, 0.37, 0.9, 50, 0.8))
     return out
 
 

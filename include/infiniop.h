@@ -4,7 +4,7 @@
  * The library implements ONE device of the InfiniOperators operator library,
  * `DevAmdGpu` (AMD Instinct MI355X, gfx950), for the four memory-bound LLM-layer
  * operators Add, RMSNorm, RoPE and SwiGLU, plus CausalSoftmax, Rearrange,
- * Matmul, the MLP and Attention composites and a fused AddRMSNorm (the one operator here that
+ * Matmul, RandomSample, the MLP and Attention composites and a fused AddRMSNorm (the one operator here that
  * the reference does not have).
  * The entry points below have the
  * names, argument order, argument meaning and status codes of the reference
@@ -17,7 +17,7 @@
  *   1. infiniopCreateHandle(&handle, DevAmdGpu, device_id)
  *   2. infiniopCreate<Op>Descriptor(handle, &desc, tensor descriptors...)
  *        all shape/stride/dtype checking happens here, once
- *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, Matmul, AddRMSNorm: always 0; MLP, Attention: their intermediates)
+ *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, Matmul, RandomSample, AddRMSNorm: always 0; MLP, Attention: their intermediates)
  *   4. infiniop<Op>(desc, ..., data pointers..., stream)
  *        enqueues on `stream` (a hipStream_t, NULL = the null stream) and
  *        returns without synchronising
@@ -348,6 +348,35 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopAttention(
     void *out, void const *q, void const *k, void const *v, void *k_cache, void *v_cache, void *stream);
 /* replaces include/ops/attention/attention.h:38 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyAttentionDescriptor(infiniopAttentionDescriptor_t desc);
+
+/* ======================================================================== *
+ * RandomSample: one token index drawn from a vector of fp16 logits.  With
+ * topp > 0 and topk > 1: the topk largest logits in descending order, their
+ * probabilities f16(expf((x - max) / temperature) / sum over all logits), the
+ * shortest prefix whose running sum reaches topp (plus one entry), and the
+ * first entry of it whose running sum exceeds random_val times the prefix sum.
+ * Otherwise: the first index of the maximum.  probs: 1-D F16, unit stride;
+ * result: U64, one element written.  Equal logits are ordered by ascending
+ * index.  topk (after clamping to the vocabulary size) may be at most 1024 in
+ * the sampling form, else STATUS_BAD_PARAM.  Needs no workspace.
+ * ======================================================================== */
+typedef struct RandomSampleDescriptor {
+    Device device;
+} RandomSampleDescriptor;
+typedef RandomSampleDescriptor *infiniopRandomSampleDescriptor_t;
+
+/* replaces include/ops/random_sample/random_sample.h:14 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateRandomSampleDescriptor(
+    infiniopHandle_t handle, infiniopRandomSampleDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t result, infiniopTensorDescriptor_t probs);
+/* replaces include/ops/random_sample/random_sample.h:16 - always 0 bytes */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetRandomSampleWorkspaceSize(infiniopRandomSampleDescriptor_t desc, uint64_t *size);
+/* replaces include/ops/random_sample/random_sample.h:18-27 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRandomSample(
+    infiniopRandomSampleDescriptor_t desc, void *workspace, uint64_t workspace_size,
+    void *result, void const *probs, float random_val, float topp, int topk, float temperature, void *stream);
+/* replaces include/ops/random_sample/random_sample.h:29 */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyRandomSampleDescriptor(infiniopRandomSampleDescriptor_t desc);
 
 /* ======================================================================== *
  * AddRMSNorm (fused residual form; no counterpart in the reference, whose

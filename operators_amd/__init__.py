@@ -19,6 +19,7 @@ from .liboperators import (  # noqa: F401
     infiniopMLPDescriptor_t,
     infiniopRearrangeDescriptor_t,
     infiniopRMSNormDescriptor_t,
+    infiniopRandomSampleDescriptor_t,
     infiniopRoPEDescriptor_t,
     infiniopSwiGLUDescriptor_t,
     infiniopTensorDescriptor_t,

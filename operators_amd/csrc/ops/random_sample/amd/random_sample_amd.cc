@@ -1,0 +1,58 @@
+// Create-time validation for RandomSample on the amd-gpu device.  Checks,
+// their order and their status codes are the reference's
+// (src/ops/random_sample/cpu/random_sample.cc:7-33): logits of rank 1, F16;
+// result U64; a result that is neither of rank 1 nor has a first extent of 1
+// is refused.  A result without dimensions (whose first extent the reference
+// reads anyway) is taken as a scalar.  Additions: a unit stride on the logits
+// (the reference reads them as dense without looking), at least one logit,
+// and fewer than 2^31 of them (the reference keeps the count in an int).
+#include "random_sample_amd.h"
+#include <new>
+
+infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampleAmdDescriptor_t *desc_ptr,
+                                                 infiniopTensorDescriptor_t result, infiniopTensorDescriptor_t probs) {
+    if (desc_ptr == nullptr) {
+        return STATUS_MEMORY_NOT_ALLOCATED;
+    }
+    if (probs->ndim != 1) {
+        return STATUS_BAD_TENSOR_SHAPE;
+    }
+    if (amd::elem_of(probs->dt) != amd::Elem::F16) {
+        return STATUS_BAD_TENSOR_DTYPE;
+    }
+    if (!amd::same_dt(result->dt, U64)) {
+        return STATUS_BAD_TENSOR_DTYPE;
+    }
+    if (result->ndim != 1 && result->ndim != 0 && result->shape[0] != 1) {
+        return STATUS_BAD_TENSOR_SHAPE;
+    }
+    if (probs->shape[0] == 0 || probs->shape[0] >= (1ull << 31)) {
+        return STATUS_BAD_TENSOR_SHAPE;
+    }
+    if (probs->shape[0] > 1 && probs->strides[0] != 1) {
+        return STATUS_BAD_TENSOR_STRIDES;
+    }
+    auto *desc = new (std::nothrow) RandomSampleAmdDescriptor{DevAmdGpu, handle->device_id,
+                                                              static_cast<uint32_t>(probs->shape[0])};
+    if (desc == nullptr) {
+        return STATUS_MEMORY_NOT_ALLOCATED;
+    }
+    *desc_ptr = desc;
+    return STATUS_SUCCESS;
+}
+
+// The reference's back ends sort in a workspace of voc * 12 (CPU) or voc * 20
+// bytes plus what their sorting library allocates per call (CUDA).  The
+// kernels here select in registers and LDS and need none.
+infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t, uint64_t *size) {
+    if (size == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    *size = 0;
+    return STATUS_SUCCESS;
+}
+
+infiniopStatus_t amdDestroyRandomSampleDescriptor(RandomSampleAmdDescriptor_t desc) {
+    delete desc;
+    return STATUS_SUCCESS;
+}

@@ -1,0 +1,340 @@
+// RandomSample on gfx950: one workgroup of 1024 lanes does the whole call in
+// one launch, in registers and LDS, without a workspace.
+//
+// The reference's CPU path (src/ops/random_sample/cpu/random_sample.cc:47-171)
+// sorts the topk largest logits to the front with a selection sort, turns the
+// logits into fp16 probabilities, keeps the sorted prefix whose running sum
+// reaches topp and draws from it with random_val.  What is reproduced here is
+// that arithmetic - fp32 (x - max) / temperature, expf, division by the sum,
+// truncation to fp16, the three running fp32 sums in sorted order, every
+// comparison - not the sort: 64 KiB of logits is no work for a sort, it is a
+// latency chain, so the topk-th largest code is found by a radix select over
+// the 16-bit codes (four passes of 4 bits, per-lane counters, no atomics), the
+// at most topk candidates are compacted into LDS in index order and ranked
+// there.
+//
+// Two things differ from the CPU path and are visible to a caller:
+//  * equal logits: the CPU's selection sort leaves equal values in an order
+//    that depends on its swap history; here they are ordered by ascending
+//    index.  The logit at the returned index is the same either way, which is
+//    what the reference's own test accepts (operatorspy/tests/random_sample.py:
+//    `indices == ans or data[indices] == data[ans]`);
+//  * the softmax denominator is summed as a tree, not left to right, so a
+//    probability can differ in its last fp16 bit in rare cases.
+// NaN logits: the greedy form treats them as the CPU does (never greater than
+// anything; one in front wins); the sampling form ranks them below -Inf.
+#include "../../../devices/amd/kernel_amd.h"
+#include "random_sample_amd.h"
+
+namespace {
+
+using namespace amd;
+
+constexpr int BS = 1024;
+constexpr int WAVES = BS / kWave;
+constexpr int KMAX = kRandomSampleMaxTopk;
+constexpr uint32_t kNoKey = 0xFFFFFFFFu;// marks a slot past the end of the logits
+
+// Order-preserving 16-bit key of an fp16 code: a greater value has a greater
+// key, -0 and +0 share one, NaN is the smallest.
+__device__ __forceinline__ uint32_t key_of(uint32_t h) {
+    if ((h & 0x7FFFu) > 0x7C00u) return 0u;
+    if (h == 0x8000u) h = 0u;
+    return (h & 0x8000u) ? (h ^ 0xFFFFu) : (h | 0x8000u);
+}
+__device__ __forceinline__ float value_of_key(uint32_t k) {
+    const uint32_t h = (k & 0x8000u) ? (k & 0x7FFFu) : (k ^ 0xFFFFu);
+    return F16Ref::one(static_cast<uint16_t>(h));
+}
+
+// The eight codes starting at element `base` (a multiple of 8): one 128-bit
+// load when they all exist and the array is 16-byte aligned, element loads
+// otherwise; slots past the end read as 0 and are flagged in `n`.
+template<bool VEC>
+__device__ __forceinline__ int load_codes(const uint16_t *p, uint32_t voc, uint32_t base, uint32_t (&h)[8]) {
+    if (base >= voc) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) h[e] = 0;
+        return 0;
+    }
+    if (VEC && base + 8 <= voc) {
+        const u32x4 v = ld16(p + base);
+        h[0] = v.x & 0xFFFFu, h[1] = v.x >> 16, h[2] = v.y & 0xFFFFu, h[3] = v.y >> 16;
+        h[4] = v.z & 0xFFFFu, h[5] = v.z >> 16, h[6] = v.w & 0xFFFFu, h[7] = v.w >> 16;
+        return 8;
+    }
+    const int n = voc - base < 8u ? static_cast<int>(voc - base) : 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = e < n ? p[base + e] : 0u;
+    return n;
+}
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(v, o);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+// Inclusive prefix sum over the lanes of a wavefront.
+__device__ __forceinline__ uint32_t wave_scan_u32(uint32_t v, int lane) {
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const uint32_t below = __shfl_up(v, o);
+        if (lane >= o) v += below;
+    }
+    return v;
+}
+
+// Greedy form (random_sample.cc:127-148): the first index holding the maximum,
+// where NaN is never greater than anything and a NaN in front is never beaten.
+template<bool VEC>
+__global__ __launch_bounds__(BS) void random_sample_greedy(uint64_t *result, const uint16_t *probs, uint32_t voc) {
+    __shared__ unsigned long long best_of[WAVES];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    unsigned long long best = 0;
+    for (uint32_t base = tid * 8u; base < voc; base += BS * 8u) {
+        uint32_t h[8];
+        const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < n) {
+                // greater key first, then the lower index
+                const unsigned long long c = (static_cast<unsigned long long>(key_of(h[e])) << 32) | (0xFFFFFFFFu - (base + e));
+                best = c > best ? c : best;
+            }
+        }
+    }
+    best = wave_max_u64(best);
+    if (lane == 0) best_of[wave] = best;
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) best = best_of[w] > best ? best_of[w] : best;
+        const uint32_t first = probs[0];
+        const bool first_is_nan = (first & 0x7FFFu) > 0x7C00u;
+        result[0] = first_is_nan ? 0ull : static_cast<unsigned long long>(0xFFFFFFFFu - static_cast<uint32_t>(best));
+    }
+}
+
+// Sampling form (random_sample.cc:47-126).  topk is already clamped to
+// [2, min(voc, KMAX)].
+template<bool VEC>
+__global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const uint16_t *probs, uint32_t voc,
+                                                          float random_val, float topp, uint32_t topk, float temperature) {
+    __shared__ uint32_t wave_cnt[WAVES * 16];        // per-wavefront digit counts of one select pass
+    __shared__ uint32_t digit_cnt[16];               // their totals
+    __shared__ uint32_t wave_key[WAVES];             // per-wavefront maximum key
+    __shared__ uint32_t scan_tot[2][WAVES][2];       // per-wavefront (greater, equal) counts of one compaction step
+    __shared__ float sum_slots[WAVES];
+    __shared__ unsigned long long cand[KMAX];        // key << 32 | ~index, in index order
+    __shared__ float sorted_p[KMAX];                 // probabilities, widened, in descending order of logit
+    __shared__ uint32_t sorted_i[KMAX];              // their indices
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t step = BS * 8u;
+
+    // ---- radix select: the key of the topk-th largest logit ----------------
+    uint32_t prefix = 0;   // the digits chosen so far
+    uint32_t want = topk;  // rank looked for among the elements that share them
+    uint32_t key_max = 0;
+#pragma unroll 1
+    for (int shift = 12; shift >= 0; shift -= 4) {
+        uint32_t cnt[16];
+#pragma unroll
+        for (int d = 0; d < 16; ++d) cnt[d] = 0;
+        for (uint32_t base = tid * 8u; base < voc; base += step) {
+            uint32_t h[8];
+            const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t k = e < n ? key_of(h[e]) : kNoKey;
+                if (shift == 12 && e < n) key_max = k > key_max ? k : key_max;
+                const bool in = (k >> (shift + 4)) == prefix;// never true for kNoKey: prefix < 2^12
+                const uint32_t digit = (k >> shift) & 15u;
+#pragma unroll
+                for (int d = 0; d < 16; ++d) cnt[d] += (in && digit == static_cast<uint32_t>(d)) ? 1u : 0u;
+            }
+        }
+        uint32_t mine = 0;
+#pragma unroll
+        for (int d = 0; d < 16; ++d) {
+            const uint32_t t = wave_sum_u32(cnt[d]);
+            if (lane == d) mine = t;
+        }
+        if (lane < 16) wave_cnt[wave * 16 + lane] = mine;
+        if (shift == 12) {
+            uint32_t m = key_max;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const uint32_t other = __shfl_xor(m, o);
+                m = other > m ? other : m;
+            }
+            if (lane == 0) wave_key[wave] = m;
+        }
+        __syncthreads();
+        if (tid < 16) {
+            uint32_t t = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) t += wave_cnt[w * 16 + tid];
+            digit_cnt[tid] = t;
+        }
+        __syncthreads();
+        uint32_t above = 0, chosen = 0;
+        bool found = false;
+#pragma unroll
+        for (int d = 15; d >= 0; --d) {
+            const uint32_t c = digit_cnt[d];
+            if (!found) {
+                if (above + c >= want) {
+                    chosen = d;
+                    found = true;
+                } else {
+                    above += c;
+                }
+            }
+        }
+        want -= above;
+        prefix = (prefix << 4) | chosen;
+    }
+    const uint32_t key_k = prefix;          // key of the topk-th largest
+    const uint32_t need_eq = want;          // how many of its equals belong to the topk
+    const uint32_t n_greater = topk - want; // elements with a greater key
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) key_max = wave_key[w] > key_max ? wave_key[w] : key_max;
+    const float top = value_of_key(key_max);
+
+    // ---- compaction in index order, and the softmax denominator ------------
+    float part = 0.0f;
+    uint32_t run_gt = 0, run_eq = 0;
+    int buf = 0;
+    const uint32_t rounds = (voc + step - 1) / step;
+#pragma unroll 1
+    for (uint32_t r = 0; r < rounds; ++r, buf ^= 1) {
+        const uint32_t base = r * step + tid * 8u;
+        uint32_t h[8], k[8];
+        const int n = load_codes<VEC>(probs, voc, base, h);
+        uint32_t c_gt = 0, c_eq = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            k[e] = e < n ? key_of(h[e]) : kNoKey;
+            if (e < n) {
+                part += expf((F16Ref::one(static_cast<uint16_t>(h[e])) - top) / temperature);
+                c_gt += k[e] > key_k ? 1u : 0u;
+                c_eq += k[e] == key_k ? 1u : 0u;
+            }
+        }
+        const uint32_t inc_gt = wave_scan_u32(c_gt, lane), inc_eq = wave_scan_u32(c_eq, lane);
+        if (lane == kWave - 1) {
+            scan_tot[buf][wave][0] = inc_gt;
+            scan_tot[buf][wave][1] = inc_eq;
+        }
+        __syncthreads();
+        uint32_t at_gt = run_gt + inc_gt - c_gt, at_eq = run_eq + inc_eq - c_eq;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const uint32_t g = scan_tot[buf][w][0], q = scan_tot[buf][w][1];
+            if (w < wave) at_gt += g, at_eq += q;
+            run_gt += g, run_eq += q;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < n) {
+                const unsigned long long c = (static_cast<unsigned long long>(k[e]) << 32) | (0xFFFFFFFFu - (base + e));
+                if (k[e] > key_k) {
+                    cand[at_gt++] = c;
+                } else if (k[e] == key_k) {
+                    if (at_eq < need_eq) cand[n_greater + at_eq] = c;
+                    ++at_eq;
+                }
+            }
+        }
+    }
+    part = wave_sum(part);
+    if (lane == 0) sum_slots[wave] = part;
+    __syncthreads();// candidates and partial sums are in LDS
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) total += sum_slots[w];
+
+    // ---- rank the candidates: greater logit first, then the lower index ----
+    if (static_cast<uint32_t>(tid) < topk) {
+        const unsigned long long mine = cand[tid];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < topk; ++j) rank += cand[j] > mine ? 1u : 0u;
+        const float x = value_of_key(static_cast<uint32_t>(mine >> 32));
+        const float p = expf((x - top) / temperature) / total;
+        sorted_p[rank] = F16Ref::one(F16Ref::narrow1(p));
+        sorted_i[rank] = 0xFFFFFFFFu - static_cast<uint32_t>(mine);
+    }
+    __syncthreads();
+
+    // ---- the running sums of random_sample.cc:97-125, in their order -------
+    if (tid == 0) {
+        float run = 0.0f;
+        uint32_t end;
+        for (end = 0; end < topk; ++end) {
+            run += sorted_p[end];
+            if (run >= topp) break;
+        }
+        // `run` is now the sum of the kept prefix in every case: the loop stops
+        // on the last kept entry or runs through all topk of them
+        end = end + 1 < topk ? end + 1 : topk;
+        const float limit = random_val * run;
+        float acc = 0.0f;
+        for (uint32_t i = 0; i < end; ++i) {
+            acc += sorted_p[i];
+            if (limit < acc) {
+                result[0] = sorted_i[i];
+                break;
+            }
+        }
+    }
+}
+
+}// namespace
+
+// Stage 4 of RandomSample.  The workspace is unused (its size is 0).  With
+// topp > 0 and topk > 1 it samples, otherwise it returns the first index of
+// the maximum, as the reference does (random_sample.cc:160-166).
+infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *, uint64_t, void *result, void const *probs,
+                                 float random_val, float topp, int topk, float temperature, void *stream) {
+    if (result == nullptr || probs == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    const bool sample = topp > 0 && topk > 1;
+    uint32_t k = 0;
+    if (sample) {
+        k = static_cast<uint32_t>(topk) > desc->voc ? desc->voc : static_cast<uint32_t>(topk);
+        if (k > static_cast<uint32_t>(kRandomSampleMaxTopk)) {
+            return STATUS_BAD_PARAM;
+        }
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    auto *out = static_cast<uint64_t *>(result);
+    auto *in = static_cast<const uint16_t *>(probs);
+    const bool vec = amd::aligned16(probs);
+    if (sample && k >= 2) {
+        if (vec) random_sample_topk<true><<<1, BS, 0, s>>>(out, in, desc->voc, random_val, topp, k, temperature);
+        else random_sample_topk<false><<<1, BS, 0, s>>>(out, in, desc->voc, random_val, topp, k, temperature);
+    } else if (sample) {
+        // a vocabulary of one logit: the only candidate has probability 1 and
+        // wins unless random_val >= 1, as in the reference's loops
+        if (random_val < 1.0f) {
+            if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, desc->voc);
+            else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, desc->voc);
+        }
+    } else {
+        if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, desc->voc);
+        else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, desc->voc);
+    }
+    AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+    return STATUS_SUCCESS;
+}

@@ -81,6 +81,10 @@ class AttentionDescriptor(_OpDescriptor):
     pass
 
 
+class RandomSampleDescriptor(_OpDescriptor):
+    pass
+
+
 infiniopAddDescriptor_t = POINTER(AddDescriptor)
 infiniopRMSNormDescriptor_t = POINTER(RMSNormDescriptor)
 infiniopRoPEDescriptor_t = POINTER(RoPEDescriptor)
@@ -91,6 +95,7 @@ infiniopAddRMSNormDescriptor_t = POINTER(AddRMSNormDescriptor)
 infiniopMatmulDescriptor_t = POINTER(MatmulDescriptor)
 infiniopMLPDescriptor_t = POINTER(MLPDescriptor)
 infiniopAttentionDescriptor_t = POINTER(AttentionDescriptor)
+infiniopRandomSampleDescriptor_t = POINTER(RandomSampleDescriptor)
 
 
 class CTensor:
@@ -148,6 +153,10 @@ _PROTOTYPES = {
     "infiniopGetAttentionWorkspaceSize": [infiniopAttentionDescriptor_t, POINTER(c_uint64)],
     "infiniopAttention": [infiniopAttentionDescriptor_t, c_void_p, c_uint64] + [c_void_p] * 7,
     "infiniopDestroyAttentionDescriptor": [infiniopAttentionDescriptor_t],
+    "infiniopCreateRandomSampleDescriptor": [infiniopHandle_t, POINTER(infiniopRandomSampleDescriptor_t), infiniopTensorDescriptor_t, infiniopTensorDescriptor_t],
+    "infiniopGetRandomSampleWorkspaceSize": [infiniopRandomSampleDescriptor_t, POINTER(c_uint64)],
+    "infiniopRandomSample": [infiniopRandomSampleDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_float, c_float, c_int, c_float, c_void_p],
+    "infiniopDestroyRandomSampleDescriptor": [infiniopRandomSampleDescriptor_t],
     "infiniopCreateAddRMSNormDescriptor": [infiniopHandle_t, POINTER(infiniopAddRMSNormDescriptor_t)] + [infiniopTensorDescriptor_t] * 5 + [c_float],
     "infiniopGetAddRMSNormWorkspaceSize": [infiniopAddRMSNormDescriptor_t, POINTER(c_uint64)],
     "infiniopAddRMSNorm": [infiniopAddRMSNormDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],

@@ -21,6 +21,7 @@ from .liboperators import (
     infiniopMatmulDescriptor_t,
     infiniopMLPDescriptor_t,
     infiniopRMSNormDescriptor_t,
+    infiniopRandomSampleDescriptor_t,
     infiniopRoPEDescriptor_t,
     infiniopSwiGLUDescriptor_t,
     open_lib,
@@ -258,6 +259,30 @@ class CausalSoftmaxPlan(_Plan):
         return y
 
 
+class RandomSamplePlan(_Plan):
+    """One token index drawn from a 1-D fp16 logits tensor into a uint64 (or
+    int64, whose bits are the same) result tensor."""
+    _destroy = "infiniopDestroyRandomSampleDescriptor"
+
+    def __init__(self, ctx, result, probs):
+        super().__init__(ctx)
+        cts = self._describe(result, probs)
+        desc = infiniopRandomSampleDescriptor_t()
+        try:
+            check_error(self.lib.infiniopCreateRandomSampleDescriptor(ctx.handle, ctypes.byref(desc), cts[0].descriptor, cts[1].descriptor))
+        finally:
+            self._release(cts)
+        self.desc = desc
+        size = ctypes.c_uint64(0)
+        check_error(self.lib.infiniopGetRandomSampleWorkspaceSize(desc, ctypes.byref(size)))
+        self.workspace_size = size.value
+
+    def __call__(self, result, probs, random_val, topp, topk, temperature, stream=None):
+        check_error(self.lib.infiniopRandomSample(self.desc, None, self.workspace_size, result.data_ptr(), probs.data_ptr(),
+                                                  random_val, topp, topk, temperature, stream))
+        return result
+
+
 class RearrangePlan(_Plan):
     _destroy = "infiniopDestroyRearrangeDescriptor"
 
@@ -333,6 +358,10 @@ class Context:
     def rearrange(self, dst, src, stream=None):
         with RearrangePlan(self, dst, src) as plan:
             return plan(dst, src, stream)
+
+    def random_sample(self, result, probs, random_val, topp, topk, temperature, stream=None):
+        with RandomSamplePlan(self, result, probs) as plan:
+            return plan(result, probs, random_val, topp, topk, temperature, stream)
 
     def causal_softmax(self, y, stream=None):
         with CausalSoftmaxPlan(self, y) as plan:

@@ -648,3 +648,113 @@ ORACLE_API int oracle_matmul(uint32_t dt, uint64_t batch, uint64_t m, uint64_t n
     }
     return ST_SUCCESS;
 }
+
+/* ------------------------------------------------------------------------ *
+ * RandomSample (fourth operator beyond the four-operator path)
+ * ------------------------------------------------------------------------ */
+
+/* Create-time checks of src/ops/random_sample/cpu/random_sample.cc:7-33 in the
+ * reference's order: probs of rank 1; probs F16; result U64; result refused
+ * only when it is neither of rank 1 nor has a first extent of 1.  A result
+ * with no dimensions (whose first extent the reference reads anyway) counts
+ * as a scalar here and passes. */
+ORACLE_API int oracle_random_sample_check(const oracle_tensor *result, const oracle_tensor *probs) {
+    if (probs->ndim != 1) {
+        return ST_BAD_TENSOR_SHAPE;
+    }
+    if (probs->dt != DT_F16) {
+        return ST_BAD_TENSOR_DTYPE;
+    }
+    if (result->dt != DT_U64) {
+        return ST_BAD_TENSOR_DTYPE;
+    }
+    if (result->ndim != 1 && result->ndim != 0 && result->shape[0] != 1) {
+        return ST_BAD_TENSOR_SHAPE;
+    }
+    return ST_SUCCESS;
+}
+
+/* src/ops/random_sample/cpu/random_sample.cc:47-171.  `logits` and `order`
+ * are the caller's scratch of voc entries each (the reference carves them out
+ * of its workspace).  Returns 1 when result[0] was written, 0 when it was
+ * left alone (the last loop of the sampling form found no entry, which
+ * happens for random_val >= 1 or NaN probabilities).
+ *
+ * Sampling form (topp > 0 and topk > 1): a partial selection sort moves the
+ * topk largest codes to the front in descending order - position i is swapped
+ * with every later position holding a strictly greater value, and the value
+ * written back goes through f16 -> f32 -> f16; then every entry becomes
+ * f32_to_f16(expf((x - max) / temperature) / sum), the sum running in fp32
+ * over the array in its permuted order; a running fp32 sum over the first
+ * topk entries finds where it reaches topp; random_val is scaled by the sum
+ * of the kept prefix and the first entry whose running sum exceeds it wins.
+ * Greedy form (otherwise): the first index holding the maximum. */
+ORACLE_API int oracle_random_sample(uint64_t *result, const uint16_t *probs, int voc, float random_val, float topp,
+                                    int topk, float temperature, uint16_t *logits, uint64_t *order) {
+    memcpy(logits, probs, (size_t) voc * sizeof(uint16_t));
+    if (!(topp > 0 && topk > 1)) {
+        float m = oracle_f16_to_f32(logits[0]);
+        int index = 0;
+        for (int j = 1; j < voc; ++j) {
+            if (m < oracle_f16_to_f32(logits[j])) {
+                m = oracle_f16_to_f32(logits[j]);
+                index = j;
+            }
+        }
+        result[0] = (uint64_t) index;
+        return 1;
+    }
+    if (topk > voc) {
+        topk = voc;
+    }
+    for (int i = 0; i < voc; ++i) {
+        order[i] = (uint64_t) i;
+    }
+    for (int i = 0; i < topk; ++i) {
+        for (int j = i + 1; j < voc; ++j) {
+            if (oracle_f16_to_f32(logits[i]) < oracle_f16_to_f32(logits[j])) {
+                const float held = oracle_f16_to_f32(logits[i]);
+                logits[i] = logits[j];
+                logits[j] = oracle_f32_to_f16(held);
+                const int t = (int) order[i];
+                order[i] = order[j];
+                order[j] = (uint64_t) t;
+            }
+        }
+    }
+    const float top = oracle_f16_to_f32(logits[0]);
+    float total = 0.0f;
+    for (int i = 0; i < voc; ++i) {
+        total += expf((oracle_f16_to_f32(logits[i]) - top) / temperature);
+    }
+    for (int i = 0; i < voc; ++i) {
+        logits[i] = oracle_f32_to_f16(expf((oracle_f16_to_f32(logits[i]) - top) / temperature) / total);
+    }
+    float run = 0.0f;
+    int end;
+    for (end = 0; end < topk; ++end) {
+        run += oracle_f16_to_f32(logits[end]);
+        if (run >= topp) {
+            break;
+        }
+    }
+    if (end < topk - 1) {
+        end += 1;
+    } else {
+        end = topk;
+    }
+    float kept = 0.0f;
+    for (int i = 0; i < end; ++i) {
+        kept += oracle_f16_to_f32(logits[i]);
+    }
+    random_val *= kept;
+    kept = 0.0f;
+    for (int i = 0; i < end; ++i) {
+        kept += oracle_f16_to_f32(logits[i]);
+        if (random_val < kept) {
+            result[0] = order[i];
+            return 1;
+        }
+    }
+    return 0;
+}

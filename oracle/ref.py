@@ -18,6 +18,7 @@ from operators_amd.liboperators import (
     infiniopAddDescriptor_t,
     infiniopCausalSoftmaxDescriptor_t,
     infiniopRearrangeDescriptor_t,
+    infiniopRandomSampleDescriptor_t,
     infiniopHandle_t,
     infiniopRMSNormDescriptor_t,
     infiniopRoPEDescriptor_t,
@@ -304,3 +305,33 @@ def attention(out, q, k, v, k_cache, v_cache, pos, dtype):
     lib().infiniopDestroyAttentionDescriptor(desc)
     _free(*ds)
     return out
+
+
+def random_sample_status(result, probs):
+    dr, dp = descriptor(*result), descriptor(*probs)
+    desc = infiniopRandomSampleDescriptor_t()
+    st = lib().infiniopCreateRandomSampleDescriptor(handle(), ctypes.byref(desc), dr, dp)
+    if st == 0:
+        lib().infiniopDestroyRandomSampleDescriptor(desc)
+    _free(dr, dp)
+    return st
+
+
+def random_sample(probs, random_val, topp, topk, temperature):
+    """Chosen index through the reference's own CPU back end, or None when it
+    leaves the result unwritten."""
+    probs = np.ascontiguousarray(probs, dtype=np.uint16)
+    result = np.full(1, 0xFFFFFFFFFFFFFFFF, dtype=np.uint64)
+    dr, dp = _desc_of(result, "u64"), _desc_of(probs, "f16")
+    desc = infiniopRandomSampleDescriptor_t()
+    st = lib().infiniopCreateRandomSampleDescriptor(handle(), ctypes.byref(desc), dr, dp)
+    assert st == 0, st
+    size = ctypes.c_uint64(0)
+    assert lib().infiniopGetRandomSampleWorkspaceSize(desc, ctypes.byref(size)) == 0
+    work = np.empty(max(int(size.value), 1), dtype=np.uint8)
+    st = lib().infiniopRandomSample(desc, work.ctypes.data, size.value, result.ctypes.data, probs.ctypes.data,
+                                    random_val, topp, topk, temperature, None)
+    assert st == 0, st
+    lib().infiniopDestroyRandomSampleDescriptor(desc)
+    _free(dr, dp)
+    return None if int(result[0]) == 0xFFFFFFFFFFFFFFFF else int(result[0])

@@ -254,6 +254,54 @@ def rearrange_vectors(rng):
     return out
 
 
+# (voc, random_val, topp, topk, temperature, kind of logits).  The first nine are the reference's own test
+# cases (operatorspy/tests/random_sample.py:161-171, uniform [0, 1) logits as there); the rest vary the
+# distribution, the tail length, the ties and the special values.
+RANDOM_SAMPLE_CASES = [
+    (512, 0.92, 0.8, 3, 0.5, "uniform"), (4096, 0.95, 0.9, 5, 1.0, "uniform"), (16384, 0.85, 0.85, 10, 2.0, "uniform"),
+    (512, 0.92, 0.0, 3, 0.5, "uniform"), (4096, 0.95, 0.9, 1, 1.0, "uniform"), (16384, 0.85, 0.0, 1, 2.0, "uniform"),
+    (16384, 0.85, 0.0, 1, 2.0, "uniform"), (32000, 0.8, 0.8, 50, 1.0, "uniform"), (32000, 0.8, 1.0, 25, 1.0, "uniform"),
+    (32000, 0.31, 0.95, 40, 0.7, "normal"), (32000, 0.999, 1.0, 64, 1.5, "normal"), (32003, 0.5, 0.9, 20, 1.0, "normal"),
+    (1001, 0.0, 0.5, 8, 1.0, "normal"), (1001, 0.77, 0.3, 8, 0.25, "normal"), (5, 0.6, 0.9, 9, 1.0, "normal"),
+    (2, 0.99, 1.0, 2, 1.0, "normal"), (1, 0.5, 0.9, 4, 1.0, "normal"), (1, 0.5, 0.0, 1, 1.0, "normal"),
+    (4096, 0.4, 0.9, 12, 1.0, "few_values"), (4096, 0.9, 1.0, 300, 1.0, "few_values"), (777, 0.2, 0.0, 5, 1.0, "few_values"),
+    (8192, 0.66, 0.99, 1000, 3.0, "normal"), (50000, 0.45, 0.8, 30, 0.9, "normal"),
+    (640, 1.0, 0.9, 6, 1.0, "normal"),            # random_val = 1: nothing is written
+    (640, 0.3, 0.0, 1, 1.0, "nan_inside"), (640, 0.3, 0.0, 1, 1.0, "nan_first"), (640, 0.3, 0.9, 1, 1.0, "neg_zero_first"),
+    (900, 0.5, 0.9, 7, 1.0, "with_inf"),
+]
+
+
+def random_sample_logits(rng, voc, kind):
+    if kind == "uniform":
+        return rng.random(voc, dtype=np.float32).astype(np.float16).view(np.uint16)
+    if kind == "few_values":
+        return rng.choice(np.array([-1.5, 0.0, 0.25, 2.0, 3.5], np.float16), voc).view(np.uint16)
+    x = (rng.standard_normal(voc, dtype=np.float32) * 3).astype(np.float16).view(np.uint16)
+    if kind == "nan_inside":
+        x[voc // 2] = 0x7E01
+    elif kind == "nan_first":
+        x[0] = 0xFE00
+    elif kind == "neg_zero_first":
+        x[:] = np.where(x & 0x8000, x, 0x0000)  # nothing positive: the maximum is zero
+        x[0], x[5] = 0x8000, 0x0000
+    elif kind == "with_inf":
+        x[3], x[17] = 0xFC00, 0xFC00
+    return x
+
+
+def random_sample_vectors():
+    rng = np.random.default_rng(20241126)
+    out, index = {}, []
+    for i, (voc, rv, topp, topk, temp, kind) in enumerate(RANDOM_SAMPLE_CASES):
+        x = random_sample_logits(rng, voc, kind)
+        got = ref.random_sample(x, rv, topp, topk, temp)
+        out[f"rs{i}_logits"] = x
+        index.append(-1 if got is None else got)
+    out["rs_index"] = np.array(index, np.int64)
+    return out
+
+
 def status_cases():
     """Create-time (and, for RMSNorm, compute-time) status codes of the reference."""
     cases = []
@@ -272,6 +320,8 @@ def status_cases():
             st = ref.causal_softmax_status(*tensors)
         elif op == "rearrange":
             st = ref.rearrange_status(*tensors)
+        elif op == "random_sample":
+            st = ref.random_sample_status(*tensors)
         cases.append({"op": op, "tensors": specs, "status": int(st), **extra})
 
     T = lambda dt, shape, st=None: (dt, tuple(shape), None if st is None else tuple(st))  # noqa: E731
@@ -350,11 +400,27 @@ def status_cases():
     rec("rearrange", [T("f16", (2, 2, 3, 4, 8)), T("f16", (2, 2, 3, 4, 8), (400, 192, 64, 10, 1))])  # dim 1 does not nest in dim 0
     rec("rearrange", [T("bf16", (4, 64)), T("bf16", (4, 64))])
     rec("rearrange", [T("u8", (4, 64)), T("u8", (4, 64), (100, 1))])
+    # RandomSample (result, probs)
+    rec("random_sample", [T("u64", (1,)), T("f16", (512,))])
+    rec("random_sample", [T("u64", (4,)), T("f16", (512,))])         # rank 1 of any length passes
+    rec("random_sample", [T("u64", (1, 3)), T("f16", (512,))])       # first extent 1 passes
+    rec("random_sample", [T("u64", (2, 3)), T("f16", (512,))])
+    rec("random_sample", [T("u64", (1,)), T("f16", (2, 256))])
+    rec("random_sample", [T("u64", (1,)), T("f32", (512,))])
+    rec("random_sample", [T("i64", (1,)), T("f16", (512,))])
+    rec("random_sample", [T("i64", (2, 3)), T("f16", (512,))])       # type is reported before shape
+    rec("random_sample", [T("u64", (1,)), T("bf16", (512,))])
     return cases
 
 
-def main():
+def main(only=None):
+    """With `only` (a set of fixture names) the other .npz files are left as they are."""
     assert ref.available(), "build oracle/_ref first: make -C oracle ref"
+    if only is not None:
+        if "random_sample" in only:
+            np.savez_compressed(os.path.join(HERE, "random_sample.npz"), **random_sample_vectors())
+        write_json()
+        return
     rng = np.random.default_rng(20241125)
     np.savez_compressed(os.path.join(HERE, "conversions.npz"), **conversions(rng))
     np.savez_compressed(os.path.join(HERE, "add.npz"), **add_vectors(rng))
@@ -363,16 +429,22 @@ def main():
     np.savez_compressed(os.path.join(HERE, "swiglu.npz"), **swiglu_vectors(rng))
     np.savez_compressed(os.path.join(HERE, "causal_softmax.npz"), **causal_softmax_vectors(rng))
     np.savez_compressed(os.path.join(HERE, "rearrange.npz"), **rearrange_vectors(rng))
+    np.savez_compressed(os.path.join(HERE, "random_sample.npz"), **random_sample_vectors())
+    write_json()
+
+
+def write_json():
     with open(os.path.join(HERE, "status_cases.json"), "w") as f:
         json.dump({"add_cases": [list(map(list, c)) for c in ADD_CASES],
                    "rope_cases": [[list(s), None if st is None else list(st), r] for s, st, r in ROPE_CASES],
                    "swiglu_cases": [[list(s), a, b, c] for s, a, b, c in SWIGLU_CASES],
                    "rearrange_cases": [[dt, list(sh), None if a is None else list(a), None if b is None else list(b)] for dt, sh, a, b in REARRANGE_CASES],
                    "causal_cases": [[list(s), None if st is None else list(st)] for s, st in CAUSAL_CASES],
+                   "random_sample_cases": [list(c) for c in RANDOM_SAMPLE_CASES],
                    "status": status_cases()}, f, indent=1)
     for name in sorted(os.listdir(HERE)):
         print(f"{name:24s} {os.path.getsize(os.path.join(HERE, name)):>9d} bytes")
 
 
 if __name__ == "__main__":
-    main()
+    main(set(sys.argv[1:]) or None)

@@ -19,7 +19,7 @@ def declared_in_header():
 
 def test_header_declares_every_entry_point():
     names = declared_in_header()
-    assert len(names) == 41  # handle 2 + tensor 2 + add 3 + rms_norm 4 + rope 4 + swiglu 3 + causal_softmax 4 + rearrange 3 + add_rms_norm 4 + matmul 4 + mlp 4 + attention 4
+    assert len(names) == 45  # handle 2 + tensor 2 + add 3 + rms_norm 4 + rope 4 + swiglu 3 + causal_softmax 4 + rearrange 3 + add_rms_norm 4 + matmul 4 + mlp 4 + attention 4 + random_sample 4
     assert sorted(EXPORTED_SYMBOLS) == names
 
 

@@ -1,0 +1,175 @@
+"""RandomSample on the GPU through the C ABI, against the compiled reference's
+golden indices and the oracle.
+
+Bar: the returned index is the oracle's, or - where equal logits exist - an
+index holding the same logit value (the reference's own criterion,
+operatorspy/tests/random_sample.py: `indices == ans or data[indices] ==
+data[ans]`; the CPU's order among equal values depends on the swap history of
+its selection sort, the GPU orders them by index).  For logits without ties
+the index itself must agree.  Where the reference leaves the result unwritten
+(random_val >= 1) the GPU must leave it unwritten too."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import golden, golden_json, to_torch
+
+pytestmark = pytest.mark.gpu
+CASES = golden_json()["random_sample_cases"]
+SENTINEL = -12345
+
+
+def gpu_sample(ctx, codes, rv, topp, topk, temp, offset=0):
+    """offset (elements) places the logits at an address that is not 16-byte aligned."""
+    import torch
+
+    codes = np.ascontiguousarray(codes, np.uint16)
+    if offset:
+        buf = to_torch(np.concatenate([np.zeros(offset, np.uint16), codes]), "f16")
+        probs = buf[offset:]
+    else:
+        probs = to_torch(codes, "f16")
+    result = torch.full((1,), SENTINEL, dtype=torch.int64, device="cuda")  # the bits of a uint64
+    view = result.view(torch.uint64)
+    ctx.random_sample(view, probs, rv, topp, topk, temp)
+    torch.cuda.synchronize()
+    got = int(result.item())
+    return None if got == SENTINEL else got
+
+
+def same_choice(codes, got, want):
+    if got == want:
+        return True
+    if got is None or want is None:
+        return False
+    v = np.asarray(codes, np.uint16).view(np.float16)
+    return 0 <= got < v.size and float(v[got]) == float(v[want])
+
+
+@pytest.mark.parametrize("i", range(len(CASES)))
+def test_golden_cases(ctx, i):
+    voc, rv, topp, topk, temp, kind = CASES[i]
+    g = golden("random_sample")
+    x = g[f"rs{i}_logits"]
+    want = int(g["rs_index"][i])
+    want = None if want < 0 else want
+    got = gpu_sample(ctx, x, rv, topp, topk, temp)
+    assert same_choice(x, got, want), (CASES[i], got, want)
+    if kind in ("uniform", "normal") and np.unique(x).size == x.size:
+        assert got == want
+
+
+@pytest.mark.parametrize("offset", [0, 3])
+def test_against_oracle_distinct_logits(ctx, offset):
+    """No two logits equal: the index itself must be the oracle's."""
+    rng = np.random.default_rng(21 + offset)
+    pool = np.arange(0x0400, 0x7C00, dtype=np.uint16)  # every positive normal fp16 code
+    pool = np.concatenate([pool, pool | 0x8000])
+    bad = []
+    for trial in range(120):
+        voc = int(rng.choice([2, 7, 8, 9, 63, 500, 1024, 4096, 8191, 8200, 32000, 50257]))
+        x = rng.choice(pool, voc, replace=False)
+        scale = rng.choice([0, 1, 2])  # squeeze the range so several candidates carry weight
+        if scale:
+            v = x.view(np.float16).astype(np.float32)
+            v = np.sign(v) * np.log1p(np.abs(v)) * (1.0 if scale == 1 else 0.3)
+            x = np.unique(v.astype(np.float16).view(np.uint16))
+            x = x[(x & 0x7FFF) != 0]
+            rng.shuffle(x)
+            voc = x.size
+        args = (float(rng.random()), float(rng.choice([0.0, 0.3, 0.8, 0.95, 1.0])), int(rng.choice([1, 2, 3, 5, 20, 50, 200, 1024])),
+                float(rng.choice([0.5, 1.0, 2.0, 10.0])))
+        want = oracle.random_sample(x, *args)
+        got = gpu_sample(ctx, x, *args, offset=offset)
+        if got != want:
+            bad.append((trial, voc, args, got, want))
+    assert not bad, bad[:5]
+
+
+def test_against_oracle_with_ties(ctx):
+    rng = np.random.default_rng(77)
+    bad = []
+    for trial in range(80):
+        voc = int(rng.choice([5, 64, 777, 4096, 32000, 151936]))
+        kind = trial % 3
+        if kind == 0:
+            x = rng.random(voc, dtype=np.float32).astype(np.float16)  # the reference test's distribution: many ties at 32000
+        elif kind == 1:
+            x = (rng.standard_normal(voc, dtype=np.float32) * 2.5).astype(np.float16)
+        else:
+            x = rng.choice(np.array([-3.0, -0.0, 0.0, 0.5, 0.5009765625, 4.0], np.float16), voc)
+        codes = x.view(np.uint16)
+        args = (float(rng.random()), float(rng.choice([0.0, 0.5, 0.9, 1.0])), int(rng.choice([1, 2, 4, 10, 50, 300, 1024, 5000])),
+                float(rng.choice([0.5, 1.0, 2.0])))
+        if min(args[2], voc) > 1024 and args[1] > 0:
+            continue  # refused, see test_limits
+        want = oracle.random_sample(codes, *args)
+        got = gpu_sample(ctx, codes, *args)
+        if not same_choice(codes, got, want):
+            bad.append((trial, voc, args, got, want))
+    assert not bad, bad[:5]
+
+
+def test_equal_logits_come_in_index_order(ctx):
+    """A flat distribution over the candidates (huge temperature, topp = 1):
+    random_val picks by rank, and equal logits are ranked by ascending index."""
+    x = np.full(4000, 1.0, np.float16)
+    x[[17, 1800, 3999]] = 2.0
+    codes = x.view(np.uint16)
+    k = 8
+    expect = [17, 1800, 3999, 0, 1, 2, 3, 4]
+    for r in range(k):
+        assert gpu_sample(ctx, codes, (r + 0.5) / k, 1.0, k, 1e9) == expect[r]
+
+
+def test_greedy_special_values(ctx):
+    x = (np.random.default_rng(1).standard_normal(5000) * 2).astype(np.float16)
+    codes = x.view(np.uint16).copy()
+    assert gpu_sample(ctx, codes, 0.5, 0.0, 5, 1.0) == int(np.argmax(x))
+    assert gpu_sample(ctx, codes, 0.5, 0.9, 1, 1.0) == int(np.argmax(x))
+    assert gpu_sample(ctx, codes, 0.5, 0.9, -7, 1.0) == int(np.argmax(x))
+    c = codes.copy()
+    c[2500] = 0x7E00  # a NaN further back is never greater than anything
+    assert gpu_sample(ctx, c, 0.5, 0.0, 1, 1.0) == oracle.random_sample(c, 0.5, 0.0, 1, 1.0) == int(np.argmax(x))
+    c[0] = 0x7E00     # a NaN in front is never beaten
+    assert gpu_sample(ctx, c, 0.5, 0.0, 1, 1.0) == oracle.random_sample(c, 0.5, 0.0, 1, 1.0) == 0
+    c = np.full(300, 0xFC00, np.uint16)  # all -Inf: the first
+    assert gpu_sample(ctx, c, 0.5, 0.0, 1, 1.0) == 0
+    c[123] = 0x8000
+    c[200] = 0x0000   # -0 and +0 are equal: the first of them
+    assert gpu_sample(ctx, c, 0.5, 0.0, 1, 1.0) == oracle.random_sample(c, 0.5, 0.0, 1, 1.0) == 123
+
+
+def test_limits(ctx):
+    import torch
+
+    from operators_amd.ops import RandomSamplePlan
+    from operators_amd.utils import InfiniopError
+
+    probs = to_torch((np.random.default_rng(2).standard_normal(4096)).astype(np.float16).view(np.uint16), "f16")
+    result = torch.zeros(1, dtype=torch.int64, device="cuda").view(torch.uint64)
+    with RandomSamplePlan(ctx, result, probs) as plan:
+        assert plan.workspace_size == 0
+        plan(result, probs, 0.5, 0.9, 1024, 1.0)          # the largest candidate count
+        torch.cuda.synchronize()
+        with pytest.raises(InfiniopError):
+            plan(result, probs, 0.5, 0.9, 1025, 1.0)
+        plan(result, probs, 0.5, 0.0, 100000, 1.0)        # greedy form: topk is not looked at
+        torch.cuda.synchronize()
+    # random_val = 1: the reference writes nothing, neither does the kernel
+    codes = (np.random.default_rng(3).standard_normal(640)).astype(np.float16).view(np.uint16)
+    assert oracle.random_sample(codes, 1.0, 0.9, 6, 1.0) is None
+    assert gpu_sample(ctx, codes, 1.0, 0.9, 6, 1.0) is None
+    # one logit
+    assert gpu_sample(ctx, codes[:1], 0.5, 0.9, 4, 1.0) == 0
+    assert gpu_sample(ctx, codes[:1], 0.5, 0.0, 1, 1.0) == 0
+
+
+def test_large_vocabulary(ctx):
+    rng = np.random.default_rng(8)
+    for voc in (151936, 1_000_003):
+        x = (rng.standard_normal(voc, dtype=np.float32) * 3).astype(np.float16).view(np.uint16)
+        for args in ((0.37, 0.9, 40, 0.8), (0.9, 0.0, 1, 1.0)):
+            want = oracle.random_sample(x, *args)
+            got = gpu_sample(ctx, x, *args)
+            assert same_choice(x, got, want), (voc, args, got, want)

@@ -35,6 +35,9 @@ def test_oracle_checks_reproduce_reference_status(i):
     elif case["op"] == "rearrange":
         assert oracle.rearrange_check(*specs) == case["status"], case
         return
+    elif case["op"] == "random_sample":
+        assert oracle.random_sample_check(*specs) == case["status"], case
+        return
     elif case["op"] == "causal_softmax":
         st = oracle.causal_softmax_check(specs[0], allow_bf16=False, unit_inner=False)
         assert st == case["status"], case
@@ -79,6 +82,7 @@ CREATE = {
     "rms_norm": ("infiniopCreateRMSNormDescriptor", "infiniopDestroyRMSNormDescriptor", oa.infiniopRMSNormDescriptor_t),
     "rearrange": ("infiniopCreateRearrangeDescriptor", "infiniopDestroyRearrangeDescriptor", oa.infiniopRearrangeDescriptor_t),
     "causal_softmax": ("infiniopCreateCausalSoftmaxDescriptor", "infiniopDestroyCausalSoftmaxDescriptor", oa.infiniopCausalSoftmaxDescriptor_t),
+    "random_sample": ("infiniopCreateRandomSampleDescriptor", "infiniopDestroyRandomSampleDescriptor", oa.infiniopRandomSampleDescriptor_t),
 }
 
 
@@ -113,6 +117,8 @@ def test_library_host_validation_reproduces_reference_status(fake_handle, i):
             assert lib.infiniopGetRMSNormWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
         if case["op"] == "rope":
             assert lib.infiniopGetRoPEWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
+        if case["op"] == "random_sample":
+            assert lib.infiniopGetRandomSampleWorkspaceSize(d, ctypes.byref(size)) == 0 and size.value == 0
         assert getattr(lib, destroy)(d) == 0
     for x in descs:
         lib.infiniopDestroyTensorDescriptor(x)
@@ -248,3 +254,29 @@ def test_null_output_pointer_is_memory_not_allocated(fake_handle):
     assert lib.infiniopCreateRoPEDescriptor(handle, None, t, p, s, s) == 6  # rotary_embedding_cpu.cc:54-55
     for x in (t, p, s):
         lib.infiniopDestroyTensorDescriptor(x)
+
+
+def test_random_sample_host_rules_beyond_the_reference(fake_handle):
+    """A strided or empty logits vector is refused at create time; more than
+    1024 candidates (after clamping topk to the vocabulary) and null pointers
+    are refused at stage 4 before anything touches the device."""
+    lib = oa.open_lib()
+    handle, _keep = fake_handle
+
+    def create(result, probs):
+        descs = [oa.make_descriptor(lib, t[1], t[2], LAYOUT[t[0]]) for t in (result, probs)]
+        d = oa.infiniopRandomSampleDescriptor_t()
+        st = lib.infiniopCreateRandomSampleDescriptor(handle, ctypes.byref(d), *descs)
+        for x in descs:
+            lib.infiniopDestroyTensorDescriptor(x)
+        return st, d
+
+    assert create(("u64", (1,), None), ("f16", (512,), (2,)))[0] == 5
+    assert create(("u64", (1,), None), ("f16", (0,), None))[0] == 4
+    assert create(("u64", (), None), ("f16", (512,), None))[0] == 0
+    st, d = create(("u64", (1,), None), ("f16", (4096,), None))
+    assert st == 0
+    f = ctypes.c_float
+    assert lib.infiniopRandomSample(d, None, 0, None, None, f(0.5), f(0.9), 4, f(1.0), None) == 2
+    assert lib.infiniopRandomSample(d, None, 0, 8, 8, f(0.5), f(0.9), 1025, f(1.0), None) == 2
+    assert lib.infiniopDestroyRandomSampleDescriptor(d) == 0
