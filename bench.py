@@ -143,7 +143,8 @@ def make_random_sample(ctx, voc, topk, gen, name):
     result = torch.zeros(1, dtype=torch.int64, device="cuda").view(torch.uint64)
     plan = RandomSamplePlan(ctx, result, logits)
     f = ctypes.c_float
-    args = (plan.desc, None, 0, result.data_ptr(), logits.data_ptr(), f(0.37), f(0.9 if topk > 1 else 0.0), topk, f(0.8))
+    ws = plan.workspace.data_ptr() if plan.workspace is not None else None
+    args = (plan.desc, ws, plan.workspace_size, result.data_ptr(), logits.data_ptr(), f(0.37), f(0.9 if topk > 1 else 0.0), topk, f(0.8))
     return Launch(name, ctx.lib.infiniopRandomSample, args, voc * 2 + 8, (plan, logits, result))
 
 

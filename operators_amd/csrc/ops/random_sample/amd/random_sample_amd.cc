@@ -32,8 +32,14 @@ infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampl
     if (probs->shape[0] > 1 && probs->strides[0] != 1) {
         return STATUS_BAD_TENSOR_STRIDES;
     }
-    auto *desc = new (std::nothrow) RandomSampleAmdDescriptor{DevAmdGpu, handle->device_id,
-                                                              static_cast<uint32_t>(probs->shape[0])};
+    const uint32_t voc = static_cast<uint32_t>(probs->shape[0]);
+    uint32_t groups = 0, vecs = 0;
+    if (voc >= kRandomSampleSplitVoc) {
+        const uint64_t per_vec = kRandomSamplePartLanes * 8ull;
+        vecs = static_cast<uint32_t>(amd::ceil_div(voc, per_vec * kRandomSampleMaxGroups));
+        groups = static_cast<uint32_t>(amd::ceil_div(voc, per_vec * vecs));
+    }
+    auto *desc = new (std::nothrow) RandomSampleAmdDescriptor{DevAmdGpu, handle->device_id, voc, groups, vecs};
     if (desc == nullptr) {
         return STATUS_MEMORY_NOT_ALLOCATED;
     }
@@ -42,13 +48,23 @@ infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampl
 }
 
 // The reference's back ends sort in a workspace of voc * 12 (CPU) or voc * 20
-// bytes plus what their sorting library allocates per call (CUDA).  The
-// kernels here select in registers and LDS and need none.
-infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t, uint64_t *size) {
+// bytes plus what their sorting library allocates per call (CUDA).  Here the
+// workspace only carries the candidates from the first launch of the
+// two-launch form to the second: one header and 512 candidates of 8 bytes per
+// workgroup, under 200 KiB whatever the vocabulary; small vocabularies need
+// none.  A call that comes without it is served by one workgroup.
+uint64_t amdRandomSampleWorkspaceBytes(const RandomSampleAmdDescriptor &d) {
+    if (d.groups == 0) {
+        return 0;
+    }
+    return kRandomSampleMaxGroups * sizeof(RandomSamplePart) + static_cast<uint64_t>(d.groups) * kRandomSamplePartCap * sizeof(uint64_t);
+}
+
+infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t desc, uint64_t *size) {
     if (size == nullptr) {
         return STATUS_BAD_PARAM;
     }
-    *size = 0;
+    *size = amdRandomSampleWorkspaceBytes(*desc);
     return STATUS_SUCCESS;
 }
 

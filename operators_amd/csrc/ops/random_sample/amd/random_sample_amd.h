@@ -10,15 +10,37 @@
 // the sampling form keeps; they live in the workgroup's LDS.
 constexpr int kRandomSampleMaxTopk = 1024;
 
+// Geometry of the two-launch form: workgroups of 256 lanes, each over
+// 2048 * vecs consecutive logits, each with room for 512 surviving candidates
+// in the workspace; at most 48 of them.
+constexpr int kRandomSamplePartLanes = 256;
+constexpr int kRandomSamplePartCap = 512;
+constexpr int kRandomSampleMaxGroups = 48;
+// topk up to which the two-launch form is used (one candidate bound per lane)
+constexpr int kRandomSamplePartTopk = 256;
+// vocabularies below this are sampled by one workgroup in one launch
+constexpr uint32_t kRandomSampleSplitVoc = 4096;
+
+// What one workgroup of the first launch leaves for the second.
+struct RandomSamplePart {
+    uint32_t count;  // candidates it found (more than the cap: the list is incomplete)
+    uint32_t key_max;// key of its largest logit
+    float sum;       // sum of expf((x - its largest) / temperature) over its logits
+    uint32_t unused;
+};
+
 struct RandomSampleAmdDescriptor {
     Device device;
     int device_id;
-    uint32_t voc;// number of logits
+    uint32_t voc;   // number of logits
+    uint32_t groups;// workgroups of the first launch of the two-launch form; 0: never used
+    uint32_t vecs;  // 8-element vectors per lane in them
 };
 typedef RandomSampleAmdDescriptor *RandomSampleAmdDescriptor_t;
 
 infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampleAmdDescriptor_t *desc_ptr,
                                                  infiniopTensorDescriptor_t result, infiniopTensorDescriptor_t probs);
+uint64_t amdRandomSampleWorkspaceBytes(const RandomSampleAmdDescriptor &desc);
 infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t desc, uint64_t *size);
 infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspace, uint64_t workspace_size,
                                  void *result, void const *probs, float random_val, float topp, int topk,

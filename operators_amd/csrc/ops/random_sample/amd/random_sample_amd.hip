@@ -74,6 +74,14 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
     return v;
 }
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = __shfl_xor(v, o);
+        v = other > v ? other : v;
+    }
+    return v;
+}
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -123,20 +131,86 @@ __global__ __launch_bounds__(BS) void random_sample_greedy(uint64_t *result, con
     }
 }
 
-// Sampling form (random_sample.cc:47-126).  topk is already clamped to
-// [2, min(voc, KMAX)].
-template<bool VEC>
-__global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const uint16_t *probs, uint32_t voc,
-                                                          float random_val, float topp, uint32_t topk, float temperature) {
-    __shared__ uint32_t wave_cnt[WAVES * 16];        // per-wavefront digit counts of one select pass
-    __shared__ uint32_t digit_cnt[16];               // their totals
-    __shared__ uint32_t wave_key[WAVES];             // per-wavefront maximum key
-    __shared__ uint32_t scan_tot[2][WAVES][2];       // per-wavefront (greater, equal) counts of one compaction step
-    __shared__ float sum_slots[WAVES];
-    __shared__ unsigned long long cand[KMAX];        // key << 32 | ~index, in index order
-    __shared__ float sorted_p[KMAX];                 // probabilities, widened, in descending order of logit
-    __shared__ uint32_t sorted_i[KMAX];              // their indices
+// LDS of the sampling kernels.
+struct TopkShared {
+    uint32_t wave_cnt[WAVES * 16];   // per-wavefront digit counts of one select pass
+    uint32_t digit_cnt[16];          // their totals
+    uint32_t wave_key[WAVES];        // per-wavefront maximum key
+    uint32_t scan_tot[2][WAVES][2];  // per-wavefront (greater, equal) counts of one compaction step
+    float sum_slots[WAVES];
+    unsigned long long cand[KMAX];   // key << 32 | ~index
+    float sorted_p[KMAX];            // probabilities, widened, in descending order of logit
+    uint32_t sorted_i[KMAX];         // their indices
+};
 
+// One step of a radix select over 16-bit keys: digit_cnt holds how many of the
+// entries that share `prefix` have each value of the next 4-bit digit; walk
+// down from 15 to the digit that contains the entry of rank `want`.
+__device__ __forceinline__ void choose_digit(const uint32_t *digit_cnt, uint32_t &prefix, uint32_t &want) {
+    uint32_t above = 0, chosen = 0;
+    bool found = false;
+#pragma unroll
+    for (int d = 15; d >= 0; --d) {
+        const uint32_t c = digit_cnt[d];
+        if (!found) {
+            if (above + c >= want) {
+                chosen = d;
+                found = true;
+            } else {
+                above += c;
+            }
+        }
+    }
+    want -= above;
+    prefix = (prefix << 4) | chosen;
+}
+
+// Rank the `count` candidates of sh.cand (greater logit first, then the lower
+// index), turn the first topk of them into fp16 probabilities and walk the
+// running sums of random_sample.cc:97-125 in their order.  Ends with the
+// result written, or left alone when no running sum exceeds the limit.
+__device__ __forceinline__ void rank_and_draw(TopkShared &sh, uint64_t *result, uint32_t count, uint32_t topk, float top,
+                                              float total, float random_val, float topp, float temperature) {
+    const int tid = threadIdx.x;
+    if (static_cast<uint32_t>(tid) < count) {
+        const unsigned long long mine = sh.cand[tid];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < count; ++j) rank += sh.cand[j] > mine ? 1u : 0u;
+        if (rank < topk) {
+            const float x = value_of_key(static_cast<uint32_t>(mine >> 32));
+            const float p = expf((x - top) / temperature) / total;
+            sh.sorted_p[rank] = F16Ref::one(F16Ref::narrow1(p));
+            sh.sorted_i[rank] = 0xFFFFFFFFu - static_cast<uint32_t>(mine);
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float run = 0.0f;
+        uint32_t end;
+        for (end = 0; end < topk; ++end) {
+            run += sh.sorted_p[end];
+            if (run >= topp) break;
+        }
+        // `run` is now the sum of the kept prefix in every case: the loop stops
+        // on the last kept entry or runs through all topk of them
+        end = end + 1 < topk ? end + 1 : topk;
+        const float limit = random_val * run;
+        float acc = 0.0f;
+        for (uint32_t i = 0; i < end; ++i) {
+            acc += sh.sorted_p[i];
+            if (limit < acc) {
+                result[0] = sh.sorted_i[i];
+                break;
+            }
+        }
+    }
+}
+
+// Sampling form (random_sample.cc:47-126), everything by one workgroup from
+// the logits themselves.  topk is already clamped to [2, min(voc, KMAX)].
+template<bool VEC>
+__device__ __forceinline__ void topk_full(TopkShared &sh, uint64_t *result, const uint16_t *probs, uint32_t voc,
+                                          float random_val, float topp, uint32_t topk, float temperature) {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t step = BS * 8u;
 
@@ -168,46 +242,26 @@ __global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const
             const uint32_t t = wave_sum_u32(cnt[d]);
             if (lane == d) mine = t;
         }
-        if (lane < 16) wave_cnt[wave * 16 + lane] = mine;
+        if (lane < 16) sh.wave_cnt[wave * 16 + lane] = mine;
         if (shift == 12) {
-            uint32_t m = key_max;
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const uint32_t other = __shfl_xor(m, o);
-                m = other > m ? other : m;
-            }
-            if (lane == 0) wave_key[wave] = m;
+            const uint32_t m = wave_max_u32(key_max);
+            if (lane == 0) sh.wave_key[wave] = m;
         }
         __syncthreads();
         if (tid < 16) {
             uint32_t t = 0;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) t += wave_cnt[w * 16 + tid];
-            digit_cnt[tid] = t;
+            for (int w = 0; w < WAVES; ++w) t += sh.wave_cnt[w * 16 + tid];
+            sh.digit_cnt[tid] = t;
         }
         __syncthreads();
-        uint32_t above = 0, chosen = 0;
-        bool found = false;
-#pragma unroll
-        for (int d = 15; d >= 0; --d) {
-            const uint32_t c = digit_cnt[d];
-            if (!found) {
-                if (above + c >= want) {
-                    chosen = d;
-                    found = true;
-                } else {
-                    above += c;
-                }
-            }
-        }
-        want -= above;
-        prefix = (prefix << 4) | chosen;
+        choose_digit(sh.digit_cnt, prefix, want);
     }
     const uint32_t key_k = prefix;          // key of the topk-th largest
     const uint32_t need_eq = want;          // how many of its equals belong to the topk
     const uint32_t n_greater = topk - want; // elements with a greater key
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) key_max = wave_key[w] > key_max ? wave_key[w] : key_max;
+    for (int w = 0; w < WAVES; ++w) key_max = sh.wave_key[w] > key_max ? sh.wave_key[w] : key_max;
     const float top = value_of_key(key_max);
 
     // ---- compaction in index order, and the softmax denominator ------------
@@ -232,14 +286,14 @@ __global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const
         }
         const uint32_t inc_gt = wave_scan_u32(c_gt, lane), inc_eq = wave_scan_u32(c_eq, lane);
         if (lane == kWave - 1) {
-            scan_tot[buf][wave][0] = inc_gt;
-            scan_tot[buf][wave][1] = inc_eq;
+            sh.scan_tot[buf][wave][0] = inc_gt;
+            sh.scan_tot[buf][wave][1] = inc_eq;
         }
         __syncthreads();
         uint32_t at_gt = run_gt + inc_gt - c_gt, at_eq = run_eq + inc_eq - c_eq;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-            const uint32_t g = scan_tot[buf][w][0], q = scan_tot[buf][w][1];
+            const uint32_t g = sh.scan_tot[buf][w][0], q = sh.scan_tot[buf][w][1];
             if (w < wave) at_gt += g, at_eq += q;
             run_gt += g, run_eq += q;
         }
@@ -248,63 +302,287 @@ __global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const
             if (e < n) {
                 const unsigned long long c = (static_cast<unsigned long long>(k[e]) << 32) | (0xFFFFFFFFu - (base + e));
                 if (k[e] > key_k) {
-                    cand[at_gt++] = c;
+                    sh.cand[at_gt++] = c;
                 } else if (k[e] == key_k) {
-                    if (at_eq < need_eq) cand[n_greater + at_eq] = c;
+                    if (at_eq < need_eq) sh.cand[n_greater + at_eq] = c;
                     ++at_eq;
                 }
             }
         }
     }
     part = wave_sum(part);
-    if (lane == 0) sum_slots[wave] = part;
+    if (lane == 0) sh.sum_slots[wave] = part;
     __syncthreads();// candidates and partial sums are in LDS
     float total = 0.0f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) total += sum_slots[w];
+    for (int w = 0; w < WAVES; ++w) total += sh.sum_slots[w];
+    rank_and_draw(sh, result, topk, topk, top, total, random_val, topp, temperature);
+}
 
-    // ---- rank the candidates: greater logit first, then the lower index ----
-    if (static_cast<uint32_t>(tid) < topk) {
-        const unsigned long long mine = cand[tid];
-        uint32_t rank = 0;
-        for (uint32_t j = 0; j < topk; ++j) rank += cand[j] > mine ? 1u : 0u;
-        const float x = value_of_key(static_cast<uint32_t>(mine >> 32));
-        const float p = expf((x - top) / temperature) / total;
-        sorted_p[rank] = F16Ref::one(F16Ref::narrow1(p));
-        sorted_i[rank] = 0xFFFFFFFFu - static_cast<uint32_t>(mine);
-    }
-    __syncthreads();
+template<bool VEC>
+__global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const uint16_t *probs, uint32_t voc,
+                                                          float random_val, float topp, uint32_t topk, float temperature) {
+    __shared__ TopkShared sh;
+    topk_full<VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
+}
 
-    // ---- the running sums of random_sample.cc:97-125, in their order -------
-    if (tid == 0) {
-        float run = 0.0f;
-        uint32_t end;
-        for (end = 0; end < topk; ++end) {
-            run += sorted_p[end];
-            if (run >= topp) break;
-        }
-        // `run` is now the sum of the kept prefix in every case: the loop stops
-        // on the last kept entry or runs through all topk of them
-        end = end + 1 < topk ? end + 1 : topk;
-        const float limit = random_val * run;
-        float acc = 0.0f;
-        for (uint32_t i = 0; i < end; ++i) {
-            acc += sorted_p[i];
-            if (limit < acc) {
-                result[0] = sorted_i[i];
-                break;
+// ---- the same in two launches, the first spread over the chip ---------------
+// First launch: workgroup w of 256 lanes takes the logits
+// [w * 2048 * vecs, (w + 1) * 2048 * vecs) and leaves in the workspace
+//   * every element that can belong to the overall topk.  The topk-th largest
+//     of the 256 lane maxima is a lower bound of the workgroup's own topk-th
+//     largest element, and an element of the overall topk is among the topk
+//     largest of its workgroup, so elements below that bound are dropped
+//     without a sort: with topk = 50 about 55 of 2048 remain;
+//   * its maximum and its sum of expf((x - maximum) / temperature), which the
+//     second launch rescales to the overall maximum.
+// Second launch: one workgroup selects the topk-th key among the survivors
+// (radix select in LDS), ranks what is left and draws.  Whenever a list
+// overflows - very many equal logits, topk close to 256 - it does the whole
+// job itself from the logits (topk_full), so the answer never depends on the
+// shortcut working.
+template<bool VEC>
+__global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(RandomSamplePart *heads, unsigned long long *lists,
+                                                                                  const uint16_t *probs, uint32_t voc,
+                                                                                  uint32_t vecs, uint32_t topk, float temperature) {
+    constexpr int PBS = kRandomSamplePartLanes, PW = PBS / kWave;
+    __shared__ uint32_t wave_cnt[PW * 16];
+    __shared__ uint32_t digit_cnt[16];
+    __shared__ uint32_t wave_key[PW];
+    __shared__ float sum_slots[PW];
+    __shared__ uint32_t fill;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t start = blockIdx.x * (PBS * 8u * vecs);
+    if (tid == 0) fill = 0;
+
+    // lane maxima and the workgroup's maximum
+    uint32_t lane_max = 0;
+    bool has = false;
+    for (uint32_t v = 0; v < vecs; ++v) {
+        const uint32_t base = start + (v * PBS + tid) * 8u;
+        if (base < voc) {
+            uint32_t h[8];
+            const int n = load_codes<VEC>(probs, voc, base, h);
+            has = true;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t k = key_of(h[e]);
+                if (e < n) lane_max = k > lane_max ? k : lane_max;
             }
         }
     }
+    {
+        const uint32_t m = wave_max_u32(lane_max);
+        if (lane == 0) wave_key[wave] = m;
+    }
+    // the topk-th largest lane maximum (0 = keep everything, when fewer than topk lanes hold data)
+    uint32_t prefix = 0, want = topk;
+    const uint32_t mine_key = has ? lane_max : kNoKey;
+    bool keep_all = false;
+#pragma unroll 1
+    for (int shift = 12; shift >= 0; shift -= 4) {
+        const bool in = (mine_key >> (shift + 4)) == prefix;
+        const uint32_t digit = (mine_key >> shift) & 15u;
+        uint32_t mine = 0;
+#pragma unroll
+        for (int d = 0; d < 16; ++d) {
+            const uint32_t c = __builtin_popcountll(__builtin_amdgcn_ballot_w64(in && digit == static_cast<uint32_t>(d)));
+            if (lane == d) mine = c;
+        }
+        if (lane < 16) wave_cnt[wave * 16 + lane] = mine;
+        __syncthreads();
+        if (tid < 16) {
+            uint32_t t = 0;
+#pragma unroll
+            for (int w = 0; w < PW; ++w) t += wave_cnt[w * 16 + tid];
+            digit_cnt[tid] = t;
+        }
+        __syncthreads();
+        if (shift == 12) {
+            uint32_t lanes_with_data = 0;
+#pragma unroll
+            for (int d = 0; d < 16; ++d) lanes_with_data += digit_cnt[d];
+            if (lanes_with_data < topk) {
+                keep_all = true;
+                break;// uniform over the workgroup
+            }
+        }
+        choose_digit(digit_cnt, prefix, want);
+    }
+    const uint32_t bound = keep_all ? 0u : prefix;
+    uint32_t key_max = 0;
+#pragma unroll
+    for (int w = 0; w < PW; ++w) key_max = wave_key[w] > key_max ? wave_key[w] : key_max;
+    const float top = value_of_key(key_max);
+
+    // survivors to the workspace, and the partial denominator
+    float part = 0.0f;
+    unsigned long long *list = lists + static_cast<size_t>(blockIdx.x) * kRandomSamplePartCap;
+    for (uint32_t v = 0; v < vecs; ++v) {
+        const uint32_t base = start + (v * PBS + tid) * 8u;
+        uint32_t h[8], k[8];
+        int n = 0;
+        uint32_t c = 0;
+        if (base < voc) {
+            n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                k[e] = e < n ? key_of(h[e]) : kNoKey;
+                if (e < n) {
+                    const float x = F16Ref::one(static_cast<uint16_t>(h[e]));
+                    // the maximum itself counts as expf(0) also when it is infinite
+                    part += k[e] == key_max ? 1.0f : expf((x - top) / temperature);
+                    c += k[e] >= bound ? 1u : 0u;
+                }
+            }
+        }
+        const uint32_t inc = wave_scan_u32(c, lane);
+        uint32_t at = 0;
+        if (lane == kWave - 1 && inc != 0) at = atomicAdd(&fill, inc);
+        at = __shfl(at, kWave - 1) + inc - c;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < n && k[e] >= bound) {
+                if (at < static_cast<uint32_t>(kRandomSamplePartCap)) {
+                    list[at] = (static_cast<unsigned long long>(k[e]) << 32) | (0xFFFFFFFFu - (base + e));
+                }
+                ++at;
+            }
+        }
+    }
+    part = wave_sum(part);
+    if (lane == 0) sum_slots[wave] = part;
+    __syncthreads();
+    if (tid == 0) {
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < PW; ++w) total += sum_slots[w];
+        RandomSamplePart head;
+        head.count = fill;
+        head.key_max = key_max;
+        head.sum = total;
+        head.unused = 0;
+        heads[blockIdx.x] = head;
+    }
+}
+
+template<bool VEC>
+__global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, const uint16_t *probs, uint32_t voc, float random_val,
+                                                           float topp, uint32_t topk, float temperature,
+                                                           const RandomSamplePart *heads, const unsigned long long *lists,
+                                                           uint32_t groups) {
+    constexpr int CMAX = 4096, PER_LANE = CMAX / BS;
+    __shared__ TopkShared sh;
+    __shared__ unsigned long long pool[CMAX];
+    __shared__ uint32_t offs[kRandomSampleMaxGroups + 1];
+    __shared__ uint32_t g_key[kRandomSampleMaxGroups];
+    __shared__ float g_sum[kRandomSampleMaxGroups];
+    __shared__ uint32_t verdict[2];// [0]: lists usable, [1]: fill of sh.cand
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+
+    if (static_cast<uint32_t>(tid) < groups) {
+        const RandomSamplePart head = heads[tid];
+        offs[tid + 1] = head.count;
+        g_key[tid] = head.key_max;
+        g_sum[tid] = head.sum;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        bool ok = true;
+        uint32_t run = 0;
+        offs[0] = 0;
+        for (uint32_t w = 0; w < groups; ++w) {
+            const uint32_t c = offs[w + 1];
+            ok = ok && c <= static_cast<uint32_t>(kRandomSamplePartCap);
+            run += c;
+            offs[w + 1] = run;
+        }
+        verdict[0] = (ok && run <= static_cast<uint32_t>(CMAX) && run >= topk) ? 1u : 0u;
+        verdict[1] = 0;
+    }
+    __syncthreads();
+    if (verdict[0] == 0) {// uniform over the workgroup
+        topk_full<VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
+        return;
+    }
+    const uint32_t count = offs[groups];
+
+    // the overall maximum and the denominator rescaled to it, in a fixed order
+    uint32_t key_max = 0;
+    for (uint32_t w = 0; w < groups; ++w) key_max = g_key[w] > key_max ? g_key[w] : key_max;
+    const float top = value_of_key(key_max);
+    float part = 0.0f;
+    if (static_cast<uint32_t>(tid) < groups) {
+        part = g_sum[tid] * expf((value_of_key(g_key[tid]) - top) / temperature);
+    }
+    part = wave_sum(part);// groups <= 64: all of them sit in the first wavefront
+    if (tid == 0) sh.sum_slots[0] = part;
+
+    // the survivors into LDS
+    for (uint32_t w = wave; w < groups; w += WAVES) {
+        const uint32_t from = offs[w], n = offs[w + 1] - from;
+        for (uint32_t j = lane; j < n; j += kWave) pool[from + j] = lists[static_cast<size_t>(w) * kRandomSamplePartCap + j];
+    }
+    __syncthreads();
+    const float total = sh.sum_slots[0];
+
+    // radix select of the topk-th key among them
+    uint32_t keys[PER_LANE];
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) {
+        const uint32_t at = tid + i * BS;
+        keys[i] = at < count ? static_cast<uint32_t>(pool[at] >> 32) : kNoKey;
+    }
+    uint32_t prefix = 0, want = topk, ties = 0;
+#pragma unroll 1
+    for (int shift = 12; shift >= 0; shift -= 4) {
+        uint32_t mine = 0;
+#pragma unroll
+        for (int d = 0; d < 16; ++d) {
+            uint32_t c = 0;
+#pragma unroll
+            for (int i = 0; i < PER_LANE; ++i) {
+                const bool hit = (keys[i] >> (shift + 4)) == prefix && ((keys[i] >> shift) & 15u) == static_cast<uint32_t>(d);
+                c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(hit));
+            }
+            if (lane == d) mine = c;
+        }
+        if (lane < 16) sh.wave_cnt[wave * 16 + lane] = mine;
+        __syncthreads();
+        if (tid < 16) {
+            uint32_t t = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) t += sh.wave_cnt[w * 16 + tid];
+            sh.digit_cnt[tid] = t;
+        }
+        __syncthreads();
+        choose_digit(sh.digit_cnt, prefix, want);
+        if (shift == 0) ties = sh.digit_cnt[prefix & 15u];
+    }
+    // everything above the topk-th key plus every entry equal to it
+    const uint32_t kept = topk - want + ties;
+    if (kept > static_cast<uint32_t>(KMAX)) {// uniform: more equal logits at the boundary than LDS ranks
+        __syncthreads();
+        topk_full<VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) {
+        if (keys[i] != kNoKey && keys[i] >= prefix) sh.cand[atomicAdd(&verdict[1], 1u)] = pool[tid + i * BS];
+    }
+    __syncthreads();
+    rank_and_draw(sh, result, kept, topk, top, total, random_val, topp, temperature);
 }
 
 }// namespace
 
-// Stage 4 of RandomSample.  The workspace is unused (its size is 0).  With
-// topp > 0 and topk > 1 it samples, otherwise it returns the first index of
-// the maximum, as the reference does (random_sample.cc:160-166).
-infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *, uint64_t, void *result, void const *probs,
-                                 float random_val, float topp, int topk, float temperature, void *stream) {
+// Stage 4 of RandomSample.  With topp > 0 and topk > 1 it samples, otherwise
+// it returns the first index of the maximum, as the reference does
+// (random_sample.cc:160-166).  The workspace is used by the two-launch form
+// only; without it (null, too small, misaligned), for more than 256
+// candidates and for small vocabularies one workgroup does the whole call.
+infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspace, uint64_t workspace_size, void *result,
+                                 void const *probs, float random_val, float topp, int topk, float temperature, void *stream) {
     if (result == nullptr || probs == nullptr) {
         return STATUS_BAD_PARAM;
     }
@@ -321,19 +599,35 @@ infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *, uint6
     auto *out = static_cast<uint64_t *>(result);
     auto *in = static_cast<const uint16_t *>(probs);
     const bool vec = amd::aligned16(probs);
+    const uint32_t voc = desc->voc;
     if (sample && k >= 2) {
-        if (vec) random_sample_topk<true><<<1, BS, 0, s>>>(out, in, desc->voc, random_val, topp, k, temperature);
-        else random_sample_topk<false><<<1, BS, 0, s>>>(out, in, desc->voc, random_val, topp, k, temperature);
+        const bool split = desc->groups != 0 && k <= static_cast<uint32_t>(kRandomSamplePartTopk) && workspace != nullptr &&
+                           workspace_size >= amdRandomSampleWorkspaceBytes(*desc) && (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0;
+        if (split) {
+            auto *heads = static_cast<RandomSamplePart *>(workspace);
+            auto *lists = reinterpret_cast<unsigned long long *>(heads + kRandomSampleMaxGroups);
+            if (vec) {
+                random_sample_partial<true><<<desc->groups, kRandomSamplePartLanes, 0, s>>>(heads, lists, in, voc, desc->vecs, k, temperature);
+                random_sample_merge<true><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature, heads, lists, desc->groups);
+            } else {
+                random_sample_partial<false><<<desc->groups, kRandomSamplePartLanes, 0, s>>>(heads, lists, in, voc, desc->vecs, k, temperature);
+                random_sample_merge<false><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature, heads, lists, desc->groups);
+            }
+        } else if (vec) {
+            random_sample_topk<true><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature);
+        } else {
+            random_sample_topk<false><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature);
+        }
     } else if (sample) {
         // a vocabulary of one logit: the only candidate has probability 1 and
         // wins unless random_val >= 1, as in the reference's loops
         if (random_val < 1.0f) {
-            if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, desc->voc);
-            else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, desc->voc);
+            if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, voc);
+            else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, voc);
         }
     } else {
-        if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, desc->voc);
-        else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, desc->voc);
+        if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, voc);
+        else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, voc);
     }
     AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
     return STATUS_SUCCESS;

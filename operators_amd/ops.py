@@ -261,10 +261,14 @@ class CausalSoftmaxPlan(_Plan):
 
 class RandomSamplePlan(_Plan):
     """One token index drawn from a 1-D fp16 logits tensor into a uint64 (or
-    int64, whose bits are the same) result tensor."""
+    int64, whose bits are the same) result tensor.  Owns the workspace the
+    library asks for; with use_workspace=False none is passed and the library
+    serves the call with one workgroup."""
     _destroy = "infiniopDestroyRandomSampleDescriptor"
 
-    def __init__(self, ctx, result, probs):
+    def __init__(self, ctx, result, probs, use_workspace=True):
+        import torch
+
         super().__init__(ctx)
         cts = self._describe(result, probs)
         desc = infiniopRandomSampleDescriptor_t()
@@ -275,10 +279,12 @@ class RandomSamplePlan(_Plan):
         self.desc = desc
         size = ctypes.c_uint64(0)
         check_error(self.lib.infiniopGetRandomSampleWorkspaceSize(desc, ctypes.byref(size)))
-        self.workspace_size = size.value
+        self.workspace_size = size.value if use_workspace else 0
+        self.workspace = torch.empty(self.workspace_size, dtype=torch.uint8, device=probs.device) if self.workspace_size else None
 
     def __call__(self, result, probs, random_val, topp, topk, temperature, stream=None):
-        check_error(self.lib.infiniopRandomSample(self.desc, None, self.workspace_size, result.data_ptr(), probs.data_ptr(),
+        check_error(self.lib.infiniopRandomSample(self.desc, self.workspace.data_ptr() if self.workspace is not None else None,
+                                                  self.workspace_size, result.data_ptr(), probs.data_ptr(),
                                                   random_val, topp, topk, temperature, stream))
         return result
 
@@ -359,9 +365,13 @@ class Context:
         with RearrangePlan(self, dst, src) as plan:
             return plan(dst, src, stream)
 
-    def random_sample(self, result, probs, random_val, topp, topk, temperature, stream=None):
-        with RandomSamplePlan(self, result, probs) as plan:
-            return plan(result, probs, random_val, topp, topk, temperature, stream)
+    def random_sample(self, result, probs, random_val, topp, topk, temperature, stream=None, use_workspace=True):
+        import torch
+
+        with RandomSamplePlan(self, result, probs, use_workspace) as plan:
+            res = plan(result, probs, random_val, topp, topk, temperature, stream)
+            torch.cuda.synchronize()  # the plan's workspace must outlive the work queued on it
+            return res
 
     def causal_softmax(self, y, stream=None):
         with CausalSoftmaxPlan(self, y) as plan:

@@ -20,7 +20,17 @@ SENTINEL = -12345
 
 
 def gpu_sample(ctx, codes, rv, topp, topk, temp, offset=0):
-    """offset (elements) places the logits at an address that is not 16-byte aligned."""
+    """offset (elements) places the logits at an address that is not 16-byte
+    aligned.  Every case runs twice: with the workspace the library asks for
+    (vocabularies of 4096 and more then take the two-launch form) and without
+    it (one workgroup); the two must give the same index."""
+    with_ws = gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, True)
+    without = gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, False)
+    assert with_ws == without, ("with workspace", with_ws, "without", without)
+    return with_ws
+
+
+def gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, use_workspace):
     import torch
 
     codes = np.ascontiguousarray(codes, np.uint16)
@@ -31,7 +41,7 @@ def gpu_sample(ctx, codes, rv, topp, topk, temp, offset=0):
         probs = to_torch(codes, "f16")
     result = torch.full((1,), SENTINEL, dtype=torch.int64, device="cuda")  # the bits of a uint64
     view = result.view(torch.uint64)
-    ctx.random_sample(view, probs, rv, topp, topk, temp)
+    ctx.random_sample(view, probs, rv, topp, topk, temp, use_workspace=use_workspace)
     torch.cuda.synchronize()
     got = int(result.item())
     return None if got == SENTINEL else got
@@ -149,7 +159,7 @@ def test_limits(ctx):
     probs = to_torch((np.random.default_rng(2).standard_normal(4096)).astype(np.float16).view(np.uint16), "f16")
     result = torch.zeros(1, dtype=torch.int64, device="cuda").view(torch.uint64)
     with RandomSamplePlan(ctx, result, probs) as plan:
-        assert plan.workspace_size == 0
+        assert 0 < plan.workspace_size < 200 * 1024
         plan(result, probs, 0.5, 0.9, 1024, 1.0)          # the largest candidate count
         torch.cuda.synchronize()
         with pytest.raises(InfiniopError):
@@ -163,6 +173,28 @@ def test_limits(ctx):
     # one logit
     assert gpu_sample(ctx, codes[:1], 0.5, 0.9, 4, 1.0) == 0
     assert gpu_sample(ctx, codes[:1], 0.5, 0.0, 1, 1.0) == 0
+
+
+def test_lists_that_overflow_fall_back_to_the_full_path(ctx):
+    """More equal logits at the top than a workgroup's candidate list holds,
+    and candidate counts close to the two-launch form's limit: the second
+    launch notices and works from the logits itself."""
+    rng = np.random.default_rng(13)
+    x = (rng.standard_normal(32000, dtype=np.float32)).astype(np.float16)
+    x[rng.choice(32000, 9000, replace=False)] = 6.0   # 9000 equal maxima: every list overflows
+    codes = x.view(np.uint16)
+    for args in ((0.4, 0.9, 50, 1.0), (0.77, 1.0, 256, 2.0), (0.1, 0.5, 2, 0.5)):
+        want = oracle.random_sample(codes, *args)
+        assert same_choice(codes, gpu_sample(ctx, codes, *args), want), args
+    y = (rng.standard_normal(20000, dtype=np.float32) * 2).astype(np.float16).view(np.uint16)
+    for topk in (200, 255, 256, 257):
+        args = (0.63, 0.97, topk, 1.3)
+        assert same_choice(y, gpu_sample(ctx, y, *args), oracle.random_sample(y, *args)), args
+    # the last workgroup holds fewer lanes with data than topk
+    z = (rng.standard_normal(4096 + 8 * 30 + 3, dtype=np.float32) * 2).astype(np.float16).view(np.uint16)
+    for topk in (20, 40, 100):
+        args = (0.5, 0.9, topk, 1.0)
+        assert same_choice(z, gpu_sample(ctx, z, *args), oracle.random_sample(z, *args)), args
 
 
 def test_large_vocabulary(ctx):
