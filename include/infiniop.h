@@ -17,7 +17,7 @@
  *   1. infiniopCreateHandle(&handle, DevAmdGpu, device_id)
  *   2. infiniopCreate<Op>Descriptor(handle, &desc, tensor descriptors...)
  *        all shape/stride/dtype checking happens here, once
- *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, Matmul, RandomSample, AddRMSNorm: always 0; MLP, Attention: their intermediates)
+ *   3. infiniopGet<Op>WorkspaceSize(desc, &bytes)        (RMSNorm, RoPE, CausalSoftmax, Matmul, AddRMSNorm: always 0; RandomSample: candidate lists, optional; MLP, Attention: their intermediates)
  *   4. infiniop<Op>(desc, ..., data pointers..., stream)
  *        enqueues on `stream` (a hipStream_t, NULL = the null stream) and
  *        returns without synchronising
@@ -358,7 +358,10 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyAttentionDescriptor(i
  * Otherwise: the first index of the maximum.  probs: 1-D F16, unit stride;
  * result: U64, one element written.  Equal logits are ordered by ascending
  * index.  topk (after clamping to the vocabulary size) may be at most 1024 in
- * the sampling form, else STATUS_BAD_PARAM.  Needs no workspace.
+ * the sampling form, else STATUS_BAD_PARAM.  The workspace (under 200 KiB, 0
+ * below 4096 logits) lets the sampling form spread its pass over the logits
+ * over the chip; a call without it is served by one workgroup, with the same
+ * result.
  * ======================================================================== */
 typedef struct RandomSampleDescriptor {
     Device device;
@@ -369,7 +372,7 @@ typedef RandomSampleDescriptor *infiniopRandomSampleDescriptor_t;
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateRandomSampleDescriptor(
     infiniopHandle_t handle, infiniopRandomSampleDescriptor_t *desc_ptr,
     infiniopTensorDescriptor_t result, infiniopTensorDescriptor_t probs);
-/* replaces include/ops/random_sample/random_sample.h:16 - always 0 bytes */
+/* replaces include/ops/random_sample/random_sample.h:16 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetRandomSampleWorkspaceSize(infiniopRandomSampleDescriptor_t desc, uint64_t *size);
 /* replaces include/ops/random_sample/random_sample.h:18-27 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRandomSample(

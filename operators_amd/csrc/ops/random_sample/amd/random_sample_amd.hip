@@ -1,17 +1,28 @@
-// RandomSample on gfx950: one workgroup of 1024 lanes does the whole call in
-// one launch, in registers and LDS, without a workspace.
+// RandomSample on gfx950.
 //
 // The reference's CPU path (src/ops/random_sample/cpu/random_sample.cc:47-171)
 // sorts the topk largest logits to the front with a selection sort, turns the
 // logits into fp16 probabilities, keeps the sorted prefix whose running sum
 // reaches topp and draws from it with random_val.  What is reproduced here is
 // that arithmetic - fp32 (x - max) / temperature, expf, division by the sum,
-// truncation to fp16, the three running fp32 sums in sorted order, every
-// comparison - not the sort: 64 KiB of logits is no work for a sort, it is a
-// latency chain, so the topk-th largest code is found by a radix select over
-// the 16-bit codes (four passes of 4 bits, per-lane counters, no atomics), the
-// at most topk candidates are compacted into LDS in index order and ranked
-// there.
+// truncation to fp16, the running fp32 sums in sorted order, every comparison -
+// not the sort.  A vocabulary is 64-300 KiB: no work for the memory system, a
+// latency chain for a sort.  So nothing is sorted:
+//  * the key of the topk-th largest logit is found by a radix select over the
+//    16-bit codes (four passes of 4 bits; counters in registers or wavefront
+//    ballots, no atomics on hot bins);
+//  * the at most topk candidates are compacted into LDS and ranked there by
+//    (logit descending, index ascending), one candidate per lane;
+//  * the first wavefront walks the sequential running sums with the
+//    probabilities in registers.
+// Two forms.  One workgroup of 1024 lanes does all of it from the logits in
+// one launch (topk_full; 79 us for 32 000 logits: one compute unit's
+// instruction rate is the limit).  With the workspace the descriptor asks for,
+// topk <= 256 and 4096 logits or more, a first launch spreads the pass over the
+// logits over up to 48 workgroups, each of which drops everything that cannot
+// be in the overall topk, and a second launch of one workgroup finishes from
+// the few hundred survivors (9.5 + 13.6 us for 32 000 logits, 11.9 + 18.6 us
+// for 151 936).
 //
 // Two things differ from the CPU path and are visible to a caller:
 //  * equal logits: the CPU's selection sort leaves equal values in an order
@@ -19,8 +30,10 @@
 //    index.  The logit at the returned index is the same either way, which is
 //    what the reference's own test accepts (operatorspy/tests/random_sample.py:
 //    `indices == ans or data[indices] == data[ans]`);
-//  * the softmax denominator is summed as a tree, not left to right, so a
-//    probability can differ in its last fp16 bit in rare cases.
+//  * the softmax denominator is summed as a tree (and, in the two-launch form,
+//    per workgroup relative to the workgroup's own maximum, then rescaled), not
+//    left to right, so a probability can differ in its last fp16 bit in rare
+//    cases.
 // NaN logits: the greedy form treats them as the CPU does (never greater than
 // anything; one in front wins); the sampling form ranks them below -Inf.
 #include "../../../devices/amd/kernel_amd.h"
@@ -184,23 +197,46 @@ __device__ __forceinline__ void rank_and_draw(TopkShared &sh, uint64_t *result, 
         }
     }
     __syncthreads();
-    if (tid == 0) {
+    // The running sums are sequential fp32 additions and have to stay so.  The
+    // first wavefront walks them with the probabilities in registers, 64 at a
+    // time, fetched by lane number: an addition and a comparison per entry,
+    // no memory access inside the chain.  Everything here is uniform over the
+    // wavefront.
+    if (tid < kWave) {
+        const auto lane_value = [](float v, uint32_t l) {
+            return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), static_cast<int>(l)));
+        };
         float run = 0.0f;
-        uint32_t end;
-        for (end = 0; end < topk; ++end) {
-            run += sh.sorted_p[end];
-            if (run >= topp) break;
+        uint32_t end = topk;
+        bool stopped = false;
+        for (uint32_t c0 = 0; c0 < topk && !stopped; c0 += kWave) {
+            const float p = c0 + tid < topk ? sh.sorted_p[c0 + tid] : 0.0f;
+            const uint32_t n = topk - c0 < static_cast<uint32_t>(kWave) ? topk - c0 : kWave;
+            for (uint32_t i = 0; i < n; ++i) {
+                run += lane_value(p, i);
+                if (run >= topp) {
+                    end = c0 + i;
+                    stopped = true;
+                    break;
+                }
+            }
         }
         // `run` is now the sum of the kept prefix in every case: the loop stops
         // on the last kept entry or runs through all topk of them
         end = end + 1 < topk ? end + 1 : topk;
         const float limit = random_val * run;
         float acc = 0.0f;
-        for (uint32_t i = 0; i < end; ++i) {
-            acc += sh.sorted_p[i];
-            if (limit < acc) {
-                result[0] = sh.sorted_i[i];
-                break;
+        bool won = false;
+        for (uint32_t c0 = 0; c0 < end && !won; c0 += kWave) {
+            const float p = c0 + tid < end ? sh.sorted_p[c0 + tid] : 0.0f;
+            const uint32_t n = end - c0 < static_cast<uint32_t>(kWave) ? end - c0 : kWave;
+            for (uint32_t i = 0; i < n; ++i) {
+                acc += lane_value(p, i);
+                if (limit < acc) {
+                    if (tid == 0) result[0] = sh.sorted_i[c0 + i];
+                    won = true;
+                    break;
+                }
             }
         }
     }
@@ -209,7 +245,7 @@ __device__ __forceinline__ void rank_and_draw(TopkShared &sh, uint64_t *result, 
 // Sampling form (random_sample.cc:47-126), everything by one workgroup from
 // the logits themselves.  topk is already clamped to [2, min(voc, KMAX)].
 template<bool VEC>
-__device__ __forceinline__ void topk_full(TopkShared &sh, uint64_t *result, const uint16_t *probs, uint32_t voc,
+__device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *result, const uint16_t *probs, uint32_t voc,
                                           float random_val, float topp, uint32_t topk, float temperature) {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t step = BS * 8u;
@@ -480,25 +516,23 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
     __shared__ uint32_t verdict[2];// [0]: lists usable, [1]: fill of sh.cand
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
 
-    if (static_cast<uint32_t>(tid) < groups) {
-        const RandomSamplePart head = heads[tid];
-        offs[tid + 1] = head.count;
-        g_key[tid] = head.key_max;
-        g_sum[tid] = head.sum;
-    }
-    __syncthreads();
-    if (tid == 0) {
-        bool ok = true;
-        uint32_t run = 0;
-        offs[0] = 0;
-        for (uint32_t w = 0; w < groups; ++w) {
-            const uint32_t c = offs[w + 1];
-            ok = ok && c <= static_cast<uint32_t>(kRandomSamplePartCap);
-            run += c;
-            offs[w + 1] = run;
+    // groups <= 48: the headers are one wavefront's work
+    if (tid < kWave) {
+        RandomSamplePart head{0, 0, 0.0f, 0};
+        if (static_cast<uint32_t>(tid) < groups) head = heads[tid];
+        const uint32_t upto = wave_scan_u32(head.count, lane);
+        const bool fits = __builtin_amdgcn_ballot_w64(head.count > static_cast<uint32_t>(kRandomSamplePartCap)) == 0;
+        if (static_cast<uint32_t>(tid) < groups) {
+            offs[tid + 1] = upto;
+            g_key[tid] = head.key_max;
+            g_sum[tid] = head.sum;
         }
-        verdict[0] = (ok && run <= static_cast<uint32_t>(CMAX) && run >= topk) ? 1u : 0u;
-        verdict[1] = 0;
+        const uint32_t all = __shfl(upto, kWave - 1);
+        if (tid == 0) {
+            offs[0] = 0;
+            verdict[0] = (fits && all <= static_cast<uint32_t>(CMAX) && all >= topk) ? 1u : 0u;
+            verdict[1] = 0;
+        }
     }
     __syncthreads();
     if (verdict[0] == 0) {// uniform over the workgroup
@@ -536,16 +570,20 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
     uint32_t prefix = 0, want = topk, ties = 0;
 #pragma unroll 1
     for (int shift = 12; shift >= 0; shift -= 4) {
+        // counting is one ballot per digit and slot; a wavefront skips the slots
+        // in which none of its entries shares the prefix any more (with a few
+        // hundred survivors most wavefronts hold one live slot or none)
         uint32_t mine = 0;
 #pragma unroll
-        for (int d = 0; d < 16; ++d) {
-            uint32_t c = 0;
+        for (int i = 0; i < PER_LANE; ++i) {
+            const bool in = (keys[i] >> (shift + 4)) == prefix;
+            if (__builtin_amdgcn_ballot_w64(in) == 0) continue;
+            const uint32_t digit = (keys[i] >> shift) & 15u;
 #pragma unroll
-            for (int i = 0; i < PER_LANE; ++i) {
-                const bool hit = (keys[i] >> (shift + 4)) == prefix && ((keys[i] >> shift) & 15u) == static_cast<uint32_t>(d);
-                c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(hit));
+            for (int d = 0; d < 16; ++d) {
+                const uint32_t c = __builtin_popcountll(__builtin_amdgcn_ballot_w64(in && digit == static_cast<uint32_t>(d)));
+                if (lane == d) mine += c;
             }
-            if (lane == d) mine = c;
         }
         if (lane < 16) sh.wave_cnt[wave * 16 + lane] = mine;
         __syncthreads();
