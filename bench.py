@@ -145,7 +145,9 @@ def make_random_sample(ctx, voc, topk, gen, name):
     f = ctypes.c_float
     ws = plan.workspace.data_ptr() if plan.workspace is not None else None
     args = (plan.desc, ws, plan.workspace_size, result.data_ptr(), logits.data_ptr(), f(0.37), f(0.9 if topk > 1 else 0.0), topk, f(0.8))
-    return Launch(name, ctx.lib.infiniopRandomSample, args, voc * 2 + 8, (plan, logits, result))
+    launch = Launch(name, ctx.lib.infiniopRandomSample, args, voc * 2 + 8, (plan, logits, result))
+    launch.latency_bound = True  # a few hundred KB at most: the time is a chain of dependent steps, not traffic
+    return launch
 
 
 def make_rearrange(ctx, tokens, heads, dtype, gen, name):
@@ -321,6 +323,8 @@ def op_entry(name, config, sets, steps, warmup, repeats):
            "us_max": round(runs[-1] * 1e6, 3), "cold_first_call_us": round(cold_us, 1), "bytes": nbytes,
            "gb_per_s": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4), "buffer_sets": len(sets),
            "calls_per_run": steps, "runs": repeats, "warmup_calls": warmup}
+    if getattr(sets[0], "latency_bound", False):
+        row.update({"bound": "latency", "frac_of_peak": None})
     if sets[0].flops:
         tflops = sets[0].flops / per_call / 1e12
         row.update({"bound": "mfma", "flops": sets[0].flops, "tflop_per_s": round(tflops, 1),

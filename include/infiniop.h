@@ -355,7 +355,8 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyAttentionDescriptor(i
  * probabilities f16(expf((x - max) / temperature) / sum over all logits), the
  * shortest prefix whose running sum reaches topp (plus one entry), and the
  * first entry of it whose running sum exceeds random_val times the prefix sum.
- * Otherwise: the first index of the maximum.  probs: 1-D F16, unit stride;
+ * Otherwise: the first index of the maximum.  probs: 1-D F16 (reference) or
+ * BF16 (extension: probabilities round to nearest even), unit stride;
  * result: U64, one element written.  Equal logits are ordered by ascending
  * index.  topk (after clamping to the vocabulary size) may be at most 1024 in
  * the sampling form, else STATUS_BAD_PARAM.  The workspace (under 200 KiB, 0

@@ -3,7 +3,9 @@
 // (src/ops/random_sample/cpu/random_sample.cc:7-33): logits of rank 1, F16;
 // result U64; a result that is neither of rank 1 nor has a first extent of 1
 // is refused.  A result without dimensions (whose first extent the reference
-// reads anyway) is taken as a scalar.  Additions: a unit stride on the logits
+// reads anyway) is taken as a scalar.  Additions: BF16 logits are accepted
+// (probabilities then round to nearest even where fp16 ones are truncated as
+// in the reference); a unit stride on the logits
 // (the reference reads them as dense without looking), at least one logit,
 // and fewer than 2^31 of them (the reference keeps the count in an int).
 #include "random_sample_amd.h"
@@ -17,7 +19,8 @@ infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampl
     if (probs->ndim != 1) {
         return STATUS_BAD_TENSOR_SHAPE;
     }
-    if (amd::elem_of(probs->dt) != amd::Elem::F16) {
+    const amd::Elem elem = amd::elem_of(probs->dt);
+    if (elem != amd::Elem::F16 && elem != amd::Elem::BF16) {
         return STATUS_BAD_TENSOR_DTYPE;
     }
     if (!amd::same_dt(result->dt, U64)) {
@@ -39,7 +42,7 @@ infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampl
         vecs = static_cast<uint32_t>(amd::ceil_div(voc, per_vec * kRandomSampleMaxGroups));
         groups = static_cast<uint32_t>(amd::ceil_div(voc, per_vec * vecs));
     }
-    auto *desc = new (std::nothrow) RandomSampleAmdDescriptor{DevAmdGpu, handle->device_id, voc, groups, vecs};
+    auto *desc = new (std::nothrow) RandomSampleAmdDescriptor{DevAmdGpu, handle->device_id, elem, voc, groups, vecs};
     if (desc == nullptr) {
         return STATUS_MEMORY_NOT_ALLOCATED;
     }

@@ -32,6 +32,7 @@ struct RandomSamplePart {
 struct RandomSampleAmdDescriptor {
     Device device;
     int device_id;
+    amd::Elem elem; // F16 or BF16
     uint32_t voc;   // number of logits
     uint32_t groups;// workgroups of the first launch of the two-launch form; 0: never used
     uint32_t vecs;  // 8-element vectors per lane in them

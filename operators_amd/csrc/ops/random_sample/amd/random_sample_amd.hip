@@ -48,16 +48,24 @@ constexpr int WAVES = BS / kWave;
 constexpr int KMAX = kRandomSampleMaxTopk;
 constexpr uint32_t kNoKey = 0xFFFFFFFFu;// marks a slot past the end of the logits
 
-// Order-preserving 16-bit key of an fp16 code: a greater value has a greater
-// key, -0 and +0 share one, NaN is the smallest.
+// Code of +Inf: everything above it (sign aside) is a NaN.
+template<typename T>
+constexpr uint32_t kInfCode = 0x7C00u;
+template<>
+constexpr uint32_t kInfCode<BF16Rne> = 0x7F80u;
+
+// Order-preserving 16-bit key of an fp16 or bf16 code (both are sign-magnitude):
+// a greater value has a greater key, -0 and +0 share one, NaN is the smallest.
+template<typename T>
 __device__ __forceinline__ uint32_t key_of(uint32_t h) {
-    if ((h & 0x7FFFu) > 0x7C00u) return 0u;
+    if ((h & 0x7FFFu) > kInfCode<T>) return 0u;
     if (h == 0x8000u) h = 0u;
     return (h & 0x8000u) ? (h ^ 0xFFFFu) : (h | 0x8000u);
 }
+template<typename T>
 __device__ __forceinline__ float value_of_key(uint32_t k) {
     const uint32_t h = (k & 0x8000u) ? (k & 0x7FFFu) : (k ^ 0xFFFFu);
-    return F16Ref::one(static_cast<uint16_t>(h));
+    return T::one(static_cast<uint16_t>(h));
 }
 
 // The eight codes starting at element `base` (a multiple of 8): one 128-bit
@@ -115,7 +123,7 @@ __device__ __forceinline__ uint32_t wave_scan_u32(uint32_t v, int lane) {
 
 // Greedy form (random_sample.cc:127-148): the first index holding the maximum,
 // where NaN is never greater than anything and a NaN in front is never beaten.
-template<bool VEC>
+template<typename T, bool VEC>
 __global__ __launch_bounds__(BS) void random_sample_greedy(uint64_t *result, const uint16_t *probs, uint32_t voc) {
     __shared__ unsigned long long best_of[WAVES];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -127,7 +135,7 @@ __global__ __launch_bounds__(BS) void random_sample_greedy(uint64_t *result, con
         for (int e = 0; e < 8; ++e) {
             if (e < n) {
                 // greater key first, then the lower index
-                const unsigned long long c = (static_cast<unsigned long long>(key_of(h[e])) << 32) | (0xFFFFFFFFu - (base + e));
+                const unsigned long long c = (static_cast<unsigned long long>(key_of<T>(h[e])) << 32) | (0xFFFFFFFFu - (base + e));
                 best = c > best ? c : best;
             }
         }
@@ -139,7 +147,7 @@ __global__ __launch_bounds__(BS) void random_sample_greedy(uint64_t *result, con
 #pragma unroll
         for (int w = 1; w < WAVES; ++w) best = best_of[w] > best ? best_of[w] : best;
         const uint32_t first = probs[0];
-        const bool first_is_nan = (first & 0x7FFFu) > 0x7C00u;
+        const bool first_is_nan = (first & 0x7FFFu) > kInfCode<T>;
         result[0] = first_is_nan ? 0ull : static_cast<unsigned long long>(0xFFFFFFFFu - static_cast<uint32_t>(best));
     }
 }
@@ -182,6 +190,7 @@ __device__ __forceinline__ void choose_digit(const uint32_t *digit_cnt, uint32_t
 // index), turn the first topk of them into fp16 probabilities and walk the
 // running sums of random_sample.cc:97-125 in their order.  Ends with the
 // result written, or left alone when no running sum exceeds the limit.
+template<typename T>
 __device__ __forceinline__ void rank_and_draw(TopkShared &sh, uint64_t *result, uint32_t count, uint32_t topk, float top,
                                               float total, float random_val, float topp, float temperature) {
     const int tid = threadIdx.x;
@@ -190,9 +199,9 @@ __device__ __forceinline__ void rank_and_draw(TopkShared &sh, uint64_t *result, 
         uint32_t rank = 0;
         for (uint32_t j = 0; j < count; ++j) rank += sh.cand[j] > mine ? 1u : 0u;
         if (rank < topk) {
-            const float x = value_of_key(static_cast<uint32_t>(mine >> 32));
+            const float x = value_of_key<T>(static_cast<uint32_t>(mine >> 32));
             const float p = expf((x - top) / temperature) / total;
-            sh.sorted_p[rank] = F16Ref::one(F16Ref::narrow1(p));
+            sh.sorted_p[rank] = T::one(T::narrow1(p));
             sh.sorted_i[rank] = 0xFFFFFFFFu - static_cast<uint32_t>(mine);
         }
     }
@@ -244,7 +253,7 @@ __device__ __forceinline__ void rank_and_draw(TopkShared &sh, uint64_t *result, 
 
 // Sampling form (random_sample.cc:47-126), everything by one workgroup from
 // the logits themselves.  topk is already clamped to [2, min(voc, KMAX)].
-template<bool VEC>
+template<typename T, bool VEC>
 __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *result, const uint16_t *probs, uint32_t voc,
                                           float random_val, float topp, uint32_t topk, float temperature) {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -264,7 +273,7 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
             const int n = load_codes<VEC>(probs, voc, base, h);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const uint32_t k = e < n ? key_of(h[e]) : kNoKey;
+                const uint32_t k = e < n ? key_of<T>(h[e]) : kNoKey;
                 if (shift == 12 && e < n) key_max = k > key_max ? k : key_max;
                 const bool in = (k >> (shift + 4)) == prefix;// never true for kNoKey: prefix < 2^12
                 const uint32_t digit = (k >> shift) & 15u;
@@ -298,7 +307,7 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
     const uint32_t n_greater = topk - want; // elements with a greater key
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) key_max = sh.wave_key[w] > key_max ? sh.wave_key[w] : key_max;
-    const float top = value_of_key(key_max);
+    const float top = value_of_key<T>(key_max);
 
     // ---- compaction in index order, and the softmax denominator ------------
     float part = 0.0f;
@@ -313,9 +322,9 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
         uint32_t c_gt = 0, c_eq = 0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            k[e] = e < n ? key_of(h[e]) : kNoKey;
+            k[e] = e < n ? key_of<T>(h[e]) : kNoKey;
             if (e < n) {
-                part += expf((F16Ref::one(static_cast<uint16_t>(h[e])) - top) / temperature);
+                part += expf((T::one(static_cast<uint16_t>(h[e])) - top) / temperature);
                 c_gt += k[e] > key_k ? 1u : 0u;
                 c_eq += k[e] == key_k ? 1u : 0u;
             }
@@ -352,14 +361,14 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
     float total = 0.0f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) total += sh.sum_slots[w];
-    rank_and_draw(sh, result, topk, topk, top, total, random_val, topp, temperature);
+    rank_and_draw<T>(sh, result, topk, topk, top, total, random_val, topp, temperature);
 }
 
-template<bool VEC>
+template<typename T, bool VEC>
 __global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const uint16_t *probs, uint32_t voc,
                                                           float random_val, float topp, uint32_t topk, float temperature) {
     __shared__ TopkShared sh;
-    topk_full<VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
+    topk_full<T, VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
 }
 
 // ---- the same in two launches, the first spread over the chip ---------------
@@ -377,7 +386,7 @@ __global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const
 // overflows - very many equal logits, topk close to 256 - it does the whole
 // job itself from the logits (topk_full), so the answer never depends on the
 // shortcut working.
-template<bool VEC>
+template<typename T, bool VEC>
 __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(RandomSamplePart *heads, unsigned long long *lists,
                                                                                   const uint16_t *probs, uint32_t voc,
                                                                                   uint32_t vecs, uint32_t topk, float temperature) {
@@ -402,7 +411,7 @@ __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(
             has = true;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const uint32_t k = key_of(h[e]);
+                const uint32_t k = key_of<T>(h[e]);
                 if (e < n) lane_max = k > lane_max ? k : lane_max;
             }
         }
@@ -449,7 +458,7 @@ __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(
     uint32_t key_max = 0;
 #pragma unroll
     for (int w = 0; w < PW; ++w) key_max = wave_key[w] > key_max ? wave_key[w] : key_max;
-    const float top = value_of_key(key_max);
+    const float top = value_of_key<T>(key_max);
 
     // survivors to the workspace, and the partial denominator
     float part = 0.0f;
@@ -463,9 +472,9 @@ __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(
             n = load_codes<VEC>(probs, voc, base, h);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                k[e] = e < n ? key_of(h[e]) : kNoKey;
+                k[e] = e < n ? key_of<T>(h[e]) : kNoKey;
                 if (e < n) {
-                    const float x = F16Ref::one(static_cast<uint16_t>(h[e]));
+                    const float x = T::one(static_cast<uint16_t>(h[e]));
                     // the maximum itself counts as expf(0) also when it is infinite
                     part += k[e] == key_max ? 1.0f : expf((x - top) / temperature);
                     c += k[e] >= bound ? 1u : 0u;
@@ -502,7 +511,7 @@ __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(
     }
 }
 
-template<bool VEC>
+template<typename T, bool VEC>
 __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, const uint16_t *probs, uint32_t voc, float random_val,
                                                            float topp, uint32_t topk, float temperature,
                                                            const RandomSamplePart *heads, const unsigned long long *lists,
@@ -536,7 +545,7 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
     }
     __syncthreads();
     if (verdict[0] == 0) {// uniform over the workgroup
-        topk_full<VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
+        topk_full<T, VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
         return;
     }
     const uint32_t count = offs[groups];
@@ -544,10 +553,10 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
     // the overall maximum and the denominator rescaled to it, in a fixed order
     uint32_t key_max = 0;
     for (uint32_t w = 0; w < groups; ++w) key_max = g_key[w] > key_max ? g_key[w] : key_max;
-    const float top = value_of_key(key_max);
+    const float top = value_of_key<T>(key_max);
     float part = 0.0f;
     if (static_cast<uint32_t>(tid) < groups) {
-        part = g_sum[tid] * expf((value_of_key(g_key[tid]) - top) / temperature);
+        part = g_sum[tid] * expf((value_of_key<T>(g_key[tid]) - top) / temperature);
     }
     part = wave_sum(part);// groups <= 64: all of them sit in the first wavefront
     if (tid == 0) sh.sum_slots[0] = part;
@@ -601,7 +610,7 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
     const uint32_t kept = topk - want + ties;
     if (kept > static_cast<uint32_t>(KMAX)) {// uniform: more equal logits at the boundary than LDS ranks
         __syncthreads();
-        topk_full<VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
+        topk_full<T, VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
         return;
     }
 #pragma unroll
@@ -609,7 +618,32 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
         if (keys[i] != kNoKey && keys[i] >= prefix) sh.cand[atomicAdd(&verdict[1], 1u)] = pool[tid + i * BS];
     }
     __syncthreads();
-    rank_and_draw(sh, result, kept, topk, top, total, random_val, topp, temperature);
+    rank_and_draw<T>(sh, result, kept, topk, top, total, random_val, topp, temperature);
+}
+
+struct RandomSampleCall {
+    uint64_t *result;
+    const uint16_t *probs;
+    uint32_t voc;
+    float random_val, topp;
+    uint32_t topk;
+    float temperature;
+    RandomSamplePart *heads;// the workspace, when the two-launch form is to be used
+    uint32_t groups, vecs;
+};
+
+// form 2: sampling, 1: greedy, 0: nothing to launch
+template<typename T, bool VEC>
+void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
+    if (form == 1) {
+        random_sample_greedy<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc);
+    } else if (form == 2 && c.heads != nullptr) {
+        auto *lists = reinterpret_cast<unsigned long long *>(c.heads + kRandomSampleMaxGroups);
+        random_sample_partial<T, VEC><<<c.groups, kRandomSamplePartLanes, 0, s>>>(c.heads, lists, c.probs, c.voc, c.vecs, c.topk, c.temperature);
+        random_sample_merge<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature, c.heads, lists, c.groups);
+    } else if (form == 2) {
+        random_sample_topk<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature);
+    }
 }
 
 }// namespace
@@ -634,38 +668,21 @@ infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspa
     }
     AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    auto *out = static_cast<uint64_t *>(result);
-    auto *in = static_cast<const uint16_t *>(probs);
+    const bool split = sample && k >= 2 && desc->groups != 0 && k <= static_cast<uint32_t>(kRandomSamplePartTopk) &&
+                       workspace != nullptr && workspace_size >= amdRandomSampleWorkspaceBytes(*desc) &&
+                       (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0;
+    const RandomSampleCall call{static_cast<uint64_t *>(result), static_cast<const uint16_t *>(probs), desc->voc, random_val, topp, k,
+                                temperature, split ? static_cast<RandomSamplePart *>(workspace) : nullptr, desc->groups, desc->vecs};
+    // greedy unless sampling; a vocabulary of one logit has one candidate of
+    // probability 1, which wins unless random_val >= 1, as in the reference's loops
+    const int form = (sample && k >= 2) ? 2 : (!sample || random_val < 1.0f) ? 1 : 0;
     const bool vec = amd::aligned16(probs);
-    const uint32_t voc = desc->voc;
-    if (sample && k >= 2) {
-        const bool split = desc->groups != 0 && k <= static_cast<uint32_t>(kRandomSamplePartTopk) && workspace != nullptr &&
-                           workspace_size >= amdRandomSampleWorkspaceBytes(*desc) && (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0;
-        if (split) {
-            auto *heads = static_cast<RandomSamplePart *>(workspace);
-            auto *lists = reinterpret_cast<unsigned long long *>(heads + kRandomSampleMaxGroups);
-            if (vec) {
-                random_sample_partial<true><<<desc->groups, kRandomSamplePartLanes, 0, s>>>(heads, lists, in, voc, desc->vecs, k, temperature);
-                random_sample_merge<true><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature, heads, lists, desc->groups);
-            } else {
-                random_sample_partial<false><<<desc->groups, kRandomSamplePartLanes, 0, s>>>(heads, lists, in, voc, desc->vecs, k, temperature);
-                random_sample_merge<false><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature, heads, lists, desc->groups);
-            }
-        } else if (vec) {
-            random_sample_topk<true><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature);
-        } else {
-            random_sample_topk<false><<<1, BS, 0, s>>>(out, in, voc, random_val, topp, k, temperature);
-        }
-    } else if (sample) {
-        // a vocabulary of one logit: the only candidate has probability 1 and
-        // wins unless random_val >= 1, as in the reference's loops
-        if (random_val < 1.0f) {
-            if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, voc);
-            else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, voc);
-        }
+    if (desc->elem == amd::Elem::F16) {
+        if (vec) launch_random_sample<amd::F16Ref, true>(call, form, s);
+        else launch_random_sample<amd::F16Ref, false>(call, form, s);
     } else {
-        if (vec) random_sample_greedy<true><<<1, BS, 0, s>>>(out, in, voc);
-        else random_sample_greedy<false><<<1, BS, 0, s>>>(out, in, voc);
+        if (vec) launch_random_sample<amd::BF16Rne, true>(call, form, s);
+        else launch_random_sample<amd::BF16Rne, false>(call, form, s);
     }
     AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
     return STATUS_SUCCESS;

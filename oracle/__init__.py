@@ -83,8 +83,8 @@ def lib():
         L.oracle_rearrange_check.argtypes, L.oracle_rearrange_check.restype = [tp, tp], ctypes.c_int
         L.oracle_rearrange.argtypes = [u32, u64, vp, vp, vp, vp, vp]
         L.oracle_rearrange.restype = ctypes.c_int
-        L.oracle_random_sample_check.argtypes, L.oracle_random_sample_check.restype = [tp, tp], ctypes.c_int
-        L.oracle_random_sample.argtypes = [vp, vp, ctypes.c_int, f32, f32, ctypes.c_int, f32, vp, vp]
+        L.oracle_random_sample_check.argtypes, L.oracle_random_sample_check.restype = [tp, tp, ctypes.c_int], ctypes.c_int
+        L.oracle_random_sample.argtypes = [u32, vp, vp, ctypes.c_int, f32, f32, ctypes.c_int, f32, vp, vp]
         L.oracle_random_sample.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -343,18 +343,20 @@ def rearrange(dst, src):
     return dst
 
 
-def random_sample_check(result, probs):
-    return lib().oracle_random_sample_check(result.ref(), probs.ref())
+def random_sample_check(result, probs, allow_bf16=False):
+    return lib().oracle_random_sample_check(result.ref(), probs.ref(), int(allow_bf16))
 
 
-def random_sample(probs, random_val, topp, topk, temperature):
-    """probs: 1-D contiguous array of fp16 codes.  Returns the chosen index, or
+def random_sample(probs, random_val, topp, topk, temperature, dtype="f16"):
+    """probs: 1-D contiguous array of fp16 (or, as an extension, bf16) codes.  Returns the chosen index, or
     None when the reference's CPU path would leave the result unwritten."""
     probs = np.ascontiguousarray(probs, dtype=np.uint16)
     voc = probs.shape[0]
     result = np.full(1, 0xFFFFFFFFFFFFFFFF, dtype=np.uint64)
     logits = np.empty(voc, dtype=np.uint16)
     order = np.empty(voc, dtype=np.uint64)
-    wrote = lib().oracle_random_sample(_ptr(result), _ptr(probs), voc, random_val, topp, topk, temperature,
+    wrote = lib().oracle_random_sample(DT[dtype], _ptr(result), _ptr(probs), voc, random_val, topp, topk, temperature,
                                        _ptr(logits), _ptr(order))
+    if wrote < 0:
+        raise RuntimeError(f"oracle_random_sample status {-wrote}")
     return int(result[0]) if wrote else None

@@ -35,6 +35,11 @@
  *       permutation matrices.  The MLP is the reference's composition of
  *       matmul, swiglu and matmul (src/ops/mlp/operator.cc:22-122), checked
  *       against the compiled reference's MLP bit for bit.
+ *   oracle_random_sample (fp16)              pinned  - golden indices written by
+ *       the compiled reference (its own nine test cases, ties, special
+ *       values), the compiled reference itself on fresh inputs, an independent
+ *       argsort/float64 model for tie-free logits, closed forms (tiny topp,
+ *       random_val 0 and 1, flat distributions, greedy = argmax).
  *   bf16 variants of the operators           PARITY UNPINNED by the reference:
  *       no reference back end accepts bf16 for these operators.  The bf16
  *       arithmetic here is this project's extension (exact widening, the same
@@ -658,11 +663,11 @@ ORACLE_API int oracle_matmul(uint32_t dt, uint64_t batch, uint64_t m, uint64_t n
  * only when it is neither of rank 1 nor has a first extent of 1.  A result
  * with no dimensions (whose first extent the reference reads anyway) counts
  * as a scalar here and passes. */
-ORACLE_API int oracle_random_sample_check(const oracle_tensor *result, const oracle_tensor *probs) {
+ORACLE_API int oracle_random_sample_check(const oracle_tensor *result, const oracle_tensor *probs, int allow_bf16) {
     if (probs->ndim != 1) {
         return ST_BAD_TENSOR_SHAPE;
     }
-    if (probs->dt != DT_F16) {
+    if (probs->dt != DT_F16 && !(allow_bf16 && probs->dt == DT_BF16)) {
         return ST_BAD_TENSOR_DTYPE;
     }
     if (result->dt != DT_U64) {
@@ -688,16 +693,22 @@ ORACLE_API int oracle_random_sample_check(const oracle_tensor *result, const ora
  * over the array in its permuted order; a running fp32 sum over the first
  * topk entries finds where it reaches topp; random_val is scaled by the sum
  * of the kept prefix and the first entry whose running sum exceeds it wins.
- * Greedy form (otherwise): the first index holding the maximum. */
-ORACLE_API int oracle_random_sample(uint64_t *result, const uint16_t *probs, int voc, float random_val, float topp,
+ * Greedy form (otherwise): the first index holding the maximum.
+ * dt = BF16 is this project's extension (the reference accepts F16 only):
+ * exact widening, the same arithmetic, round-to-nearest-even where the
+ * reference truncates to fp16.  PARITY UNPINNED by the reference. */
+ORACLE_API int oracle_random_sample(uint32_t dt, uint64_t *result, const uint16_t *probs, int voc, float random_val, float topp,
                                     int topk, float temperature, uint16_t *logits, uint64_t *order) {
+    if (dt != DT_F16 && dt != DT_BF16) {
+        return -ST_BAD_TENSOR_DTYPE;
+    }
     memcpy(logits, probs, (size_t) voc * sizeof(uint16_t));
     if (!(topp > 0 && topk > 1)) {
-        float m = oracle_f16_to_f32(logits[0]);
+        float m = load16(dt, logits + 0);
         int index = 0;
         for (int j = 1; j < voc; ++j) {
-            if (m < oracle_f16_to_f32(logits[j])) {
-                m = oracle_f16_to_f32(logits[j]);
+            if (m < load16(dt, logits + j)) {
+                m = load16(dt, logits + j);
                 index = j;
             }
         }
@@ -712,28 +723,28 @@ ORACLE_API int oracle_random_sample(uint64_t *result, const uint16_t *probs, int
     }
     for (int i = 0; i < topk; ++i) {
         for (int j = i + 1; j < voc; ++j) {
-            if (oracle_f16_to_f32(logits[i]) < oracle_f16_to_f32(logits[j])) {
-                const float held = oracle_f16_to_f32(logits[i]);
+            if (load16(dt, logits + i) < load16(dt, logits + j)) {
+                const float held = load16(dt, logits + i);
                 logits[i] = logits[j];
-                logits[j] = oracle_f32_to_f16(held);
+                store16(dt, logits + j, held);
                 const int t = (int) order[i];
                 order[i] = order[j];
                 order[j] = (uint64_t) t;
             }
         }
     }
-    const float top = oracle_f16_to_f32(logits[0]);
+    const float top = load16(dt, logits + 0);
     float total = 0.0f;
     for (int i = 0; i < voc; ++i) {
-        total += expf((oracle_f16_to_f32(logits[i]) - top) / temperature);
+        total += expf((load16(dt, logits + i) - top) / temperature);
     }
     for (int i = 0; i < voc; ++i) {
-        logits[i] = oracle_f32_to_f16(expf((oracle_f16_to_f32(logits[i]) - top) / temperature) / total);
+        store16(dt, logits + i, expf((load16(dt, logits + i) - top) / temperature) / total);
     }
     float run = 0.0f;
     int end;
     for (end = 0; end < topk; ++end) {
-        run += oracle_f16_to_f32(logits[end]);
+        run += load16(dt, logits + end);
         if (run >= topp) {
             break;
         }
@@ -745,12 +756,12 @@ ORACLE_API int oracle_random_sample(uint64_t *result, const uint16_t *probs, int
     }
     float kept = 0.0f;
     for (int i = 0; i < end; ++i) {
-        kept += oracle_f16_to_f32(logits[i]);
+        kept += load16(dt, logits + i);
     }
     random_val *= kept;
     kept = 0.0f;
     for (int i = 0; i < end; ++i) {
-        kept += oracle_f16_to_f32(logits[i]);
+        kept += load16(dt, logits + i);
         if (random_val < kept) {
             result[0] = order[i];
             return 1;

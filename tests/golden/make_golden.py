@@ -409,7 +409,7 @@ def status_cases():
     rec("random_sample", [T("u64", (1,)), T("f32", (512,))])
     rec("random_sample", [T("i64", (1,)), T("f16", (512,))])
     rec("random_sample", [T("i64", (2, 3)), T("f16", (512,))])       # type is reported before shape
-    rec("random_sample", [T("u64", (1,)), T("bf16", (512,))])
+    rec("random_sample", [T("u64", (1,)), T("bf16", (512,))], bf16_extension=True)
     return cases
 
 

@@ -19,26 +19,26 @@ CASES = golden_json()["random_sample_cases"]
 SENTINEL = -12345
 
 
-def gpu_sample(ctx, codes, rv, topp, topk, temp, offset=0):
+def gpu_sample(ctx, codes, rv, topp, topk, temp, offset=0, dt="f16"):
     """offset (elements) places the logits at an address that is not 16-byte
     aligned.  Every case runs twice: with the workspace the library asks for
     (vocabularies of 4096 and more then take the two-launch form) and without
     it (one workgroup); the two must give the same index."""
-    with_ws = gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, True)
-    without = gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, False)
+    with_ws = gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, True, dt)
+    without = gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, False, dt)
     assert with_ws == without, ("with workspace", with_ws, "without", without)
     return with_ws
 
 
-def gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, use_workspace):
+def gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, use_workspace, dt="f16"):
     import torch
 
     codes = np.ascontiguousarray(codes, np.uint16)
     if offset:
-        buf = to_torch(np.concatenate([np.zeros(offset, np.uint16), codes]), "f16")
+        buf = to_torch(np.concatenate([np.zeros(offset, np.uint16), codes]), dt)
         probs = buf[offset:]
     else:
-        probs = to_torch(codes, "f16")
+        probs = to_torch(codes, dt)
     result = torch.full((1,), SENTINEL, dtype=torch.int64, device="cuda")  # the bits of a uint64
     view = result.view(torch.uint64)
     ctx.random_sample(view, probs, rv, topp, topk, temp, use_workspace=use_workspace)
@@ -47,12 +47,12 @@ def gpu_sample_once(ctx, codes, rv, topp, topk, temp, offset, use_workspace):
     return None if got == SENTINEL else got
 
 
-def same_choice(codes, got, want):
+def same_choice(codes, got, want, dt="f16"):
     if got == want:
         return True
     if got is None or want is None:
         return False
-    v = np.asarray(codes, np.uint16).view(np.float16)
+    v = oracle.decode(np.asarray(codes, np.uint16), dt)
     return 0 <= got < v.size and float(v[got]) == float(v[want])
 
 
@@ -195,6 +195,30 @@ def test_lists_that_overflow_fall_back_to_the_full_path(ctx):
     for topk in (20, 40, 100):
         args = (0.5, 0.9, topk, 1.0)
         assert same_choice(z, gpu_sample(ctx, z, *args), oracle.random_sample(z, *args)), args
+
+
+def test_bf16_extension_against_oracle(ctx):
+    """bf16 logits (accepted here, refused by the reference): against the
+    oracle's bf16 form - same arithmetic, probabilities rounded to nearest
+    even.  Parity unpinned by the reference."""
+    rng = np.random.default_rng(31)
+    bad = []
+    for trial in range(60):
+        voc = int(rng.choice([3, 100, 4096, 5000, 32000, 128256]))
+        x = oracle.f32_to_bf16((rng.standard_normal(voc, dtype=np.float32) * (3.0 if trial % 2 else 0.7)).astype(np.float32))
+        if trial % 3 == 0:  # distinct codes only
+            x = np.unique(x)
+            x = x[(x & 0x7FFF) != 0]
+            rng.shuffle(x)
+            voc = x.size
+        args = (float(rng.random()), float(rng.choice([0.0, 0.5, 0.9, 1.0])), int(rng.choice([1, 2, 8, 50, 256, 600])), float(rng.choice([0.5, 1.0, 2.0])))
+        want = oracle.random_sample(x, *args, dtype="bf16")
+        got = gpu_sample(ctx, x, *args, dt="bf16")
+        if not same_choice(x, got, want, "bf16") or (trial % 3 == 0 and got != want):
+            bad.append((trial, voc, args, got, want))
+    assert not bad, bad[:5]
+    # the codes are read as bf16, not as fp16: 1.0, 2.0, then fp16's 1.0 (bf16 0.0078125)
+    assert gpu_sample(ctx, np.array([0x3F80, 0x4000, 0x3C00], np.uint16), 0.5, 0.0, 1, 1.0, dt="bf16") == 1
 
 
 def test_large_vocabulary(ctx):

@@ -37,6 +37,8 @@ def test_oracle_checks_reproduce_reference_status(i):
         return
     elif case["op"] == "random_sample":
         assert oracle.random_sample_check(*specs) == case["status"], case
+        if case.get("bf16_extension"):
+            assert oracle.random_sample_check(*specs, allow_bf16=True) == 0
         return
     elif case["op"] == "causal_softmax":
         st = oracle.causal_softmax_check(specs[0], allow_bf16=False, unit_inner=False)
