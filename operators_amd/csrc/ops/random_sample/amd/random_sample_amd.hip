@@ -90,10 +90,18 @@ __device__ __forceinline__ int load_codes(const uint16_t *p, uint32_t voc, uint3
     return n;
 }
 
+// Sum over the 64 lanes with DPP adds (the lane pattern of amd::wave_sum):
+// four steps inside each row of 16 lanes, then row broadcasts 15 and 31; the
+// total lands in lane 63 and is read back to every lane through an SGPR.
 __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
+    int x = static_cast<int>(v);
+    x += __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, false); // quad_perm [1,0,3,2]
+    x += __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, false); // quad_perm [2,3,0,1]
+    x += __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, false);// row_half_mirror
+    x += __builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, false);// row_mirror
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);// row_bcast:15 -> rows 1, 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);// row_bcast:31 -> rows 2, 3
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(x, 63));
 }
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 #pragma unroll
@@ -154,7 +162,7 @@ __global__ __launch_bounds__(BS) void random_sample_greedy(uint64_t *result, con
 
 // LDS of the sampling kernels.
 struct TopkShared {
-    uint32_t wave_cnt[WAVES * 16];   // per-wavefront digit counts of one select pass
+    uint32_t wave_cnt[2][WAVES * 16];// per-wavefront digit counts of one select pass (two sets, used in turn)
     uint32_t digit_cnt[16];          // their totals
     uint32_t wave_key[WAVES];        // per-wavefront maximum key
     uint32_t scan_tot[2][WAVES][2];  // per-wavefront (greater, equal) counts of one compaction step
@@ -206,46 +214,51 @@ __device__ __forceinline__ void rank_and_draw(TopkShared &sh, uint64_t *result, 
         }
     }
     __syncthreads();
-    // The running sums are sequential fp32 additions and have to stay so.  The
-    // first wavefront walks them with the probabilities in registers, 64 at a
-    // time, fetched by lane number: an addition and a comparison per entry,
-    // no memory access inside the chain.  Everything here is uniform over the
-    // wavefront.
+    // The reference walks the sorted probabilities three times with a running
+    // fp32 sum that starts from zero each time: to find where it reaches topp,
+    // to total the kept prefix, to find where it exceeds random_val times that
+    // total.  All three see the same sequence of partial sums, and those have
+    // to be formed by sequential additions to round as the reference's do.
+    // So the first wavefront forms them once, 64 at a time, in a branch-free
+    // chain - the addends come out of a register by constant lane number, lane
+    // i keeps the i-th partial sum - and takes the two decisions with ballots
+    // over the stored sums.  (A loop that adds, compares and branches per
+    // entry costs 47 ns per entry here: 4.7 us for topk = 50.)
     if (tid < kWave) {
-        const auto lane_value = [](float v, uint32_t l) {
-            return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), static_cast<int>(l)));
-        };
-        float run = 0.0f;
+        float run = 0.0f, kept = 0.0f;
         uint32_t end = topk;
         bool stopped = false;
         for (uint32_t c0 = 0; c0 < topk && !stopped; c0 += kWave) {
-            const float p = c0 + tid < topk ? sh.sorted_p[c0 + tid] : 0.0f;
-            const uint32_t n = topk - c0 < static_cast<uint32_t>(kWave) ? topk - c0 : kWave;
-            for (uint32_t i = 0; i < n; ++i) {
-                run += lane_value(p, i);
-                if (run >= topp) {
-                    end = c0 + i;
-                    stopped = true;
-                    break;
-                }
+            const bool live = c0 + tid < topk;
+            const float p = live ? sh.sorted_p[c0 + tid] : 0.0f;
+            float mine = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kWave; ++i) {
+                run += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, p), i));
+                mine = tid == i ? run : mine;
+            }
+            if (live) sh.sorted_p[c0 + tid] = mine;// from here on the array holds the partial sums
+            const unsigned long long reached = __builtin_amdgcn_ballot_w64(live && mine >= topp);
+            if (reached != 0) {
+                const int at = __builtin_ctzll(reached);
+                end = c0 + at;
+                kept = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), at));
+                stopped = true;
             }
         }
-        // `run` is now the sum of the kept prefix in every case: the loop stops
-        // on the last kept entry or runs through all topk of them
+        // the sum of the kept prefix: the partial sum at the entry where the
+        // walk stopped (that entry is the last one kept, or the last of all),
+        // or the sum of all topk entries when it never stopped
+        if (!stopped) kept = run;
         end = end + 1 < topk ? end + 1 : topk;
-        const float limit = random_val * run;
-        float acc = 0.0f;
-        bool won = false;
-        for (uint32_t c0 = 0; c0 < end && !won; c0 += kWave) {
-            const float p = c0 + tid < end ? sh.sorted_p[c0 + tid] : 0.0f;
-            const uint32_t n = end - c0 < static_cast<uint32_t>(kWave) ? end - c0 : kWave;
-            for (uint32_t i = 0; i < n; ++i) {
-                acc += lane_value(p, i);
-                if (limit < acc) {
-                    if (tid == 0) result[0] = sh.sorted_i[c0 + i];
-                    won = true;
-                    break;
-                }
+        const float limit = random_val * kept;
+        for (uint32_t c0 = 0; c0 < end; c0 += kWave) {
+            const bool live = c0 + tid < end;
+            const float upto = live ? sh.sorted_p[c0 + tid] : 0.0f;
+            const unsigned long long above = __builtin_amdgcn_ballot_w64(live && limit < upto);
+            if (above != 0) {
+                if (tid == 0) result[0] = sh.sorted_i[c0 + __builtin_ctzll(above)];
+                break;
             }
         }
     }
@@ -287,7 +300,7 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
             const uint32_t t = wave_sum_u32(cnt[d]);
             if (lane == d) mine = t;
         }
-        if (lane < 16) sh.wave_cnt[wave * 16 + lane] = mine;
+        if (lane < 16) sh.wave_cnt[0][wave * 16 + lane] = mine;
         if (shift == 12) {
             const uint32_t m = wave_max_u32(key_max);
             if (lane == 0) sh.wave_key[wave] = m;
@@ -296,7 +309,7 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
         if (tid < 16) {
             uint32_t t = 0;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) t += sh.wave_cnt[w * 16 + tid];
+            for (int w = 0; w < WAVES; ++w) t += sh.wave_cnt[0][w * 16 + tid];
             sh.digit_cnt[tid] = t;
         }
         __syncthreads();
@@ -391,16 +404,14 @@ __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(
                                                                                   const uint16_t *probs, uint32_t voc,
                                                                                   uint32_t vecs, uint32_t topk, float temperature) {
     constexpr int PBS = kRandomSamplePartLanes, PW = PBS / kWave;
-    __shared__ uint32_t wave_cnt[PW * 16];
-    __shared__ uint32_t digit_cnt[16];
-    __shared__ uint32_t wave_key[PW];
+    __shared__ __attribute__((aligned(16))) uint32_t lane_rank_key[PBS];
+    __shared__ uint32_t bound_slot, max_slot, data_lanes;
     __shared__ float sum_slots[PW];
     __shared__ uint32_t fill;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t start = blockIdx.x * (PBS * 8u * vecs);
-    if (tid == 0) fill = 0;
 
-    // lane maxima and the workgroup's maximum
+    // lane maxima
     uint32_t lane_max = 0;
     bool has = false;
     for (uint32_t v = 0; v < vecs; ++v) {
@@ -416,48 +427,39 @@ __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(
             }
         }
     }
+    // The topk-th largest lane maximum, by rank: every lane reads all 256
+    // (one LDS round trip, 64 four-word reads) and counts those that beat its
+    // own; the lane number breaks ties so the ranks are a permutation, and the
+    // lane of rank topk - 1 holds the bound.  Lanes without data rank last;
+    // with fewer than topk lanes holding data everything is kept.  (A
+    // four-pass radix select over the 256 values, two barriers a pass, took
+    // 3.9 us of this kernel's 7.5.)
+    const uint32_t my_rank_key = has ? ((lane_max << 8) | (255u - static_cast<uint32_t>(tid))) + 1u : 0u;
+    lane_rank_key[tid] = my_rank_key;
+    if (tid == 0) {
+        fill = 0;
+        bound_slot = 0;
+        data_lanes = PBS;
+    }
+    __syncthreads();
+    uint32_t rank = 0;
     {
-        const uint32_t m = wave_max_u32(lane_max);
-        if (lane == 0) wave_key[wave] = m;
+        const u32x4 *all = reinterpret_cast<const u32x4 *>(lane_rank_key);
+#pragma unroll 8
+        for (int j = 0; j < PBS / 4; ++j) {
+            const u32x4 q = all[j];
+            rank += (q.x > my_rank_key ? 1u : 0u) + (q.y > my_rank_key ? 1u : 0u) + (q.z > my_rank_key ? 1u : 0u) + (q.w > my_rank_key ? 1u : 0u);
+        }
     }
-    // the topk-th largest lane maximum (0 = keep everything, when fewer than topk lanes hold data)
-    uint32_t prefix = 0, want = topk;
-    const uint32_t mine_key = has ? lane_max : kNoKey;
-    bool keep_all = false;
-#pragma unroll 1
-    for (int shift = 12; shift >= 0; shift -= 4) {
-        const bool in = (mine_key >> (shift + 4)) == prefix;
-        const uint32_t digit = (mine_key >> shift) & 15u;
-        uint32_t mine = 0;
-#pragma unroll
-        for (int d = 0; d < 16; ++d) {
-            const uint32_t c = __builtin_popcountll(__builtin_amdgcn_ballot_w64(in && digit == static_cast<uint32_t>(d)));
-            if (lane == d) mine = c;
-        }
-        if (lane < 16) wave_cnt[wave * 16 + lane] = mine;
-        __syncthreads();
-        if (tid < 16) {
-            uint32_t t = 0;
-#pragma unroll
-            for (int w = 0; w < PW; ++w) t += wave_cnt[w * 16 + tid];
-            digit_cnt[tid] = t;
-        }
-        __syncthreads();
-        if (shift == 12) {
-            uint32_t lanes_with_data = 0;
-#pragma unroll
-            for (int d = 0; d < 16; ++d) lanes_with_data += digit_cnt[d];
-            if (lanes_with_data < topk) {
-                keep_all = true;
-                break;// uniform over the workgroup
-            }
-        }
-        choose_digit(digit_cnt, prefix, want);
-    }
-    const uint32_t bound = keep_all ? 0u : prefix;
-    uint32_t key_max = 0;
-#pragma unroll
-    for (int w = 0; w < PW; ++w) key_max = wave_key[w] > key_max ? wave_key[w] : key_max;
+    // what the ranks say besides the bound: rank 0 holds the workgroup's
+    // maximum, and a lane without data is beaten by exactly the lanes with data
+    if (has && rank == 0) max_slot = lane_max;
+    if (!has) data_lanes = rank;// every such lane writes the same number
+    if (has && rank == topk - 1) bound_slot = lane_max;
+    __syncthreads();
+    const bool keep_all = data_lanes < topk;// uniform over the workgroup
+    const uint32_t bound = keep_all ? 0u : bound_slot;
+    const uint32_t key_max = max_slot;
     const float top = value_of_key<T>(key_max);
 
     // survivors to the workspace, and the partial denominator
@@ -579,32 +581,57 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
     uint32_t prefix = 0, want = topk, ties = 0;
 #pragma unroll 1
     for (int shift = 12; shift >= 0; shift -= 4) {
-        // counting is one ballot per digit and slot; a wavefront skips the slots
-        // in which none of its entries shares the prefix any more (with a few
-        // hundred survivors most wavefronts hold one live slot or none)
+        // Counting: a lane's entry becomes a one in an 8-bit field - digit d in
+        // field d & 3 of word d >> 2 - and four DPP wave sums add the fields of
+        // all 64 lanes at once (a field holds at most 64); lane d then picks
+        // its field.  A wavefront skips the slots in which none of its entries
+        // shares the prefix any more (with a few hundred survivors most
+        // wavefronts hold one live slot or none).  One ballot and population
+        // count per digit and slot, the first form, took 1.5 us a pass.
         uint32_t mine = 0;
 #pragma unroll
         for (int i = 0; i < PER_LANE; ++i) {
             const bool in = (keys[i] >> (shift + 4)) == prefix;
             if (__builtin_amdgcn_ballot_w64(in) == 0) continue;
             const uint32_t digit = (keys[i] >> shift) & 15u;
+            const uint32_t one = in ? 1u << (8u * (digit & 3u)) : 0u;
+            const uint32_t word = digit >> 2;
+            const uint32_t s0 = wave_sum_u32(word == 0 ? one : 0u), s1 = wave_sum_u32(word == 1 ? one : 0u);
+            const uint32_t s2 = wave_sum_u32(word == 2 ? one : 0u), s3 = wave_sum_u32(word == 3 ? one : 0u);
+            const uint32_t lw = static_cast<uint32_t>(lane) >> 2;
+            const uint32_t sel = lw == 0 ? s0 : lw == 1 ? s1 : lw == 2 ? s2 : s3;
+            mine += (sel >> (8u * (static_cast<uint32_t>(lane) & 3u))) & 0xFFu;// lanes past 15 hold nothing of use
+        }
+        // one barrier a pass: every wavefront totals the columns itself (lane d
+        // the column of digit d) and walks them through lane reads; the two
+        // sets of counters take turns, so a wavefront that is a pass ahead
+        // never overwrites what a slower one still reads
+        uint32_t *set = sh.wave_cnt[(shift >> 2) & 1];
+        if (lane < 16) set[wave * 16 + lane] = mine;
+        __syncthreads();
+        uint32_t column = 0;
+        if (lane < 16) {
 #pragma unroll
-            for (int d = 0; d < 16; ++d) {
-                const uint32_t c = __builtin_popcountll(__builtin_amdgcn_ballot_w64(in && digit == static_cast<uint32_t>(d)));
-                if (lane == d) mine += c;
+            for (int w = 0; w < WAVES; ++w) column += set[w * 16 + lane];
+        }
+        uint32_t above = 0, chosen = 0, chosen_count = 0;
+        bool found = false;
+#pragma unroll
+        for (int d = 15; d >= 0; --d) {
+            const uint32_t c = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(column), d));
+            if (!found) {
+                if (above + c >= want) {
+                    chosen = d;
+                    chosen_count = c;
+                    found = true;
+                } else {
+                    above += c;
+                }
             }
         }
-        if (lane < 16) sh.wave_cnt[wave * 16 + lane] = mine;
-        __syncthreads();
-        if (tid < 16) {
-            uint32_t t = 0;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) t += sh.wave_cnt[w * 16 + tid];
-            sh.digit_cnt[tid] = t;
-        }
-        __syncthreads();
-        choose_digit(sh.digit_cnt, prefix, want);
-        if (shift == 0) ties = sh.digit_cnt[prefix & 15u];
+        want -= above;
+        prefix = (prefix << 4) | chosen;
+        if (shift == 0) ties = chosen_count;
     }
     // everything above the topk-th key plus every entry equal to it
     const uint32_t kept = topk - want + ties;
