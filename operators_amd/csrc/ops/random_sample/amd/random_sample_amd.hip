@@ -9,19 +9,20 @@
 // not the sort.  A vocabulary is 64-300 KiB: no work for the memory system, a
 // latency chain for a sort.  So nothing is sorted:
 //  * the key of the topk-th largest logit is found by a radix select over the
-//    16-bit codes (four passes of 4 bits; counters in registers or wavefront
-//    ballots, no atomics on hot bins);
+//    16-bit codes (four passes of 4 bits; counters in registers or packed
+//    fields summed over the wavefront with DPP adds, no atomics on hot bins);
 //  * the at most topk candidates are compacted into LDS and ranked there by
 //    (logit descending, index ascending), one candidate per lane;
-//  * the first wavefront walks the sequential running sums with the
-//    probabilities in registers.
+//  * the first wavefront forms the sequential running sums once, as a
+//    branch-free chain with the addends in registers, and takes the top-p and
+//    random_val decisions with ballots over them.
 // Two forms.  One workgroup of 1024 lanes does all of it from the logits in
 // one launch (topk_full; 79 us for 32 000 logits: one compute unit's
 // instruction rate is the limit).  With the workspace the descriptor asks for,
 // topk <= 256 and 4096 logits or more, a first launch spreads the pass over the
 // logits over up to 48 workgroups, each of which drops everything that cannot
 // be in the overall topk, and a second launch of one workgroup finishes from
-// the few hundred survivors (9.5 + 13.6 us for 32 000 logits, 11.9 + 18.6 us
+// the few hundred survivors (7.4 + 10.7 us for 32 000 logits, 10.0 + 14.5 us
 // for 151 936).
 //
 // Two things differ from the CPU path and are visible to a caller:
