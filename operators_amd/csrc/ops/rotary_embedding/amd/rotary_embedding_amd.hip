@@ -323,7 +323,8 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
     // 47.0 us looping with 2 workgroups per unit against 48.5 us one tile per
     // workgroup; [4096,32,128] fp16, 2048 tiles, 14.1 us (4 per unit) against
     // 16.8 us; k [8192,8,128], 1024 tiles, is faster one tile per workgroup
-    // (9.7 against 10.5 us) and stays on rope_vec.  Workgroups of 64 or 128
+    // (9.7 against 10.5 us) and stays on rope_vec (with two heads per lane, and
+    // so twice the workgroups, it takes 10.8 us).  Workgroups of 64 or 128
     // lanes, one tile each, measure the same as 256 for all three shapes, and
     // so does a 2-D grid with the token in blockIdx.y (position and table base
     // then come through scalar loads): 47.3 us for q.  With table loads and
