@@ -133,15 +133,16 @@ def make_causal_softmax(ctx, heads, seq, total, dtype, gen, name):
     return Launch(name, ctx.lib.infiniopCausalSoftmax, (plan.desc, None, 0, y.data_ptr()), nbytes, (plan, y))
 
 
-def make_random_sample(ctx, voc, topk, gen, name):
-    """One draw from `voc` fp16 logits ~ N(0, 3): top-p 0.9, top-k `topk`, temperature 0.8 (greedy when topk is 1)."""
+def make_random_sample(ctx, voc, topk, gen, name, use_workspace=True):
+    """One draw from `voc` fp16 logits ~ N(0, 3): top-p 0.9, top-k `topk`, temperature 0.8 (greedy when topk is 1).
+    Without the workspace the library serves the call with one workgroup."""
     import torch
 
     from operators_amd.ops import RandomSamplePlan
 
     logits = (_randn((voc,), torch.float32, gen) * 3).to(torch.float16)
     result = torch.zeros(1, dtype=torch.int64, device="cuda").view(torch.uint64)
-    plan = RandomSamplePlan(ctx, result, logits)
+    plan = RandomSamplePlan(ctx, result, logits, use_workspace)
     f = ctypes.c_float
     ws = plan.workspace.data_ptr() if plan.workspace is not None else None
     args = (plan.desc, ws, plan.workspace_size, result.data_ptr(), logits.data_ptr(), f(0.37), f(0.9 if topk > 1 else 0.0), topk, f(0.8))
@@ -377,6 +378,7 @@ def ops_table(ctx, args, gen):
         "S1 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample") for _ in range(MAX_SETS)],
         "S2 random_sample f16 voc 32000, greedy": lambda: [make_random_sample(ctx, 32000, 1, gen, "random_sample") for _ in range(MAX_SETS)],
         "S3 random_sample f16 voc 151936, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 50, gen, "random_sample") for _ in range(MAX_SETS)],
+        "S4 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8, no workspace (one workgroup)": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample", False) for _ in range(MAX_SETS)],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
@@ -500,6 +502,7 @@ def cpu_per_op(T):
     del y7
     l9 = (rng.standard_normal(151936, dtype=np.float32) * 3).astype(np.float16).view(np.uint16)
     run("S1 random_sample", "f16", lambda: oracle.random_sample(l9[:32000], 0.37, 0.9, 50, 0.8), lambda: ref.random_sample(l9[:32000], 0.37, 0.9, 50, 0.8))
+    out["S4 random_sample"] = dict(out["S1 random_sample"])  # the same call, served by one workgroup on the GPU
     run("S2 random_sample", "f16", lambda: oracle.random_sample(l9[:32000], 0.37, 0.0, 1, 0.8), lambda: ref.random_sample(l9[:32000], 0.37, 0.0, 1, 0.8))
     run("S3 random_sample", "f16", lambda: oracle.random_sample(l9, 0.37, 0.9, 50, 0.8), lambda: ref.random_sample(l9, 0.37, 0.9, 50, 0.8))
     return out

@@ -17,8 +17,8 @@
 //    branch-free chain with the addends in registers, and takes the top-p and
 //    random_val decisions with ballots over them.
 // Two forms.  One workgroup of 1024 lanes does all of it from the logits in
-// one launch (topk_full; 79 us for 32 000 logits: one compute unit's
-// instruction rate is the limit).  With the workspace the descriptor asks for,
+// one launch (topk_full; 32 000 logits take it several times as long as the
+// two-launch form: one compute unit's instruction rate is the limit).  With the workspace the descriptor asks for,
 // topk <= 256 and 4096 logits or more, a first launch spreads the pass over the
 // logits over up to 48 workgroups, each of which drops everything that cannot
 // be in the overall topk, and a second launch of one workgroup finishes from
@@ -279,9 +279,20 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
     uint32_t key_max = 0;
 #pragma unroll 1
     for (int shift = 12; shift >= 0; shift -= 4) {
-        uint32_t cnt[16];
+        // Per-lane digit counts.  An element adds a one to an 8-bit field (digit
+        // d: field d & 3 of word d >> 2), four conditional adds instead of
+        // sixteen; a lane adds at most eight ones per round, so the fields are
+        // emptied into full-width counters every 31 rounds.
+        uint32_t cnt[16], packed[4] = {0, 0, 0, 0};
 #pragma unroll
         for (int d = 0; d < 16; ++d) cnt[d] = 0;
+        const auto unpack = [&]() {
+#pragma unroll
+            for (int d = 0; d < 16; ++d) cnt[d] += (packed[d >> 2] >> (8 * (d & 3))) & 0xFFu;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) packed[w] = 0;
+        };
+        uint32_t since = 0;
         for (uint32_t base = tid * 8u; base < voc; base += step) {
             uint32_t h[8];
             const int n = load_codes<VEC>(probs, voc, base, h);
@@ -291,10 +302,17 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
                 if (shift == 12 && e < n) key_max = k > key_max ? k : key_max;
                 const bool in = (k >> (shift + 4)) == prefix;// never true for kNoKey: prefix < 2^12
                 const uint32_t digit = (k >> shift) & 15u;
+                const uint32_t one = in ? 1u << (8u * (digit & 3u)) : 0u;
+                const uint32_t word = digit >> 2;
 #pragma unroll
-                for (int d = 0; d < 16; ++d) cnt[d] += (in && digit == static_cast<uint32_t>(d)) ? 1u : 0u;
+                for (int w = 0; w < 4; ++w) packed[w] += word == static_cast<uint32_t>(w) ? one : 0u;
+            }
+            if (++since == 31) {
+                unpack();
+                since = 0;
             }
         }
+        unpack();
         uint32_t mine = 0;
 #pragma unroll
         for (int d = 0; d < 16; ++d) {
