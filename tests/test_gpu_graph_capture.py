@@ -62,3 +62,47 @@ def test_chain_replays_from_a_hip_graph(ctx):
             assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), (replay, name)
     for p in plans:
         p.close()
+
+
+def test_random_sample_replays_from_a_hip_graph(ctx):
+    """The two launches of the sampling form, captured once: every replay
+    draws from whatever the logits buffer holds at that moment and must give
+    the index an eager call gives for the same logits."""
+    import torch
+
+    from operators_amd.ops import RandomSamplePlan
+
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    draws = [(torch.randn(32000, device="cuda", generator=gen) * 3).to(torch.float16) for _ in range(4)]
+    logits = draws[0].clone()
+    result = torch.full((1,), -1, dtype=torch.int64, device="cuda")
+    plan = RandomSamplePlan(ctx, result.view(torch.uint64), logits)
+    assert plan.workspace_size > 0
+    args = (0.61, 0.9, 40, 0.9)
+
+    want = []
+    for d in draws:
+        logits.copy_(d)
+        plan(result.view(torch.uint64), logits, *args, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        want.append(int(result.item()))
+    assert len(set(want)) > 1  # the draws differ, so a replay that ignored the buffer would show
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            plan(result.view(torch.uint64), logits, *args, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    for replay, d in enumerate(draws):
+        logits.copy_(d)
+        result.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(result.item()) == want[replay], replay
+    plan.close()
