@@ -120,14 +120,20 @@ __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
     }
     return v;
 }
-// Inclusive prefix sum over the lanes of a wavefront.
-__device__ __forceinline__ uint32_t wave_scan_u32(uint32_t v, int lane) {
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-        const uint32_t below = __shfl_up(v, o);
-        if (lane >= o) v += below;
-    }
-    return v;
+// Inclusive prefix sum over the lanes of a wavefront with DPP adds: shifts by
+// 1, 2, 4 and 8 lanes inside each row of 16, then the last lane of row 0 and
+// of row 2 onto the rows that follow (row_bcast:15 for rows 1 and 3), then the
+// last lane of row 1 onto rows 2 and 3 (row_bcast:31).  Lanes a shift does not
+// reach add zero.
+__device__ __forceinline__ uint32_t wave_scan_u32(uint32_t v) {
+    int x = static_cast<int>(v);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false);// row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false);// row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false);// row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false);// row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);// row_bcast:15 -> rows 1, 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);// row_bcast:31 -> rows 2, 3
+    return static_cast<uint32_t>(x);
 }
 
 // Greedy form (random_sample.cc:127-148): the first index holding the maximum,
@@ -361,7 +367,7 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
                 c_eq += k[e] == key_k ? 1u : 0u;
             }
         }
-        const uint32_t inc_gt = wave_scan_u32(c_gt, lane), inc_eq = wave_scan_u32(c_eq, lane);
+        const uint32_t inc_gt = wave_scan_u32(c_gt), inc_eq = wave_scan_u32(c_eq);
         if (lane == kWave - 1) {
             sh.scan_tot[buf][wave][0] = inc_gt;
             sh.scan_tot[buf][wave][1] = inc_eq;
@@ -502,7 +508,7 @@ __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(
                 }
             }
         }
-        const uint32_t inc = wave_scan_u32(c, lane);
+        const uint32_t inc = wave_scan_u32(c);
         uint32_t at = 0;
         if (lane == kWave - 1 && inc != 0) at = atomicAdd(&fill, inc);
         at = __shfl(at, kWave - 1) + inc - c;
@@ -550,7 +556,7 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
     if (tid < kWave) {
         RandomSamplePart head{0, 0, 0.0f, 0};
         if (static_cast<uint32_t>(tid) < groups) head = heads[tid];
-        const uint32_t upto = wave_scan_u32(head.count, lane);
+        const uint32_t upto = wave_scan_u32(head.count);
         const bool fits = __builtin_amdgcn_ballot_w64(head.count > static_cast<uint32_t>(kRandomSamplePartCap)) == 0;
         if (static_cast<uint32_t>(tid) < groups) {
             offs[tid + 1] = upto;
