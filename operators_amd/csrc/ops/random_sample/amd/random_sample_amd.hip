@@ -22,7 +22,7 @@
 // topk <= 256 and 4096 logits or more, a first launch spreads the pass over the
 // logits over up to 48 workgroups, each of which drops everything that cannot
 // be in the overall topk, and a second launch of one workgroup finishes from
-// the few hundred survivors (7.4 + 10.7 us for 32 000 logits, 10.0 + 14.5 us
+// the few hundred survivors (6.9 + 10.3 us for 32 000 logits, 9.7 + 14.0 us
 // for 151 936).
 //
 // Two things differ from the CPU path and are visible to a caller:
