@@ -39,12 +39,27 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 MFMA_PEAK_TFLOPS_16BIT = 2500.0  # MI355X published dense bf16 / fp16 matrix peak
 
 # HBM bytes per launch of the dominant kernel at the default workload
-# (swiglu bf16 [8192, 28672] from a fused [8192, 57344] buffer), measured with
-# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, each scaled by what the same
-# counter reads for a plain 128 MiB device copy (1.99960 and 1.00000); the runs
-# are summarised in profiles/c5_kernels_hbm_traffic_pmc.txt.  Algorithmic bytes
-# for the same launch: 1 409 286 144.
-MEASURED_TRAFFIC_SWIGLU_8192 = 1409140152
+# (swiglu bf16 [8192, 28672] from a fused [8192, 57344] buffer) are read from
+# the committed summary of the hardware-counter runs: rocprofv3 --pmc FETCH_SIZE
+# and --pmc WRITE_SIZE, each scaled by what the same counter reads for a plain
+# 128 MiB device copy.  The summary names the commands that made it.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "c5_kernels_hbm_traffic_pmc.txt")
+DOMINANT_KERNEL = "swiglu_rows<amd::BF16Rne"
+
+
+def measured_traffic(path=TRAFFIC_PROFILE, kernel=DOMINANT_KERNEL):
+    """HBM bytes per launch of `kernel` from its row of the counter summary
+    (columns: kernel (grid), FETCH KiB, WRITE KiB, HBM bytes/launch,
+    algorithmic, ratio).  No file or no row is an error: a roofline line whose
+    traffic figure comes from nowhere would be worse than none."""
+    if not os.path.isfile(path):
+        raise FileNotFoundError(f"{path}: the hardware-counter summary the roofline's traffic figure is read from is missing")
+    with open(path) as f:
+        for line in f:
+            if line.startswith(kernel):
+                cols = line.split()
+                return int(cols[-3])
+    raise LookupError(f"{path} has no row for {kernel}")
 
 
 def parse():
@@ -581,6 +596,8 @@ def main():
               "there is no multi-GPU path to measure) - run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    traffic = measured_traffic() if args.tokens == 8192 else None  # before anything runs: a missing summary stops the run
+
     import torch
 
     from operators_amd.ops import Context, sin_cos_table
@@ -616,7 +633,7 @@ def main():
     roofline = {
         "bound": "hbm", "achieved": round(sw_bytes / sw_time / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(sw_bytes / sw_time / 1e9 / HBM_PEAK_GBPS, 4),
-        "traffic": MEASURED_TRAFFIC_SWIGLU_8192 if T == 8192 else None,
+        "traffic": traffic,
         "kernel": f"swiglu_rows<bf16> [{T},28672] from fused [{T},57344]",
         "bytes_per_launch": sw_bytes, "us_per_launch": round(sw_time * 1e6, 2),
     }

@@ -99,10 +99,7 @@ def install(root):
     ($INFINI_ROOT/lib/libinfiniop.so, operatorspy/liboperators.py:11,55)."""
     os.makedirs(os.path.join(root, "lib"), exist_ok=True)
     shutil.copy2(LIB_PATH, os.path.join(root, "lib", "libinfiniop.so"))
-    dst_inc = os.path.join(root, "include")
-    os.makedirs(dst_inc, exist_ok=True)
-    for f in os.listdir(INCLUDE):
-        shutil.copy2(os.path.join(INCLUDE, f), os.path.join(dst_inc, f))
+    shutil.copytree(INCLUDE, os.path.join(root, "include"), dirs_exist_ok=True)
 
 
 if __name__ == "__main__":

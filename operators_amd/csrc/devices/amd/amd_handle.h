@@ -5,7 +5,7 @@
 #ifndef INFINIOP_AMD_HANDLE_H
 #define INFINIOP_AMD_HANDLE_H
 
-#include "infiniop.h"
+#include "operators.h"
 
 // Plain C layout; `device` must stay first (the dispatchers read only it).
 struct AmdContext {

@@ -5,9 +5,10 @@
 #ifndef INFINIOP_AMD_COMMON_H
 #define INFINIOP_AMD_COMMON_H
 
-#include "infiniop.h"
+#include "operators.h"
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <hip/hip_runtime_api.h>
 
@@ -55,12 +56,28 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
 
+// The largest 1-D grid of `lanes`-wide workgroups HIP accepts: a launch may
+// not span 2^32 work-items or more along one axis.  Kernels launched with a
+// capped grid stride over the rest of their range.
+inline uint64_t max_grid_1d(unsigned lanes) { return 0xFFFFFFFFull / lanes; }
+
 // Outputs of at least this many bytes are written through L2 (cache policy
 // "sc1 nt") by the kernels that write one byte per byte read; smaller ones
 // are left for L2 to absorb.  Measured on MI355X (32 MiB of L2 in all): a
 // 16 MiB output is 7 % faster absorbed, a 32 MiB one is even, 128 MiB and
 // more are 1-3 % faster written through.
 constexpr uint64_t kWriteThroughBytes = 64ull << 20;
+
+// Launch-shape experiments: a build with -DINFINIOP_AMD_TUNE reads integer
+// knobs from the environment; the normal build folds every knob to its default.
+#ifdef INFINIOP_AMD_TUNE
+inline long tune(const char *name, long dflt) {
+    const char *v = std::getenv(name);
+    return v != nullptr ? std::atol(v) : dflt;
+}
+#else
+constexpr long tune(const char *, long dflt) { return dflt; }
+#endif
 
 }// namespace amd
 

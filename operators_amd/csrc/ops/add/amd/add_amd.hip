@@ -21,11 +21,11 @@ using namespace amd;
 // 16-byte access per lane per operand, one workgroup per KiB of output, take
 // 61.4 us; 128 lanes 61.6; 256 lanes 63.1-63.7; 2 or 4 accesses per lane
 // 62.7-65.8; workgroups that loop over tiles (16-64 per compute unit)
-// 65.4-69.6.  The broadcast kernels keep 256 lanes: with an operand that is
-// re-read through the caches, [8192, 4096] fp16 plus a [4096] row takes 24.4 us
-// that way and 31-32 us as a 2-D grid of single-wavefront workgroups (only 8
-// of them per row; the same workgroups numbered along one grid axis, with the
-// row found by division, take 24.1 us - not worth a second kernel shape).
+// 65.4-69.6.  The general broadcast kernels keep 256 lanes: with an operand
+// that is re-read through the caches, [8192, 4096] fp16 plus a [4096] row takes
+// 24.4 us that way and 31-32 us as a 2-D grid of single-wavefront workgroups
+// (only 8 of them per row); the same workgroups numbered along one grid axis
+// are the form add_rowvec_tiles below takes for that shape.
 constexpr int kBlock = 256;// lanes per workgroup of the broadcast and element-wise kernels
 
 // ---- per-type arithmetic on one 128-bit word ---------------------------------
@@ -68,7 +68,7 @@ struct Add32 {
 // One wavefront per workgroup, one vector per lane, one workgroup per KiB: the
 // dispatcher hands out consecutive KiBs in order and every wavefront gives its
 // slot back the moment it is done.  (The loop only runs more than once for
-// ranges beyond 2^31 workgroups.)
+// ranges beyond what one launch may span: 2^32 work-items.)
 template<typename Op>
 __global__ __launch_bounds__(kWave) void add_flat_vec(u32x4 *c, const u32x4 *a, const u32x4 *b, uint64_t nvec) {
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kWave;
@@ -182,6 +182,30 @@ __global__ __launch_bounds__(kBlock) void add_bcast_rows(u32x4 *c, const typenam
     }
 }
 
+// ---- a whole tensor plus one row:  c[r, :] = full[r, :] + vec[:] ---------------
+// The residual-plus-bias shape.  It is the flat kernel's launch shape -
+// workgroups of one wavefront, one vector per lane, tiles in address order -
+// with the row's tile found from the workgroup number; the row itself (a few
+// KiB) comes through the caches.  One read and one write per output byte, so
+// large outputs are written through L2 (THROUGH, see StreamOut).  Measured on
+// MI355X, [8192, 4096] fp16 plus a [4096] row: 23.2 us, against 24.5 us for a
+// 2-D grid of 256-lane workgroups (add_bcast_rows), 23.6-25.5 us for workgroups
+// that keep their piece of the row in registers and walk down the rows, and
+// 23.6-24.0 us for single-wavefront workgroups that own 2 or 4 rows of a tile;
+// [8192, 8192] bf16: 40.9 against 42.7 us.
+// SWAP says the row is operand a (the sum is formed as a + b either way).
+template<typename Op, bool SWAP, bool THROUGH>
+__global__ __launch_bounds__(kWave) void add_rowvec_tiles(u32x4 *c, const u32x4 *full, const u32x4 *vec, uint32_t tiles_per_row, uint64_t ntiles) {
+    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {// more than one pass only beyond what one launch may span
+        const uint32_t ct = static_cast<uint32_t>(tile % tiles_per_row);
+        const u32x4 vv = ld16(vec + ct * kWave + threadIdx.x);
+        const u32x4 vf = ld16_stream(full + tile * kWave + threadIdx.x);
+        const u32x4 r = SWAP ? Op::vec(vv, vf) : Op::vec(vf, vv);
+        if constexpr (THROUGH) StreamOut<true>(c + tile * kWave).st16(threadIdx.x * 16, r);
+        else st16_stream(c + tile * kWave + threadIdx.x, r);
+    }
+}
+
 // Element form: any strides.
 template<typename Op, typename Idx>
 __global__ __launch_bounds__(kBlock) void add_bcast_scalar(typename Op::scalar *c, const typename Op::scalar *a,
@@ -200,7 +224,7 @@ inline unsigned grid_for(uint64_t work_items, uint64_t per_block, int cu_count, 
     const uint64_t want = ceil_div(work_items, per_block);
     const uint64_t cap = blocks_per_cu > 0 ? static_cast<uint64_t>(cu_count) * blocks_per_cu : want;
     uint64_t g = want < cap ? want : cap;
-    g = g < 0x7FFFFFFFull ? g : 0x7FFFFFFFull;// the kernels stride over whatever one launch cannot index
+    g = g < max_grid_1d(static_cast<unsigned>(per_block)) ? g : max_grid_1d(static_cast<unsigned>(per_block));// the kernels stride over the rest
     return static_cast<unsigned>(g == 0 ? 1 : g);
 }
 
@@ -277,6 +301,21 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         // one streamed operand and a large output: write through L2
         const bool through = (ma == kFull) != (mb == kFull) && n * sizeof(S) >= kWriteThroughBytes && inner_vecs < (1ull << 28);
         bool launched = false;
+        // a whole tensor plus one row whose length is a multiple of a wavefront of vectors
+        if (desc.ndim == 2 && inner_vecs % kWave == 0 && inner_vecs < (1ull << 31) &&
+            ((ma == kFull && mb == kRuns && desc.b_stride[1] == 0) || (ma == kRuns && mb == kFull && desc.a_stride[1] == 0))) {
+            const bool swap = ma == kRuns;
+            const u32x4 *full = static_cast<const u32x4 *>(swap ? b : a), *vec = static_cast<const u32x4 *>(swap ? a : b);
+            u32x4 *pc = static_cast<u32x4 *>(c);
+            const uint32_t tpr = static_cast<uint32_t>(inner_vecs / kWave);
+            const uint64_t ntiles = desc.shape[1] * tpr;
+            const unsigned g = static_cast<unsigned>(ntiles < max_grid_1d(kWave) ? ntiles : max_grid_1d(kWave));
+            if (swap && through) add_rowvec_tiles<Op, true, true><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
+            else if (swap) add_rowvec_tiles<Op, true, false><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
+            else if (through) add_rowvec_tiles<Op, false, true><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
+            else add_rowvec_tiles<Op, false, false><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
+            return STATUS_SUCCESS;
+        }
 #define ADD_BCAST_CASE(MA, MB)                                        \
     if (ma == MA && mb == MB) {                                       \
         if (rows_form && through) go_rows(add_bcast_rows<Op, MA, MB, true>);  \

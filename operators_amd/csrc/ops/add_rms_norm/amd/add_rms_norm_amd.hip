@@ -26,10 +26,14 @@ infiniopStatus_t amdAddRMSNorm(AddRMSNormAmdDescriptor_t desc, void *, uint64_t,
     hipStream_t s = static_cast<hipStream_t>(stream);
     const RowsShape shape{desc->cu_count, desc->lds_per_block, desc->n, desc->d, desc->stride_y, desc->stride_a, desc->epsilon};
     const Residual<true> res{static_cast<uint16_t *>(c), static_cast<const uint16_t *>(b), desc->stride_c, desc->stride_b};
-    const bool ok = desc->elem == amd::Elem::F16 ? launch_by_weight<amd::F16Ref, true>(desc->w_elem, shape, y, a, w, res, s)
-                                                 : launch_by_weight<amd::BF16Rne, true>(desc->w_elem, shape, y, a, w, res, s);
-    if (!ok) {
+    const int w_kind = weight_kind(desc->w_elem);
+    if (w_kind < 0) {
         return STATUS_BAD_TENSOR_DTYPE;
+    }
+    if (desc->elem == amd::Elem::F16) {
+        launch_rms_norm<amd::F16Ref, true>(shape, y, a, w, w_kind, res, s);
+    } else {
+        launch_rms_norm<amd::BF16Rne, true>(shape, y, a, w, w_kind, res, s);
     }
     AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
     return STATUS_SUCCESS;

@@ -42,6 +42,17 @@ infiniopStatus_t amdCreateRearrangeDescriptor(AmdHandle_t handle, RearrangeAmdDe
     desc->device = DevAmdGpu;
     desc->device_id = handle->device_id;
     desc->cu_count = handle->cu_count;
+    // An extent of zero anywhere: nothing to copy (the reference's loops run
+    // zero times).  Decided here, before any extent is divided by.
+    for (uint64_t i = 0; i < ndim; ++i) {
+        if (dst->shape[i] == 0) {
+            desc->rows = 0;
+            desc->row_bytes = 0;
+            desc->ndim = 0;
+            *desc_ptr = desc;
+            return STATUS_SUCCESS;
+        }
+    }
     desc->row_bytes = dst->shape[ndim - 1] * static_cast<uint64_t>(elem);
     desc->rows = 1;
 

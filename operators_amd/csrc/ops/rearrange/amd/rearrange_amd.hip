@@ -76,33 +76,35 @@ __global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint
 template<int BYTES, typename Idx, bool BUFST>
 __global__ __launch_bounds__(Lanes<BYTES>::value) void rearrange_flat(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t total_units, Idx units_per_row) {
     typedef typename Unit<BYTES>::type U;
-    const uint64_t idx64 = static_cast<uint64_t>(blockIdx.x) * Lanes<BYTES>::value + threadIdx.x;
-    if (idx64 >= total_units) return;
-    const Idx idx = static_cast<Idx>(idx64);
-    Idx rest = idx / units_per_row;
-    const Idx col = idx - rest * units_per_row;
-    int64_t od = 0, os = 0;
+    // one pass for anything a single launch can span (2^32 work-items); the loop covers the rest
+    const uint64_t step = static_cast<uint64_t>(gridDim.x) * Lanes<BYTES>::value;
+    for (uint64_t idx64 = static_cast<uint64_t>(blockIdx.x) * Lanes<BYTES>::value + threadIdx.x; idx64 < total_units; idx64 += step) {
+        const Idx idx = static_cast<Idx>(idx64);
+        Idx rest = idx / units_per_row;
+        const Idx col = idx - rest * units_per_row;
+        int64_t od = 0, os = 0;
 #pragma unroll
-    for (int k = 0; k < kRearrangeMaxDims; ++k) {
-        if (k < d.ndim) {
-            const Idx ext = static_cast<Idx>(d.shape[k]);
-            const Idx q = rest / ext;
-            const Idx i = rest - q * ext;
-            rest = q;
-            od += static_cast<int64_t>(i) * d.dst_stride[k];
-            os += static_cast<int64_t>(i) * d.src_stride[k];
+        for (int k = 0; k < kRearrangeMaxDims; ++k) {
+            if (k < d.ndim) {
+                const Idx ext = static_cast<Idx>(d.shape[k]);
+                const Idx q = rest / ext;
+                const Idx i = rest - q * ext;
+                rest = q;
+                od += static_cast<int64_t>(i) * d.dst_stride[k];
+                os += static_cast<int64_t>(i) * d.src_stride[k];
+            }
         }
-    }
-    const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
-    if constexpr (BUFST) {
-        StreamOut<true>(dst).st16(static_cast<uint32_t>(od) + static_cast<uint32_t>(col) * 16, v);
-    } else {
-        __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+        const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
+        if constexpr (BUFST) {
+            StreamOut<true>(dst).st16(static_cast<uint32_t>(od) + static_cast<uint32_t>(col) * 16, v);
+        } else {
+            __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+        }
     }
 }
 
 template<int BYTES>
-bool launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, const void *src, hipStream_t stream) {
+void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, const void *src, hipStream_t stream) {
     auto *pd = static_cast<uint8_t *>(dst);
     auto *ps = static_cast<const uint8_t *>(src);
     const uint64_t upr = desc.row_bytes / BYTES;
@@ -133,10 +135,8 @@ bool launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         }
     } else {// short rows, or a single row too long for 32-bit column numbers
         const uint64_t total = desc.rows * upr;
-        const uint64_t blocks = ceil_div(total, kBlock);
-        if (blocks > 0x7FFFFFFFull) {
-            return false;
-        }
+        const uint64_t want = ceil_div(total, kBlock);
+        const uint64_t blocks = want < max_grid_1d(kBlock) ? want : max_grid_1d(kBlock);
         if (total < (1ull << 32)) {
             if (BYTES == 16 && large && forward && dst_span < (1ull << 32)) {
                 rearrange_flat<BYTES, uint32_t, BYTES == 16><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr));
@@ -147,7 +147,6 @@ bool launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
             rearrange_flat<BYTES, uint64_t, false><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, upr);
         }
     }
-    return true;
 }
 
 }// namespace
@@ -175,15 +174,11 @@ infiniopStatus_t amdRearrange(RearrangeAmdDescriptor_t desc, void *dst, void con
     }
     AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    bool ok;
-    if (align % 16 == 0) ok = launch<16>(*desc, d, dst, src, s);
-    else if (align % 8 == 0) ok = launch<8>(*desc, d, dst, src, s);
-    else if (align % 4 == 0) ok = launch<4>(*desc, d, dst, src, s);
-    else if (align % 2 == 0) ok = launch<2>(*desc, d, dst, src, s);
-    else ok = launch<1>(*desc, d, dst, src, s);
-    if (!ok) {// more than 2^31 workgroups of short rows: beyond what one launch addresses
-        return STATUS_BAD_TENSOR_SHAPE;
-    }
+    if (align % 16 == 0) launch<16>(*desc, d, dst, src, s);
+    else if (align % 8 == 0) launch<8>(*desc, d, dst, src, s);
+    else if (align % 4 == 0) launch<4>(*desc, d, dst, src, s);
+    else if (align % 2 == 0) launch<2>(*desc, d, dst, src, s);
+    else launch<1>(*desc, d, dst, src, s);
     AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
     return STATUS_SUCCESS;
 }

@@ -22,10 +22,14 @@ infiniopStatus_t amdRMSNorm(RMSNormAmdDescriptor_t desc, void *, uint64_t, void 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const RowsShape shape{desc->cu_count, desc->lds_per_block, desc->n, desc->d, desc->stride_y, desc->stride_x, desc->epsilon};
     const Residual<false> none{};
-    const bool ok = desc->elem == amd::Elem::F16 ? launch_by_weight<amd::F16Ref, false>(desc->w_elem, shape, y, x, w, none, s)
-                                                 : launch_by_weight<amd::BF16Rne, false>(desc->w_elem, shape, y, x, w, none, s);
-    if (!ok) {
+    const int w_kind = weight_kind(desc->w_elem);
+    if (w_kind < 0) {
         return STATUS_BAD_TENSOR_DTYPE;
+    }
+    if (desc->elem == amd::Elem::F16) {
+        launch_rms_norm<amd::F16Ref, false>(shape, y, x, w, w_kind, none, s);
+    } else {
+        launch_rms_norm<amd::BF16Rne, false>(shape, y, x, w, w_kind, none, s);
     }
     AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
     return STATUS_SUCCESS;

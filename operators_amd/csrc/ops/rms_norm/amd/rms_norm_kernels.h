@@ -22,7 +22,10 @@
 #include "../../../devices/amd/common_amd.h"
 #include "../../../devices/amd/kernel_amd.h"
 
+// Internal linkage: each including translation unit owns its copies, and none
+// of them appears in the library's dynamic symbol table.
 namespace rms_norm_kernels {
+namespace {
 
 using namespace amd;
 
@@ -48,9 +51,29 @@ struct W16 {
     }
 };
 
+// The weight row's element type is a run-time property of the call (kind), not
+// a template parameter: it only matters where the weights are fetched, which
+// is once per workgroup when they are staged in LDS.
+enum WeightKind { kWKindF32 = 0, kWKindF16 = 1, kWKindBF16 = 2 };
+
+__device__ __forceinline__ void load_w8(const void *w, int kind, uint32_t vec, float (&g)[8]) {
+    if (kind == kWKindF32) WF32::load8(w, vec, g);
+    else if (kind == kWKindF16) W16<F16Ref>::load8(w, vec, g);
+    else W16<BF16Rne>::load8(w, vec, g);
+}
+__device__ __forceinline__ float load_w1(const void *w, int kind, uint64_t j) {
+    if (kind == kWKindF32) return WF32::one(w, j);
+    if (kind == kWKindF16) return W16<F16Ref>::one(w, j);
+    return W16<BF16Rne>::one(w, j);
+}
+
 __device__ __forceinline__ float inv_rms(float sum_sq, uint64_t d, float eps) {
     const float mean_eps = sum_sq / static_cast<float>(d) + eps;
+#ifdef RMS_DIAG_F32
+    return __builtin_amdgcn_rsqf(mean_eps);
+#else
     return static_cast<float>(1.0 / sqrt(static_cast<double>(mean_eps)));
+#endif
 }
 
 // ---- rows that fit in registers -----------------------------------------------
@@ -98,10 +121,10 @@ struct Residual<true> {
     int64_t stride_c, stride_b;
 };
 
-template<typename T, typename W, int BS, int NV, int WHOME, bool EXACT, bool THROUGH, bool ADD>
-__global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w,
+template<typename T, int BS, int NV, int WHOME, bool EXACT, bool THROUGH, bool ADD>
+__global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
-                                                     Residual<ADD> res) {
+                                                     uint64_t first_mul, uint64_t hop, uint64_t span, Residual<ADD> res) {
     constexpr int WAVES = BS / kWave;
     __shared__ float red[2 * WAVES];
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
@@ -127,29 +150,44 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
         }
     };
 
-    uint64_t row = blockIdx.x;
+    // This workgroup's rows: first, first + hop, ... below `last`.
+    uint64_t row = blockIdx.x * first_mul;
     if (row >= n) return;
+    const uint64_t last = row + span < n ? row + span : n;
     u32x4 xv[NV], xn[NV], bv[NB], bn[NB];
     load_row(row, xv, bv);// in flight while the weights are fetched below
+    bool more = row + hop < last;// this workgroup owns a row after the current one
 
     if constexpr (WHOME == kWLds) {
-        // all of this lane's weight loads are issued before the first is
-        // consumed: one memory latency for the staging, not one per vector
-        float g[NV][8];
+        // All of this lane's weight loads are issued before the first is
+        // consumed, and the second row's loads go out behind them before
+        // anything waits: the workgroup pays one memory latency before it
+        // streams, not one for the weights and another for the prefetch.
+        auto stage = [&](auto tag) {
+            typedef decltype(tag) W;
+            float g[NV][8];
 #pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
-            W::load8(w, EXACT || v < nvec ? v : 0, g[k]);
-        }
-#pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
-            if (EXACT || v < nvec) {
-                w_lo[v] = f32x4{g[k][0], g[k][1], g[k][2], g[k][3]};
-                w_hi[v] = f32x4{g[k][4], g[k][5], g[k][6], g[k][7]};
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                W::load8(w, EXACT || v < nvec ? v : 0, g[k]);
             }
-        }
+            if (more) load_row(row + hop, xn, bn);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                if (EXACT || v < nvec) {
+                    w_lo[v] = f32x4{g[k][0], g[k][1], g[k][2], g[k][3]};
+                    w_hi[v] = f32x4{g[k][4], g[k][5], g[k][6], g[k][7]};
+                }
+            }
+        };
+        if (w_kind == kWKindF32) stage(WF32{});
+        else if (w_kind == kWKindF16) stage(W16<F16Ref>{});
+        else stage(W16<BF16Rne>{});
         __syncthreads();
+    } else {
+        if (more) load_row(row + hop, xn, bn);
     }
 
     // One row: reduce, scale by the weights, store.
@@ -193,12 +231,18 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
             if (EXACT || v < nvec) {
                 float f[8], g[8];
                 widen8<T>(cur[k], f);
+#ifdef RMS_DIAG_NOW
+                if constexpr (true) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) g[i] = 1.0f;
+                } else
+#endif
                 if constexpr (WHOME == kWLds) {
                     const f32x4 a = w_lo[v], b = w_hi[v];
                     g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
                     g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
                 } else {
-                    W::load8(w, v, g);
+                    load_w8(w, w_kind, v, g);
                 }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
@@ -210,31 +254,170 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
     // Steady state: the next row's loads are issued, unconditionally, before
     // the current row is reduced.  Two register sets take turns (no copies, so
     // the wait for a prefetched row comes only when that row is reduced) and a
-    // row's loads are never issued unless this workgroup owns that row.
-    const uint64_t hop = gridDim.x;
-    while (true) {
-        if (row + hop >= n) {
-            finish_row(row, xv, bv, 0);
-            break;
-        }
-        load_row(row + hop, xn, bn);
+    // row's loads are never issued unless this workgroup owns that row.  The
+    // first row is finished ahead of the loop - the second is already on its
+    // way - so that the loop is entered with the memory operations in the
+    // order every later pass leaves them in, and the waits inside it count
+    // the younger operations instead of draining the queue.
+    if (!more) {
         finish_row(row, xv, bv, 0);
-        row += hop;
-        if (row + hop >= n) {
+        return;
+    }
+    finish_row(row, xv, bv, 0);
+    row += hop;
+    while (true) {
+        if (row + hop >= last) {
             finish_row(row, xn, bn, 1);
             break;
         }
         load_row(row + hop, xv, bv);
         finish_row(row, xn, bn, 1);
         row += hop;
+        if (row + hop >= last) {
+            finish_row(row, xv, bv, 0);
+            break;
+        }
+        load_row(row + hop, xn, bn);
+        finish_row(row, xv, bv, 0);
+        row += hop;
+    }
+}
+
+// ---- one pass in dispatch order ----------------------------------------------
+// A workgroup serves R consecutive rows and retires; the grid is n / R
+// workgroups, handed out in address order.  Everything a workgroup will ever
+// load - its rows and the weight row, which it keeps in registers - is
+// requested before the first wait, so it pays one memory latency.  The weight
+// row comes through L2 once per R rows.  The R sums of squares share one
+// barrier.
+template<typename T, int BS, int NV, int R, bool EXACT, bool THROUGH, bool ADD>
+__global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
+                                                     uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
+                                                     Residual<ADD> res) {
+    constexpr int WAVES = BS / kWave;
+    __shared__ float red[R * WAVES];
+    const uint32_t nvec = d / 8;
+    const uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * R;
+    const int rows_here = n - row0 < static_cast<uint64_t>(R) ? static_cast<int>(n - row0) : R;
+
+    u32x4 xv[R][NV];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint64_t row = row0 + (r < rows_here ? r : 0);
+        const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            xv[r][k] = ld16_stream(xr + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
+        }
+    }
+    constexpr int RB = ADD ? R : 1;
+    u32x4 bv[RB][NV];
+    if constexpr (ADD) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint64_t row = row0 + (r < rows_here ? r : 0);
+            const uint16_t *br = res.b + static_cast<int64_t>(row) * res.stride_b;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                bv[r][k] = ld16_stream(br + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
+            }
+        }
+    }
+    float g[NV][8];
+    if (w_kind == kWKindF32) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            WF32::load8(w, EXACT || v < nvec ? v : 0, g[k]);
+        }
+    } else {
+        u32x4 raw[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            raw[k] = ld16(static_cast<const uint16_t *>(w) + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
+        }
+        if (w_kind == kWKindF16) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) widen8<F16Ref>(raw[k], g[k]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) widen8<BF16Rne>(raw[k], g[k]);
+        }
+    }
+
+    float part[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if constexpr (ADD) {// the row becomes a + b, rounded as Add rounds, and goes out to c
+            const StreamOut<THROUGH> cr(res.c + static_cast<int64_t>(row0 + r) * res.stride_c);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                float p[8], q[8];
+                widen8<T>(xv[r][k], p);
+                widen8<T>(bv[r][k], q);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) p[i] += q[i];
+                xv[r][k] = narrow8<T>(p);
+                if (r < rows_here && (EXACT || v < nvec)) cr.st16(v * 16, xv[r][k]);
+            }
+        }
+        part[r] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            float f[8];
+            widen8<T>(xv[r][k], f);
+            if constexpr (!EXACT) {
+                if (k * BS + threadIdx.x >= nvec) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) f[i] = 0.0f;
+                }
+            }
+            const float s01 = f[0] * f[0] + f[1] * f[1], s23 = f[2] * f[2] + f[3] * f[3];
+            const float s45 = f[4] * f[4] + f[5] * f[5], s67 = f[6] * f[6] + f[7] * f[7];
+            part[r] += (s01 + s23) + (s45 + s67);
+        }
+        part[r] = wave_sum(part[r]);
+    }
+    if constexpr (WAVES > 1) {
+        const int wave = threadIdx.x / kWave;
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) red[r * WAVES + wave] = part[r];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float total = 0.0f;
+#pragma unroll
+            for (int i = 0; i < WAVES; ++i) total += red[r * WAVES + i];
+            part[r] = total;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float k_row = inv_rms(part[r], d, eps);
+        const StreamOut<THROUGH> yr(y + static_cast<int64_t>(row0 + r) * stride_y);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            float f[8];
+            widen8<T>(xv[r][k], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[k][i];
+            if (r < rows_here && (EXACT || v < nvec)) yr.st16(v * 16, narrow8<T>(f));
+        }
     }
 }
 
 // ---- any row length, any alignment ----------------------------------------------
 // Two passes over the row with element accesses; the second pass re-reads x,
 // which the first pass left in cache for rows of ordinary length.
-template<typename T, typename W, bool ADD>
-__global__ __launch_bounds__(256) void rms_norm_generic(uint16_t *y, const uint16_t *x, const void *w,
+template<typename T, bool ADD>
+__global__ __launch_bounds__(256) void rms_norm_generic(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                          uint64_t n, uint64_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                          Residual<ADD> res) {
     constexpr int BS = 256, WAVES = BS / kWave;
@@ -262,7 +445,7 @@ __global__ __launch_bounds__(256) void rms_norm_generic(uint16_t *y, const uint1
         }
         const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
         for (uint64_t j = threadIdx.x; j < d; j += BS) {
-            yr[j] = T::narrow1((k_row * T::one(xr[j])) * W::one(w, j));
+            yr[j] = T::narrow1((k_row * T::one(xr[j])) * load_w1(w, w_kind, j));
         }
         // y may alias x (and c may alias a or b): every lane re-reads only elements it wrote itself.
     }
@@ -278,8 +461,18 @@ struct RowsShape {
     float epsilon;
 };
 
-template<typename T, typename W, bool ADD>
-void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *w, const Residual<ADD> &res, hipStream_t stream) {
+// Weight element type -> kind; negative when the type is not supported.
+inline int weight_kind(amd::Elem w_elem) {
+    switch (w_elem) {
+        case amd::Elem::F32: return kWKindF32;
+        case amd::Elem::F16: return kWKindF16;
+        case amd::Elem::BF16: return kWKindBF16;
+        default: return -1;
+    }
+}
+
+template<typename T, bool ADD>
+void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *w, int w_kind, const Residual<ADD> &res, hipStream_t stream) {
     auto *py = static_cast<uint16_t *>(y);
     auto *px = static_cast<const uint16_t *>(x);
     const uint64_t n = desc.n, d = desc.d;
@@ -292,8 +485,43 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     }
     if (!vec_ok) {
         const uint64_t cap = static_cast<uint64_t>(desc.cu_count) * 8;
-        rms_norm_generic<T, W, ADD><<<static_cast<unsigned>(n < cap ? n : cap), 256, 0, stream>>>(
-            py, px, w, n, d, desc.stride_y, desc.stride_x, desc.epsilon, res);
+        rms_norm_generic<T, ADD><<<static_cast<unsigned>(n < cap ? n : cap), 256, 0, stream>>>(
+            py, px, w, w_kind, n, d, desc.stride_y, desc.stride_x, desc.epsilon, res);
+        return;
+    }
+
+    const bool through_once = n * d * sizeof(uint16_t) >= kWriteThroughBytes;
+    if (const long r1 = amd::tune("RMS_ONCE", 0); r1 != 0 && nvec <= 4096) {// experiment: one pass in dispatch order, r1 rows per workgroup
+        const uint64_t grid1 = ceil_div(n, static_cast<uint64_t>(r1));
+        const bool thr = amd::tune("RMS_THROUGH", through_once ? 1 : 0) != 0;
+#define RMS_ONCE_GO(BS, NV, R, E, TH)                                                                              \
+    rms_norm_once<T, BS, NV, R, E, TH, ADD><<<static_cast<unsigned>(grid1), BS, 0, stream>>>(                      \
+        py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res)
+#define RMS_ONCE_R(BS, NV, R)                                                                                      \
+    do {                                                                                                           \
+        const bool exact = nvec == static_cast<uint64_t>(BS) * NV;                                                 \
+        if (exact && thr) RMS_ONCE_GO(BS, NV, R, true, true);                                                      \
+        else if (exact) RMS_ONCE_GO(BS, NV, R, true, false);                                                       \
+        else if (thr) RMS_ONCE_GO(BS, NV, R, false, true);                                                         \
+        else RMS_ONCE_GO(BS, NV, R, false, false);                                                                 \
+    } while (0)
+#define RMS_ONCE(BS, NV)                                                                                           \
+    do {                                                                                                           \
+        if (r1 == 1) RMS_ONCE_R(BS, NV, 1);                                                                        \
+        else RMS_ONCE_R(BS, NV, 2);                                                                                \
+    } while (0)
+        const long bs1 = amd::tune("RMS_BS", 0);
+        if (nvec <= 64) RMS_ONCE(64, 1);
+        else if (nvec <= 256) RMS_ONCE(256, 1);
+        else if (nvec <= 512) RMS_ONCE(256, 2);
+        else if (nvec <= 1024 && bs1 == 512) RMS_ONCE(512, 2);
+        else if (nvec <= 1024 && bs1 == 1024) RMS_ONCE(1024, 1);
+        else if (nvec <= 1024) RMS_ONCE(256, 4);
+        else if (nvec <= 2048) RMS_ONCE(512, 4);
+        else RMS_ONCE(1024, 4);
+#undef RMS_ONCE
+#undef RMS_ONCE_R
+#undef RMS_ONCE_GO
         return;
     }
 
@@ -309,6 +537,7 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // bytes in flight per workgroup, so they get proportionally more of them.
     uint64_t per_cu = ceil_div(32 * 1024, d * sizeof(uint16_t));
     per_cu = per_cu < 2 ? 2 : (per_cu > 16 ? 16 : per_cu);
+    per_cu = static_cast<uint64_t>(amd::tune("RMS_PER_CU", static_cast<long>(per_cu)));
     int home = kWLds;
     if (lds_bytes <= lds_limit && lds_bytes <= 64 * 1024) {
         const uint64_t fit = (160 * 1024) / (lds_bytes + 256);// 160 KiB of LDS per compute unit
@@ -317,34 +546,37 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         home = kWGlobal;
     }
     uint64_t grid = static_cast<uint64_t>(desc.cu_count) * per_cu;
-    if (n <= grid) {
+    if (n <= grid || amd::tune("RMS_ONESHOT", 0)) {
         grid = n;
         home = kWGlobal;// one row per workgroup: staging would only add a pass
     }
+    // rows of a workgroup: blockIdx.x, + grid, + 2*grid, ...
+    uint64_t first_mul = 1, hop = grid, span = n;
+    if (const long r = amd::tune("RMS_BLOCKED", 0); r > 0 && home == kWLds) {// experiment: r consecutive rows per workgroup
+        grid = ceil_div(n, static_cast<uint64_t>(r));
+        first_mul = span = static_cast<uint64_t>(r);
+        hop = 1;
+    }
 
+    // Large outputs are written through L2; the kernels that re-read the
+    // weights from memory per row exist in one form only (inexact row length,
+    // plain non-temporal stores): they serve one-row workgroups and rows too
+    // long for LDS, where neither refinement is measurable.
     const bool through = n * d * sizeof(uint16_t) >= kWriteThroughBytes;
-#define RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, EXACT)                                                                      \
-    do {                                                                                                                \
-        if (through)                                                                                                    \
-            rms_norm_rows<T, W, BS, NV, HOME, EXACT, true, ADD><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(      \
-                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res);                \
-        else                                                                                                            \
-            rms_norm_rows<T, W, BS, NV, HOME, EXACT, false, ADD><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(     \
-                py, px, w, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res);                \
-    } while (0)
-#define RMS_LAUNCH_HOME(BS, NV, HOME, LDS)                                                                              \
-    do {                                                                                                                \
-        if (nvec == static_cast<uint64_t>(BS) * NV) RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, true);                          \
-        else RMS_LAUNCH_EXACT(BS, NV, HOME, LDS, false);                                                                \
-    } while (0)
-#define RMS_LAUNCH(BS, NV)                                                                                              \
-    do {                                                                                                                \
-        if (home == kWLds) RMS_LAUNCH_HOME(BS, NV, kWLds, lds_bytes);                                                   \
-        else RMS_LAUNCH_HOME(BS, NV, kWGlobal, 0);                                                                      \
+#define RMS_GO(BS, NV, HOME, LDS, EXACT, THROUGH)                                                                      \
+    rms_norm_rows<T, BS, NV, HOME, EXACT, THROUGH, ADD><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(             \
+        py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res)
+#define RMS_LAUNCH(BS, NV)                                                                                             \
+    do {                                                                                                               \
+        const bool exact = nvec == static_cast<uint64_t>(BS) * NV;                                                     \
+        if (home != kWLds) RMS_GO(BS, NV, kWGlobal, 0, false, false);                                                  \
+        else if (exact && through) RMS_GO(BS, NV, kWLds, lds_bytes, true, true);                                       \
+        else if (exact) RMS_GO(BS, NV, kWLds, lds_bytes, true, false);                                                 \
+        else if (through) RMS_GO(BS, NV, kWLds, lds_bytes, false, true);                                               \
+        else RMS_GO(BS, NV, kWLds, lds_bytes, false, false);                                                           \
     } while (0)
 
     if (nvec <= 64) RMS_LAUNCH(64, 1);
-    else if (nvec <= 128) RMS_LAUNCH(128, 1);
     else if (nvec <= 256) RMS_LAUNCH(256, 1);
     else if (nvec <= 512) RMS_LAUNCH(256, 2);
     else if (nvec <= 1024) RMS_LAUNCH(256, 4);// d = 8192: 512x2 measures the same, 1024x1 is 8 % slower
@@ -352,28 +584,10 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     else if (nvec <= 4096) RMS_LAUNCH(1024, 4);
     else RMS_LAUNCH(1024, 8);
 #undef RMS_LAUNCH
-#undef RMS_LAUNCH_HOME
-#undef RMS_LAUNCH_EXACT
+#undef RMS_GO
 }
 
-// Weight element type -> kernel family.  False when the type is not supported.
-template<typename T, bool ADD>
-bool launch_by_weight(amd::Elem w_elem, const RowsShape &desc, void *y, const void *x, const void *w, const Residual<ADD> &res, hipStream_t s) {
-    switch (w_elem) {
-        case amd::Elem::F32:
-            launch_rms_norm<T, WF32, ADD>(desc, y, x, w, res, s);
-            return true;
-        case amd::Elem::F16:
-            launch_rms_norm<T, W16<amd::F16Ref>, ADD>(desc, y, x, w, res, s);
-            return true;
-        case amd::Elem::BF16:
-            launch_rms_norm<T, W16<amd::BF16Rne>, ADD>(desc, y, x, w, res, s);
-            return true;
-        default:
-            return false;
-    }
-}
-
+}// namespace
 }// namespace rms_norm_kernels
 
 #endif

@@ -15,7 +15,9 @@
 // the table rows of a token are fetched once per lane, through the caches, and
 // reused for every head that lane rotates.  (Staging the rows in LDS with one
 // head per lane was measured on MI355X and is slower: 52.7 against 48.9 us at
-// q = [8192, 64, 128] bf16.)
+// q = [8192, 64, 128] bf16.)  One pass, one tile per workgroup, in dispatch
+// order: workgroups that loop over tiles with the next tile's loads in flight
+// were measured at every shape of the benchmark and are never faster.
 #include "../../../devices/amd/kernel_amd.h"
 #include "rotary_embedding_amd.h"
 
@@ -48,10 +50,11 @@ __device__ __forceinline__ Idx first_lane(Idx v) {
 // lanes of a wavefront cover consecutive 16-byte pieces of consecutive heads.
 // Lane (g, cv) rotates heads g, g+G, g+2G, ... (G = number of head groups):
 // at every step the wavefront's accesses are again to neighbouring heads.
-// BUFST: results are written through L2 by buffer stores relative to the
-// wavefront's first token (see StreamOut); the host selects it for large
-// outputs when strides are non-negative and the 64 tokens a wavefront can span
-// fit a 32-bit byte offset.
+//
+// rope_vec is the general form of this map - any item count (Idx may be 64
+// bits wide), head counts that HPT does not divide - and serves what
+// rope_once below does not take.  BUFST: results are written through L2 by
+// buffer stores relative to the wavefront's first token (see StreamOut).
 template<typename T, typename Idx, int HPT, bool BUFST>
 __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
                                                    uint64_t total_items, Idx items_per_token, Idx vecs_per_head, Idx groups,
@@ -105,181 +108,71 @@ __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *
     }
 }
 
-// The same lane-to-data map as rope_vec, as a looping kernel: a workgroup
-// walks tiles of kBlock work items and always has the next tile's loads (t
-// and table rows) in flight while it rotates and stores the current one.  All
-// loads are unconditional - items or heads past the end are redirected to the
-// last valid one and simply not stored - so the compiler can count the loads
-// in flight and wait for the current tile only.
-template<typename T, int HPT>
-struct RopeTile {
-    u32x4 tv[HPT];
-    f32x4 s_lo, s_hi, c_lo, c_hi;
-    uint16_t *base;
-    uint16_t *out_base;// wavefront-uniform: the first lane's token
-    uint32_t off;      // this lane's byte offset from out_base, head 0
-    uint32_t g;
-    bool live;
-};
-
-template<typename T, typename Idx, int HPT, bool BUFST>
-__global__ __launch_bounds__(kBlock) void rope_vec_loop(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
-                                                        uint64_t total_items, Idx items_per_token, Idx vecs_per_head, Idx groups,
-                                                        uint32_t heads, uint32_t head_dim, int64_t stride_token, int64_t stride_head) {
-    const uint64_t tiles = (total_items + kBlock - 1) / kBlock;
-    auto fetch = [&](uint64_t tile, RopeTile<T, HPT> &r) {
-        const uint64_t item64 = tile * kBlock + threadIdx.x;
-        r.live = item64 < total_items;
-        const Idx item = static_cast<Idx>(r.live ? item64 : total_items - 1);
-        const Idx token = item / items_per_token;
-        const Idx rem = item - token * items_per_token;
-        const Idx g = rem / vecs_per_head;
-        const Idx cv = rem - g * vecs_per_head;
-        r.g = static_cast<uint32_t>(g);
-        r.base = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(cv) * 8;
-        if constexpr (BUFST) {
-            const Idx token0 = first_lane(token);
-            r.out_base = t + static_cast<int64_t>(token0) * stride_token;
-            r.off = static_cast<uint32_t>(token - token0) * static_cast<uint32_t>(stride_token) * 2 + static_cast<uint32_t>(cv) * 16;
-        }
-#pragma unroll
-        for (int i = 0; i < HPT; ++i) {
-            uint32_t h = r.g + i * static_cast<uint32_t>(groups);
-            h = h < heads ? h : heads - 1;
-            r.tv[i] = ld16_stream(r.base + static_cast<int64_t>(h) * stride_head);
-        }
-        const uint64_t row = pos[token] * head_dim + static_cast<uint64_t>(cv) * 8;
-        r.s_lo = ld16f(sin_t + row), r.s_hi = ld16f(sin_t + row + 4);
-        r.c_lo = ld16f(cos_t + row), r.c_hi = ld16f(cos_t + row + 4);
-    };
-    auto rotate = [&](const RopeTile<T, HPT> &r) {
-        const float sn[8] = {r.s_lo.x, r.s_lo.y, r.s_lo.z, r.s_lo.w, r.s_hi.x, r.s_hi.y, r.s_hi.z, r.s_hi.w};
-        const float cs[8] = {r.c_lo.x, r.c_lo.y, r.c_lo.z, r.c_lo.w, r.c_hi.x, r.c_hi.y, r.c_hi.z, r.c_hi.w};
-        const StreamOut<true> out(BUFST ? r.out_base : t);
-#pragma unroll
-        for (int i = 0; i < HPT; ++i) {
-            const uint32_t h = r.g + i * static_cast<uint32_t>(groups);
-            float f[8], o[8];
-            widen8<T>(r.tv[i], f);
-#pragma unroll
-            for (int k = 0; k < 8; k += 2) {
-                const float a = f[k], b = f[k + 1];
-                const float ac = a * cs[k], bs = b * sn[k];
-                const float as = a * sn[k + 1], bc = b * cs[k + 1];
-                o[k] = ac - bs;
-                o[k + 1] = as + bc;
-            }
-            const u32x4 packed = narrow8<T>(o);
-            if (r.live && h < heads) {
-                if constexpr (BUFST) {
-                    out.st16(r.off + h * static_cast<uint32_t>(stride_head) * 2, packed);
-                } else {
-                    st16_stream(r.base + static_cast<int64_t>(h) * stride_head, packed);
-                }
-            }
-        }
-    };
-
-    uint64_t tile = blockIdx.x;
-    if (tile >= tiles) return;
-    const uint64_t hop = gridDim.x;
-    RopeTile<T, HPT> a, b;
-    fetch(tile, a);
-    while (true) {
-        if (tile + hop >= tiles) {
-            rotate(a);
-            break;
-        }
-        fetch(tile + hop, b);
-        rotate(a);
-        tile += hop;
-        if (tile + hop >= tiles) {
-            rotate(b);
-            break;
-        }
-        fetch(tile + hop, a);
-        rotate(b);
-        tile += hop;
+// One pass, one tile of BS work items per workgroup, in the order the
+// dispatcher hands workgroups out.  The position is requested first, then the
+// data, then - as soon as the position is there, while the data is still on
+// its way (loads return in issue order) - the table rows.  UNI: a token's work
+// items are a multiple of BS, so a workgroup lies inside one token and its
+// position and table base are found with scalar arithmetic and scalar loads.
+// The head count is a multiple of HPT (every lane's heads exist): nothing is
+// predicated, so no load can sink into a branch behind the wait for another.
+template<typename T, int BS, int HPT, bool BUFST, bool UNI>
+__global__ __launch_bounds__(BS) void rope_once(uint16_t *__restrict__ t, const uint64_t *__restrict__ pos,
+                                                const float *__restrict__ sin_t, const float *__restrict__ cos_t,
+                                                uint32_t total_items, uint32_t items_per_token, uint32_t vecs_per_head, uint32_t groups,
+                                                uint32_t head_dim, int64_t stride_token, int64_t stride_head) {
+    uint32_t token, rem;
+    if constexpr (UNI) {
+        const uint32_t item0 = blockIdx.x * BS;
+        token = item0 / items_per_token;
+        rem = item0 - token * items_per_token + threadIdx.x;
+    } else {
+        const uint32_t item = blockIdx.x * BS + threadIdx.x;
+        if (item >= total_items) return;
+        token = item / items_per_token;
+        rem = item - token * items_per_token;
     }
-}
+    const uint32_t g = rem / vecs_per_head;
+    const uint32_t cv = rem - g * vecs_per_head;
+    const uint64_t p = pos[token];
 
-// One token per tile: when a token's work items fill a workgroup exactly
-// (heads / HPT * head_dim / 8 == kBlock), a lane's head group and column group
-// never change, the token is the same for the whole workgroup, and its
-// position and table rows are found with scalar loads and scalar arithmetic.
-// Nothing is predicated.  Workgroups loop over tokens with the next token's
-// loads in flight, as rope_vec_loop does.
-template<typename T, int HPT>
-struct RopeTokenTile {
+    uint16_t *base = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(cv) * 8;
     u32x4 tv[HPT];
-    f32x4 s_lo, s_hi, c_lo, c_hi;
-    uint16_t *base;// the token's row: wavefront-uniform
-};
+#pragma unroll
+    for (int i = 0; i < HPT; ++i) {
+        const uint32_t h = g + i * groups;
+        tv[i] = ld16_stream(base + static_cast<int64_t>(h) * stride_head);
+    }
+    __builtin_amdgcn_sched_barrier(0);// the data loads leave before anything waits for the position
 
-template<typename T, int HPT, bool BUFST>
-__global__ __launch_bounds__(kBlock) void rope_token_loop(uint16_t *__restrict__ t, const uint64_t *__restrict__ pos,
-                                                          const float *__restrict__ sin_t, const float *__restrict__ cos_t,
-                                                          uint64_t tokens, uint32_t vecs_per_head, uint32_t groups, uint32_t head_dim,
-                                                          int64_t stride_token, int64_t stride_head) {
-    const uint32_t g = threadIdx.x / vecs_per_head;
-    const uint32_t cv = threadIdx.x - g * vecs_per_head;
-    int64_t lane_off[HPT];// elements from the token's row to this lane's vector of head g + i * groups
-#pragma unroll
-    for (int i = 0; i < HPT; ++i) lane_off[i] = static_cast<int64_t>(g + i * groups) * stride_head + static_cast<int64_t>(cv) * 8;
+    const uint64_t row = p * head_dim + static_cast<uint64_t>(cv) * 8;
+    const f32x4 s_lo = ld16f(sin_t + row), s_hi = ld16f(sin_t + row + 4);
+    const f32x4 c_lo = ld16f(cos_t + row), c_hi = ld16f(cos_t + row + 4);
+    const float sn[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+    const float cs[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
 
-    auto fetch = [&](uint64_t token, RopeTokenTile<T, HPT> &r) {
-        r.base = t + static_cast<int64_t>(token) * stride_token;
+    // buffer stores address from the wavefront's first token
+    const uint32_t token0 = UNI || !BUFST ? token : first_lane(token);
+    const StreamOut<true> out(t + static_cast<int64_t>(token0) * stride_token);
+    const uint32_t off = (token - token0) * static_cast<uint32_t>(stride_token) * 2 + cv * 16;
 #pragma unroll
-        for (int i = 0; i < HPT; ++i) r.tv[i] = ld16_stream(r.base + lane_off[i]);
-        const uint64_t row = pos[token] * head_dim;
-        const float *sp = sin_t + row + cv * 8, *cp = cos_t + row + cv * 8;
-        r.s_lo = ld16f(sp), r.s_hi = ld16f(sp + 4);
-        r.c_lo = ld16f(cp), r.c_hi = ld16f(cp + 4);
-    };
-    auto rotate = [&](const RopeTokenTile<T, HPT> &r) {
-        const float sn[8] = {r.s_lo.x, r.s_lo.y, r.s_lo.z, r.s_lo.w, r.s_hi.x, r.s_hi.y, r.s_hi.z, r.s_hi.w};
-        const float cs[8] = {r.c_lo.x, r.c_lo.y, r.c_lo.z, r.c_lo.w, r.c_hi.x, r.c_hi.y, r.c_hi.z, r.c_hi.w};
-        const StreamOut<true> out(r.base);
+    for (int i = 0; i < HPT; ++i) {
+        const uint32_t h = g + i * groups;
+        float f[8], r[8];
+        widen8<T>(tv[i], f);
 #pragma unroll
-        for (int i = 0; i < HPT; ++i) {
-            float f[8], o[8];
-            widen8<T>(r.tv[i], f);
-#pragma unroll
-            for (int k = 0; k < 8; k += 2) {
-                const float a = f[k], b = f[k + 1];
-                const float ac = a * cs[k], bs = b * sn[k];
-                const float as = a * sn[k + 1], bc = b * cs[k + 1];
-                o[k] = ac - bs;
-                o[k + 1] = as + bc;
-            }
-            if constexpr (BUFST) {
-                out.st16(static_cast<uint32_t>(lane_off[i]) * 2, narrow8<T>(o));
-            } else {
-                st16_stream(r.base + lane_off[i], narrow8<T>(o));
-            }
+        for (int k = 0; k < 8; k += 2) {
+            const float a = f[k], b = f[k + 1];
+            const float ac = a * cs[k], bs = b * sn[k];
+            const float as = a * sn[k + 1], bc = b * cs[k + 1];
+            r[k] = ac - bs;
+            r[k + 1] = as + bc;
         }
-    };
-
-    uint64_t token = blockIdx.x;
-    if (token >= tokens) return;
-    const uint64_t hop = gridDim.x;
-    RopeTokenTile<T, HPT> a, b;
-    fetch(token, a);
-    while (true) {
-        if (token + hop >= tokens) {
-            rotate(a);
-            break;
+        if constexpr (BUFST) {
+            out.st16(off + h * static_cast<uint32_t>(stride_head) * 2, narrow8<T>(r));
+        } else {
+            st16_stream(base + static_cast<int64_t>(h) * stride_head, narrow8<T>(r));
         }
-        fetch(token + hop, b);
-        rotate(a);
-        token += hop;
-        if (token + hop >= tokens) {
-            rotate(b);
-            break;
-        }
-        fetch(token + hop, a);
-        rotate(b);
-        token += hop;
     }
 }
 
@@ -307,85 +200,84 @@ __global__ __launch_bounds__(kBlock) void rope_pairs(uint16_t *t, const uint64_t
 template<typename T, typename Idx>
 void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, const float *sn, const float *cs, hipStream_t stream) {
     const uint64_t vph = d.head_dim / 8;
-    const int hpt = d.heads >= kHeadsPerLane ? kHeadsPerLane : (d.heads >= 2 ? 2 : 1);
-    const uint64_t groups = ceil_div(d.heads, hpt);
-    const uint64_t ipt = groups * vph;
-    const uint64_t total = d.tokens * ipt;
-    const unsigned grid = static_cast<unsigned>(ceil_div(total, kBlock));
     // Large outputs are written through L2 with buffer stores, which address
     // 32 bits from the first token of a wavefront (it spans at most 64 tokens).
     const bool bufst = d.tokens * d.heads * d.head_dim * sizeof(uint16_t) >= kWriteThroughBytes &&
                        d.stride_token >= 0 && d.stride_head >= 0 &&
                        static_cast<uint64_t>(d.stride_token) < (1ull << 23) &&
                        d.heads * static_cast<uint64_t>(d.stride_head) < (1ull << 30) && d.head_dim < (1ull << 24);
-    // Enough tiles to keep every compute unit looping: the prefetching form.
-    // Measured on MI355X (256 compute units): q [8192,64,128] bf16, 8192 tiles,
-    // 47.0 us looping with 2 workgroups per unit against 48.5 us one tile per
-    // workgroup; [4096,32,128] fp16, 2048 tiles, 14.1 us (4 per unit) against
-    // 16.8 us; k [8192,8,128], 1024 tiles, is faster one tile per workgroup
-    // (9.7 against 10.5 us) and stays on rope_vec (with two heads per lane, and
-    // so twice the workgroups, it takes 10.8 us).  Workgroups of 64 or 128
-    // lanes, one tile each, measure the same as 256 for all three shapes, and
-    // so does a 2-D grid with the token in blockIdx.y (position and table base
-    // then come through scalar loads): 47.3 us for q.  With table loads and
-    // arithmetic removed the looping form takes 44.7 us for q, so they cost
-    // 1.7 us; an out-of-place copy of the same strided rows takes 41.9 us.
-    // A token per tile, when some number of heads per lane makes a token fill a
-    // workgroup exactly and there are tokens enough to loop over.  Measured on
-    // MI355X: q [8192,64,128] bf16 45.1 us with 2 workgroups per compute unit
-    // (46.3 with 4, 45.9 with 8) against 46.4 us for rope_vec_loop, whose lanes
-    // recompute token, head group and column for every tile; [4096,32,128]
-    // fp16 (2 heads per lane) 14.1 us either way.
-    if (sizeof(Idx) == 4 && d.tokens >= 8ull * d.cu_count) {
-        int h2 = 0;
-        for (int cand : {4, 2, 8}) {// not 1: a lane that rotates one head loads four table vectors for it ([32768,32,64]: 62 us against 47)
-            if (h2 == 0 && d.heads % cand == 0 && (d.heads / cand) * vph == kBlock) h2 = cand;
-        }
-        if (h2 != 0) {
-            const uint64_t cap2 = static_cast<uint64_t>(d.cu_count) * 2;
-            const unsigned g2 = static_cast<unsigned>(d.tokens < cap2 ? d.tokens : cap2);
-            const bool b2 = bufst && d.heads * static_cast<uint64_t>(d.stride_head) < (1ull << 30);
-#define ROPE_TL(HPT, B) rope_token_loop<T, HPT, B><<<g2, kBlock, 0, stream>>>(t, pos, sn, cs, d.tokens, static_cast<uint32_t>(vph), static_cast<uint32_t>(d.heads / HPT), static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
-            if (b2) { if (h2 == 4) ROPE_TL(4, true); else if (h2 == 2) ROPE_TL(2, true); else ROPE_TL(8, true); }
-            else { if (h2 == 4) ROPE_TL(4, false); else if (h2 == 2) ROPE_TL(2, false); else ROPE_TL(8, false); }
-#undef ROPE_TL
-            return;
+
+    // Heads per lane.  Two things pull against each other: every lane fetches
+    // the 64 bytes of table values of its column group whatever the number of
+    // heads it rotates with them, so few heads per lane multiply the table
+    // traffic through L2; many heads per lane leave few lanes.  A token whose
+    // lanes fill a workgroup exactly (UNI) is best when the head count allows
+    // it; a handful of heads goes to one lane per column group.  Measured on
+    // MI355X, one pass (rope_once), 256 lanes:
+    //   q [8192,64,128] bf16 in [8192,80,128]:  2/4/8 heads per lane 43.4 / 43.4 / 46.6 us
+    //                                           (45.5 us for workgroups looping over tokens with prefetch)
+    //   k [8192,8,128] bf16:                    2/4/8 heads per lane 10.5 / 10.6 / 8.65 us (9.05 the position loaded last)
+    //   [4096,32,128] fp16 in [4096,96,128]:    2/4/8 heads per lane 14.1 / 14.4 / 14.3 us
+    // Workgroups of 64 or 128 lanes measure the same or worse (k: 8.6, q: 44.7-48.7 us).
+    int hpt = 1;
+    for (int cand : {8, 4, 2}) {// the largest that divides the head count and still leaves a workgroup's worth of lanes per token
+        if (d.heads % cand == 0 && (d.heads / cand) * vph >= kBlock) {
+            hpt = cand;
+            break;
         }
     }
-    if (grid >= 8u * static_cast<unsigned>(d.cu_count)) {
-        const uint64_t per_cu = grid >= 16u * static_cast<unsigned>(d.cu_count) ? 2 : 4;
-        const uint64_t cap = static_cast<uint64_t>(d.cu_count) * per_cu;
-        const unsigned lgrid = static_cast<unsigned>(grid < cap ? grid : cap);
-#define ROPE_LAUNCH_LOOP(HPT, B)                                                                                                    \
-    rope_vec_loop<T, Idx, HPT, B><<<lgrid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph), \
-                                                                static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),           \
-                                                                static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
-        if (bufst) {
-            if (hpt == 4) ROPE_LAUNCH_LOOP(4, true);
-            else if (hpt == 2) ROPE_LAUNCH_LOOP(2, true);
-            else ROPE_LAUNCH_LOOP(1, true);
-        } else {
-            if (hpt == 4) ROPE_LAUNCH_LOOP(4, false);
-            else if (hpt == 2) ROPE_LAUNCH_LOOP(2, false);
-            else ROPE_LAUNCH_LOOP(1, false);
+    if (hpt == 1) {// fewer lanes than a workgroup per token whatever is chosen: as many heads per lane as divide the count
+        for (int cand : {8, 4, 2}) {
+            if (d.heads % cand == 0) {
+                hpt = cand;
+                break;
+            }
         }
-#undef ROPE_LAUNCH_LOOP
+    }
+    if (const long forced = amd::tune("ROPE_HPT", 0); forced > 0 && d.heads % forced == 0) hpt = static_cast<int>(forced);
+    const uint64_t groups = d.heads / hpt;
+    const uint64_t ipt = groups * vph;
+    const uint64_t total = d.tokens * ipt;
+    if (sizeof(Idx) == 4 && total < (1ull << 31) && amd::tune("ROPE_ONCE", 1)) {
+        const bool uni = ipt % kBlock == 0;
+        const unsigned grid = static_cast<unsigned>(ceil_div(total, kBlock));
+        const bool b1 = bufst && static_cast<uint64_t>(kWave) * static_cast<uint64_t>(d.stride_token) * 2 +
+                                         d.heads * static_cast<uint64_t>(d.stride_head) * 2 < (1ull << 31);
+#define ROPE_ONCE_GO(HPT, B, U)                                                                                              \
+    rope_once<T, kBlock, HPT, B, U><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, static_cast<uint32_t>(total),                \
+                                                                 static_cast<uint32_t>(ipt), static_cast<uint32_t>(vph),      \
+                                                                 static_cast<uint32_t>(groups), static_cast<uint32_t>(d.head_dim), \
+                                                                 d.stride_token, d.stride_head)
+#define ROPE_ONCE_BU(HPT)                                \
+    do {                                                 \
+        if (b1 && uni) ROPE_ONCE_GO(HPT, true, true);    \
+        else if (b1) ROPE_ONCE_GO(HPT, true, false);     \
+        else if (uni) ROPE_ONCE_GO(HPT, false, true);    \
+        else ROPE_ONCE_GO(HPT, false, false);            \
+    } while (0)
+        if (hpt == 8) ROPE_ONCE_BU(8);
+        else if (hpt == 4) ROPE_ONCE_BU(4);
+        else if (hpt == 2) ROPE_ONCE_BU(2);
+        else ROPE_ONCE_BU(1);
+#undef ROPE_ONCE_BU
+#undef ROPE_ONCE_GO
         return;
     }
-#define ROPE_LAUNCH(HPT, B)                                                                                                   \
-    rope_vec<T, Idx, HPT, B><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, total, static_cast<Idx>(ipt), static_cast<Idx>(vph), \
-                                                          static_cast<Idx>(groups), static_cast<uint32_t>(d.heads),           \
-                                                          static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
-    if (bufst) {
-        if (hpt == 4) ROPE_LAUNCH(4, true);
-        else if (hpt == 2) ROPE_LAUNCH(2, true);
-        else ROPE_LAUNCH(1, true);
-    } else {
-        if (hpt == 4) ROPE_LAUNCH(4, false);
-        else if (hpt == 2) ROPE_LAUNCH(2, false);
-        else ROPE_LAUNCH(1, false);
-    }
+    // more work items than 32 bits index: the general form, lanes find their token by division
+    {
+        const int h2 = d.heads >= kHeadsPerLane ? kHeadsPerLane : (d.heads >= 2 ? 2 : 1);
+        const uint64_t g2 = ceil_div(d.heads, h2);
+        const uint64_t ipt2 = g2 * vph, total2 = d.tokens * ipt2;
+        const unsigned grid = static_cast<unsigned>(ceil_div(total2, kBlock));
+#define ROPE_LAUNCH(HPT)                                                                                                          \
+    rope_vec<T, Idx, HPT, false><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, total2, static_cast<Idx>(ipt2), static_cast<Idx>(vph), \
+                                                              static_cast<Idx>(g2), static_cast<uint32_t>(d.heads),                \
+                                                              static_cast<uint32_t>(d.head_dim), d.stride_token, d.stride_head)
+        if (h2 == 4) ROPE_LAUNCH(4);
+        else if (h2 == 2) ROPE_LAUNCH(2);
+        else ROPE_LAUNCH(1);
 #undef ROPE_LAUNCH
+    }
 }
 
 template<typename T>

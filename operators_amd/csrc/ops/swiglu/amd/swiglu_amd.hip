@@ -173,7 +173,7 @@ void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const v
     const uint64_t nvec = n / 8;
     const uint64_t vpr = d.di / 8;
     const uint64_t want = ceil_div(nvec, kWave);
-    const uint64_t max_grid = 0x7FFFFFFFull;
+    const uint64_t max_grid = max_grid_1d(kWave);
     const unsigned grid = static_cast<unsigned>(want < max_grid ? want : max_grid);
     // One row, or every row stride equal to the width: the tensors are dense.
     const bool dense = d.rows == 1 || (d.stride_a == di && d.stride_b == di && d.stride_c == di);

@@ -400,6 +400,9 @@ def status_cases():
     rec("rearrange", [T("f16", (2, 2, 3, 4, 8)), T("f16", (2, 2, 3, 4, 8), (400, 192, 64, 10, 1))])  # dim 1 does not nest in dim 0
     rec("rearrange", [T("bf16", (4, 64)), T("bf16", (4, 64))])
     rec("rearrange", [T("u8", (4, 64)), T("u8", (4, 64), (100, 1))])
+    rec("rearrange", [T("f16", (0, 4)), T("f16", (0, 4))])                      # an extent of zero: accepted, nothing to copy
+    rec("rearrange", [T("f16", (3, 0, 8)), T("f16", (3, 0, 8), (64, 8, 1))])
+    rec("rearrange", [T("f16", (4, 0)), T("f16", (4, 0))])
     # RandomSample (result, probs)
     rec("random_sample", [T("u64", (1,)), T("f16", (512,))])
     rec("random_sample", [T("u64", (4,)), T("f16", (512,))])         # rank 1 of any length passes

@@ -59,7 +59,7 @@ SHAPES = [
     # c, a, b
     ((1000003,), (1000003,), (1000003,)),           # flat, odd length: vector body + tail
     ((257, 4096), (257, 4096), (4096,)),            # residual-style leading broadcast
-    ((6, 1, 40), (6, 1, 40), (1, 5, 1)),            # NOT broadcastable onto c -> skipped below
+    ((6, 5, 40), (6, 1, 40), (1, 5, 1)),            # both operands broadcast, along different dims
     ((7, 33, 16), (7, 1, 16), (33, 1)),             # alternating broadcast, inner vectorisable
     ((7, 33, 15), (7, 1, 15), (33, 1)),             # same with an odd inner extent: element path
     ((5, 6, 7, 8), (5, 6, 7, 8), (1,)),             # scalar-like operand
@@ -73,8 +73,7 @@ SHAPES = [
 def test_against_oracle(ctx, dt, case):
     cs, as_, bs = SHAPES[case]
     spec = lambda s: oracle.Spec(dt, s)  # noqa: E731
-    if oracle.add_check(spec(cs), spec(as_), spec(bs), allow_bf16=True) != 0:
-        pytest.skip("shape triple is not a valid broadcast (covered by the status tests)")
+    assert oracle.add_check(spec(cs), spec(as_), spec(bs), allow_bf16=True) == 0, "every triple of SHAPES is a valid broadcast"
     rng = np.random.default_rng(100 + case)
     a = oracle.encode(rng.standard_normal(as_).astype(np.float32) * 3, dt)
     b = oracle.encode(rng.standard_normal(bs).astype(np.float32) * 3, dt)

@@ -119,3 +119,28 @@ def test_status_codes_match_reference(ctx):
             assert lib.infiniopDestroyRearrangeDescriptor(d) == 0
         for x in descs:
             lib.infiniopDestroyTensorDescriptor(x)
+
+
+@pytest.mark.parametrize("shape,strides", [((0, 4), None), ((3, 0, 8), (64, 8, 1)), ((4, 0), None), ((2, 3, 0, 8), (96, 32, 8, 1))])
+def test_zero_extent_copies_nothing(ctx, shape, strides):
+    """An extent of zero anywhere: the descriptor is accepted (as by the
+    reference, whose loops then run zero times) and the call leaves the
+    destination as it was."""
+    import ctypes
+
+    import torch
+
+    from operators_amd import F16, infiniopRearrangeDescriptor_t, make_descriptor
+
+    lib = ctx.lib
+    dst_d, src_d = make_descriptor(lib, shape, None, F16), make_descriptor(lib, shape, strides, F16)
+    d = infiniopRearrangeDescriptor_t()
+    assert lib.infiniopCreateRearrangeDescriptor(ctx.handle, ctypes.byref(d), dst_d, src_d) == 0
+    dst = torch.full((64,), 7.0, dtype=torch.float16, device="cuda")
+    src = torch.full((64,), 3.0, dtype=torch.float16, device="cuda")
+    assert lib.infiniopRearrange(d, dst.data_ptr(), src.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert bool((dst == 7.0).all())
+    assert lib.infiniopDestroyRearrangeDescriptor(d) == 0
+    lib.infiniopDestroyTensorDescriptor(dst_d)
+    lib.infiniopDestroyTensorDescriptor(src_d)
