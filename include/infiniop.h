@@ -379,6 +379,18 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetRandomSampleWorkspaceSize
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRandomSample(
     infiniopRandomSampleDescriptor_t desc, void *workspace, uint64_t workspace_size,
     void *result, void const *probs, float random_val, float topp, int topk, float temperature, void *stream);
+/* no counterpart in the reference.  For callers that cannot allocate device
+ * memory or hand over a workspace (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): infiniopRandomSample with the
+ * candidate lists of its two-launch form kept in an array of 197 376 bytes
+ * that the library holds on every GPU it runs on until the process ends.  The
+ * call allocates nothing.  Same results as infiniopRandomSample with a
+ * workspace.  Descriptors of more than 1 048 576 logits answer
+ * STATUS_BAD_PARAM (and a line on stderr).  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU, on whatever streams, race. */
+INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRandomSampleNoAlloc(
+    infiniopRandomSampleDescriptor_t desc, void *result, void const *probs,
+    float random_val, float topp, int topk, float temperature, void *stream);
 /* replaces include/ops/random_sample/random_sample.h:29 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyRandomSampleDescriptor(infiniopRandomSampleDescriptor_t desc);
 

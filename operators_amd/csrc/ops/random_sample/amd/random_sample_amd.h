@@ -20,6 +20,8 @@ constexpr int kRandomSampleMaxGroups = 48;
 constexpr int kRandomSamplePartTopk = 256;
 // vocabularies below this are sampled by one workgroup in one launch
 constexpr uint32_t kRandomSampleSplitVoc = 4096;
+// largest vocabulary the entry point without workspace and allocation serves
+constexpr uint32_t kRandomSampleNoAllocMaxVoc = 1u << 20;
 
 // What one workgroup of the first launch leaves for the second.
 struct RandomSamplePart {
@@ -46,6 +48,8 @@ infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t des
 infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspace, uint64_t workspace_size,
                                  void *result, void const *probs, float random_val, float topp, int topk,
                                  float temperature, void *stream);
+infiniopStatus_t amdRandomSampleNoAlloc(RandomSampleAmdDescriptor_t desc, void *result, void const *probs, float random_val,
+                                        float topp, int topk, float temperature, void *stream);
 infiniopStatus_t amdDestroyRandomSampleDescriptor(RandomSampleAmdDescriptor_t desc);
 
 #endif

@@ -39,6 +39,7 @@
 // anything; one in front wins); the sampling form ranks them below -Inf.
 #include "../../../devices/amd/kernel_amd.h"
 #include "random_sample_amd.h"
+#include <mutex>
 
 namespace {
 
@@ -698,7 +699,66 @@ void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
     }
 }
 
+// ---- the library's own candidate lists ----------------------------------------
+// For callers that cannot hand over a workspace they allocated: the two-launch
+// form's lists in a fixed array in device memory, one copy per GPU, held until
+// the process ends.  Host code never uses the array's name as an address (on
+// the host it is only a handle for the symbol): the address on a GPU is asked
+// for once, with that GPU current, and kept.
+constexpr uint64_t kScratchBytes = kRandomSampleMaxGroups * sizeof(RandomSamplePart) +
+                                   static_cast<uint64_t>(kRandomSampleMaxGroups) * kRandomSamplePartCap * sizeof(uint64_t);
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxGpus = 64;
+std::mutex scratch_lock;
+void *scratch_on_gpu[kMaxGpus];// null until asked for
+
+// The address of this GPU's copy; `device_id` is the current device.
+infiniopStatus_t scratch_address(int device_id, void **address) {
+    if (device_id < 0 || device_id >= kMaxGpus) {
+        return STATUS_BAD_DEVICE;
+    }
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (scratch_on_gpu[device_id] == nullptr) {
+        void *ptr = nullptr;
+        AMD_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), STATUS_EXECUTION_FAILED);
+        if (ptr == nullptr) {
+            return STATUS_EXECUTION_FAILED;
+        }
+        scratch_on_gpu[device_id] = ptr;
+    }
+    *address = scratch_on_gpu[device_id];
+    return STATUS_SUCCESS;
+}
+
 }// namespace
+
+// RandomSample without a caller-provided workspace and without any allocation:
+// the candidate lists of the two-launch form live in this library's own array
+// on the GPU.  Same results as amdRandomSample with a workspace.  Nothing in
+// the array has to be cleared between calls (the first launch writes every
+// header and every list entry the second one reads).  All calls on one GPU
+// share the array: two of them in flight at once, on any streams, race.
+infiniopStatus_t amdRandomSampleNoAlloc(RandomSampleAmdDescriptor_t desc, void *result, void const *probs, float random_val,
+                                        float topp, int topk, float temperature, void *stream) {
+    if (desc->voc > kRandomSampleNoAllocMaxVoc) {
+        std::fprintf(stderr, "infiniop[amd-gpu]: RandomSampleNoAlloc serves at most %u logits, the descriptor has %u; "
+                             "use infiniopRandomSample with a workspace\n", kRandomSampleNoAllocMaxVoc, desc->voc);
+        return STATUS_BAD_PARAM;
+    }
+    if (amdRandomSampleWorkspaceBytes(*desc) > kScratchBytes) {
+        std::fprintf(stderr, "infiniop[amd-gpu]: RandomSampleNoAlloc: the lists of %u logits need %llu bytes, the library holds %llu\n",
+                     desc->voc, static_cast<unsigned long long>(amdRandomSampleWorkspaceBytes(*desc)), static_cast<unsigned long long>(kScratchBytes));
+        return STATUS_BAD_PARAM;
+    }
+    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
+    void *lists = nullptr;
+    const infiniopStatus_t st = scratch_address(desc->device_id, &lists);
+    if (st != STATUS_SUCCESS) {
+        return st;
+    }
+    return amdRandomSample(desc, lists, kScratchBytes, result, probs, random_val, topp, topk, temperature, stream);
+}
 
 // Stage 4 of RandomSample.  With topp > 0 and topk > 1 it samples, otherwise
 // it returns the first index of the maximum, as the reference does

@@ -46,6 +46,21 @@ INFINIOP_C infiniopStatus_t infiniopRandomSample(infiniopRandomSampleDescriptor_
     }
 }
 
+INFINIOP_C infiniopStatus_t infiniopRandomSampleNoAlloc(infiniopRandomSampleDescriptor_t desc, void *result, void const *probs,
+                                                        float random_val, float topp, int topk, float temperature,
+                                                        void *stream) {
+    if (desc == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
+    switch (desc->device) {
+        case DevAmdGpu:
+            return amdRandomSampleNoAlloc(reinterpret_cast<RandomSampleAmdDescriptor_t>(desc), result, probs, random_val,
+                                          topp, topk, temperature, stream);
+        default:
+            return STATUS_BAD_DEVICE;
+    }
+}
+
 INFINIOP_C infiniopStatus_t infiniopDestroyRandomSampleDescriptor(infiniopRandomSampleDescriptor_t desc) {
     if (desc == nullptr) {
         return STATUS_BAD_PARAM;

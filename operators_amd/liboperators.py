@@ -156,6 +156,7 @@ _PROTOTYPES = {
     "infiniopCreateRandomSampleDescriptor": [infiniopHandle_t, POINTER(infiniopRandomSampleDescriptor_t), infiniopTensorDescriptor_t, infiniopTensorDescriptor_t],
     "infiniopGetRandomSampleWorkspaceSize": [infiniopRandomSampleDescriptor_t, POINTER(c_uint64)],
     "infiniopRandomSample": [infiniopRandomSampleDescriptor_t, c_void_p, c_uint64, c_void_p, c_void_p, c_float, c_float, c_int, c_float, c_void_p],
+    "infiniopRandomSampleNoAlloc": [infiniopRandomSampleDescriptor_t, c_void_p, c_void_p, c_float, c_float, c_int, c_float, c_void_p],
     "infiniopDestroyRandomSampleDescriptor": [infiniopRandomSampleDescriptor_t],
     "infiniopCreateAddRMSNormDescriptor": [infiniopHandle_t, POINTER(infiniopAddRMSNormDescriptor_t)] + [infiniopTensorDescriptor_t] * 5 + [c_float],
     "infiniopGetAddRMSNormWorkspaceSize": [infiniopAddRMSNormDescriptor_t, POINTER(c_uint64)],
@@ -167,7 +168,7 @@ EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
 
 
 # Entry points of this library that the reference does not have.
-EXTENSION_SYMBOLS = tuple(n for n in _PROTOTYPES if "AddRMSNorm" in n)
+EXTENSION_SYMBOLS = tuple(n for n in _PROTOTYPES if "AddRMSNorm" in n or "NoAlloc" in n)
 
 
 def bind_prototypes(lib, extensions=True):

@@ -288,6 +288,13 @@ class RandomSamplePlan(_Plan):
                                                   random_val, topp, topk, temperature, stream))
         return result
 
+    def no_alloc(self, result, probs, random_val, topp, topk, temperature, stream=None):
+        """The same draw through the entry point that neither takes a workspace
+        nor allocates: the library's own array on the GPU carries the lists."""
+        check_error(self.lib.infiniopRandomSampleNoAlloc(self.desc, result.data_ptr(), probs.data_ptr(),
+                                                         random_val, topp, topk, temperature, stream))
+        return result
+
 
 class RearrangePlan(_Plan):
     _destroy = "infiniopDestroyRearrangeDescriptor"
