@@ -96,6 +96,15 @@ __device__ __forceinline__ bool f16_fast_ok(float v) {
 // narrow2: two floats -> one 32-bit word, with the type's rounding rule.
 struct F16Ref {
     static constexpr bool kNeedsFixup = true;
+    // two elements compared at once in their own format (v_pk_max_f16, v_pk_min_f16)
+    static constexpr bool kPackedMinMax = true;
+    typedef f16x2 pair;
+    __device__ static __forceinline__ pair as_pair(uint32_t w) { return __builtin_bit_cast(f16x2, w); }
+    __device__ static __forceinline__ pair splat(float v) { return f16x2{static_cast<_Float16>(v), static_cast<_Float16>(v)}; }
+    __device__ static __forceinline__ pair max2(pair a, pair b) { return __builtin_elementwise_max(a, b); }
+    __device__ static __forceinline__ pair min2(pair a, pair b) { return __builtin_elementwise_min(a, b); }
+    __device__ static __forceinline__ float first(pair p) { return static_cast<float>(p.x); }
+    __device__ static __forceinline__ float second(pair p) { return static_cast<float>(p.y); }
     __device__ static __forceinline__ float lo(uint32_t w) {
         return static_cast<float>(__builtin_bit_cast(f16x2, w).x);
     }
@@ -123,6 +132,8 @@ struct F16Ref {
 // (v_cvt_pk_bf16_f32 on gfx950); NaN stays NaN.
 struct BF16Rne {
     static constexpr bool kNeedsFixup = false;
+    static constexpr bool kPackedMinMax = false;// no packed bf16 comparison on this part
+    typedef uint32_t pair;
     __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
     __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
     __device__ static __forceinline__ float one(uint16_t h) {
@@ -138,6 +149,19 @@ struct BF16Rne {
         return __builtin_bit_cast(uint16_t, static_cast<__bf16>(a));
     }
 };
+
+// The integer rule applied to eight values.  Deliberately not inlined: it is
+// reached only when a value leaves the hardware pack's exact domain, and one
+// shared copy keeps the kernels that narrow several times small.
+template<typename T>
+__device__ __attribute__((noinline)) u32x4 narrow8_any(float r0, float r1, float r2, float r3, float r4, float r5, float r6, float r7) {
+    u32x4 out;
+    out.x = T::narrow2_any(r0, r1);
+    out.y = T::narrow2_any(r2, r3);
+    out.z = T::narrow2_any(r4, r5);
+    out.w = T::narrow2_any(r6, r7);
+    return out;
+}
 
 // Eight results -> one 128-bit word.  For fp16 the hardware pack is used when
 // all eight are inside its exact domain; the test is made wave-uniform with a
@@ -157,10 +181,7 @@ __device__ __forceinline__ u32x4 narrow8(const float (&r)[8]) {
             worst = mag > worst ? mag : worst;
         }
         if (__builtin_amdgcn_ballot_w64(worst >= 0x47800000u) != 0) {
-            out.x = T::narrow2_any(r[0], r[1]);
-            out.y = T::narrow2_any(r[2], r[3]);
-            out.z = T::narrow2_any(r[4], r[5]);
-            out.w = T::narrow2_any(r[6], r[7]);
+            out = narrow8_any<T>(r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]);
         }
     }
     return out;

@@ -90,19 +90,48 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
     auto finish_row = [&](const Row &row, const u32x4(&cur)[NV], int phase) {
         const uint32_t keep = row.keep;
         const uint32_t keep_vecs = (keep + 7) / 8;
+        // Maximum and minimum of the kept part.  fp16 rows are compared two
+        // elements at a time in their own format (v_pk_max_f16 / v_pk_min_f16
+        // ignore a NaN operand like fmaxf / fminf do); the boundary vector,
+        // whose tail is masked, and bf16 rows go element by element in fp32.
         float f[NV][8];
-        float mx = neg_inf;
+        float mx = neg_inf, mn = __builtin_inff();
+        if constexpr (T::kPackedMinMax) {
+            typename T::pair mx2 = T::splat(neg_inf), mn2 = T::splat(__builtin_inff());
 #pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
-            if (v >= keep_vecs) continue;// wholly masked: nothing to reduce, zeros are stored below
-            widen8<T>(cur[k], f[k]);
-            if (v * 8 + 8 > keep) {// the boundary vector
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                if (v >= keep_vecs) continue;// wholly masked: nothing to reduce, zeros are stored below
+                if (v * 8 + 8 > keep) {
+                    float b[8];
+                    widen8<T>(cur[k], b);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) f[k][e] = v * 8 + e < keep ? f[k][e] : neg_inf;
+                    for (int e = 0; e < 8; ++e) {
+                        if (v * 8 + e < keep) mx = fmaxf(mx, b[e]), mn = fminf(mn, b[e]);
+                    }
+                } else {
+                    const uint32_t w[4] = {cur[k].x, cur[k].y, cur[k].z, cur[k].w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        mx2 = T::max2(mx2, T::as_pair(w[i]));
+                        mn2 = T::min2(mn2, T::as_pair(w[i]));
+                    }
+                }
             }
+            mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
+            mn = fminf(mn, fminf(T::first(mn2), T::second(mn2)));
+        } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[k][e]);
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * BS + threadIdx.x;
+                if (v >= keep_vecs) continue;
+                float b[8];
+                widen8<T>(cur[k], b);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (v * 8 + e < keep) mx = fmaxf(mx, b[e]), mn = fminf(mn, b[e]);
+                }
+            }
         }
         mx = block_max<WAVES>(mx, red, phase);
 
@@ -110,20 +139,20 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
         // here and is zeroed after the exponential.  Anything below the lean
         // exponential's range (-inf inputs, very long tails) sends the wavefront
         // through the library routine; NaN passes through either form as NaN.
-        float lowest = 0.0f;
+        // The smallest d of this lane is its minimum less the row's maximum.
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = k * BS + threadIdx.x;
             if (v >= keep_vecs) continue;
+            widen8<T>(cur[k], f[k]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) f[k][e] -= mx;
             if (v * 8 + 8 > keep) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) f[k][e] = v * 8 + e < keep ? f[k][e] : 0.0f;
             }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) lowest = fminf(lowest, f[k][e]);
         }
+        const float lowest = mn - mx;// +inf - max for a lane without kept elements: passes the test below
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
         float part = 0.0f;
 #pragma unroll

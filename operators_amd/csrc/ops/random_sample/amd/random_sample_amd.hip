@@ -403,6 +403,232 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
     rank_and_draw<T>(sh, result, topk, topk, top, total, random_val, topp, temperature);
 }
 
+// ---- more candidates than LDS ranks: sampling without a sorted list -----------
+// The reference keeps any topk up to the vocabulary size (random_sample.cc:
+// 67-74 only clamps it).  Beyond KMAX candidates nothing is compacted or
+// ranked.  Equal logits have equal probabilities, so the sorted sequence the
+// reference walks is fully described by how often every 16-bit code occurs: a
+// histogram over the ordered keys, walked from the largest key down, adding
+// each key's probability as many times as the key occurs - the same sequential
+// fp32 additions, the same comparisons.  One workgroup:
+//   1. the largest key and the softmax denominator (two passes over the logits);
+//   2. walk 1 finds where the running sum reaches topp (or the topk-th entry)
+//      and with it the sum of the kept prefix; walk 2 finds the entry whose
+//      running sum exceeds random_val times that sum.  A walk takes the key
+//      space in ranges of kWideBins keys from the top: count the logits of the
+//      range into an LDS histogram, compute every occupied key's probability
+//      in parallel, then the first wavefront adds them up in order.  Walks
+//      stop as soon as their question is answered - for ordinary top-p values
+//      within the first range;
+//   3. the answer is "occurrence r of key K": every lane counts K in its
+//      contiguous share of the logits, a prefix sum finds the share holding
+//      occurrence r, and that lane looks it up.  Equal logits are thereby
+//      ordered by ascending index, as in the other forms.
+// The chain of additions is as long as the reference's (at most topk, for a
+// topp no running sum reaches); entries whose probability rounds to zero are
+// skipped in one step.  Milliseconds in that worst case, against the
+// reference's topk * vocabulary comparisons.
+constexpr int kWideBins = 4096;
+
+struct WideShared {
+    uint32_t hist[kWideBins];
+    float p_of[kWideBins];
+    uint32_t wave_key[WAVES];
+    float sum_slots[WAVES];
+    uint32_t wave_tot[WAVES];
+    // state of a walk, written by the first wavefront
+    uint32_t done, found, entry, key, occurrence;
+    float run;
+    uint32_t n;
+};
+
+// One walk over the sorted sequence.  MODE 0: stop at the first entry whose
+// running sum reaches `threshold` (found = 1, entry = its rank), or after
+// `limit_n` entries.  MODE 1: stop at the first entry whose running sum
+// exceeds `threshold` (found = 1, key/occurrence name it), or after `limit_n`.
+// Leaves the running sum in sh.run.  All lanes call it.
+template<typename T, bool VEC, int MODE>
+__device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs, uint32_t voc, uint32_t key_max, float top,
+                                          float total, float temperature, float threshold, uint32_t limit_n) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    if (tid == 0) {
+        sh.done = limit_n == 0 ? 1u : 0u;
+        sh.found = 0;
+        sh.run = 0.0f;
+        sh.n = 0;
+    }
+    __syncthreads();
+    for (int64_t hi = key_max; hi >= 0; hi -= kWideBins) {
+        if (sh.done != 0) break;// uniform: written before the last barrier
+        for (int b = tid; b < kWideBins; b += BS) sh.hist[b] = 0;
+        __syncthreads();
+        for (uint32_t base = tid * 8u; base < voc; base += BS * 8u) {
+            uint32_t h[8];
+            const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (e < n) {
+                    const uint32_t below = static_cast<uint32_t>(hi) - key_of<T>(h[e]);// wraps for keys above the range
+                    if (below < static_cast<uint32_t>(kWideBins)) atomicAdd(&sh.hist[below], 1u);
+                }
+            }
+        }
+        __syncthreads();
+        for (int b = tid; b < kWideBins; b += BS) {
+            float p = 0.0f;
+            if (sh.hist[b] != 0 && static_cast<int64_t>(b) <= hi) {
+                const float x = value_of_key<T>(static_cast<uint32_t>(hi - b));
+                p = T::one(T::narrow1(expf((x - top) / temperature) / total));
+            }
+            sh.p_of[b] = p;
+        }
+        __syncthreads();
+        if (tid < kWave) {
+            float run = sh.run;
+            uint32_t n = sh.n;
+            bool done = false;
+            for (int b0 = 0; b0 < kWideBins && !done; b0 += kWave) {
+                const uint32_t c = sh.hist[b0 + lane];
+                const float p = sh.p_of[b0 + lane];
+                unsigned long long occupied = __builtin_amdgcn_ballot_w64(c != 0);
+                while (occupied != 0 && !done) {
+                    const int j = __builtin_ctzll(occupied);
+                    occupied &= occupied - 1;
+                    const uint32_t cj = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(c), j));
+                    const float pj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, p), j));
+                    const uint32_t take = cj < limit_n - n ? cj : limit_n - n;
+                    if (__builtin_bit_cast(uint32_t, pj) == 0u) {
+                        // adding +0 leaves the sum as it is: the comparison gives for every one of these entries
+                        // what it gives for the first
+                        if (take != 0 && (MODE == 0 ? run >= threshold : threshold < run)) {
+                            if (lane == 0) {
+                                sh.found = 1;
+                                sh.entry = n;
+                                sh.key = static_cast<uint32_t>(hi - (b0 + j));
+                                sh.occurrence = 0;
+                            }
+                            ++n;
+                            done = true;
+                        } else {
+                            n += take;
+                        }
+                    } else {
+                        for (uint32_t i = 0; i < take; ++i) {
+                            run += pj;
+                            ++n;
+                            if (MODE == 0 ? run >= threshold : threshold < run) {
+                                if (lane == 0) {
+                                    sh.found = 1;
+                                    sh.entry = n - 1;
+                                    sh.key = static_cast<uint32_t>(hi - (b0 + j));
+                                    sh.occurrence = i;
+                                }
+                                done = true;
+                                break;
+                            }
+                        }
+                    }
+                    if (n >= limit_n) done = true;
+                }
+            }
+            if (lane == 0) {
+                sh.run = run;
+                sh.n = n;
+                sh.done = done ? 1u : 0u;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template<typename T, bool VEC>
+__global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const uint16_t *probs, uint32_t voc,
+                                                          float random_val, float topp, uint32_t topk, float temperature) {
+    __shared__ WideShared sh;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t step = BS * 8u;
+
+    // the largest key, then the denominator in the accumulation order of the other one-workgroup form
+    uint32_t key_max = 0;
+    for (uint32_t base = tid * 8u; base < voc; base += step) {
+        uint32_t h[8];
+        const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < n) {
+                const uint32_t k = key_of<T>(h[e]);
+                key_max = k > key_max ? k : key_max;
+            }
+        }
+    }
+    key_max = wave_max_u32(key_max);
+    if (lane == 0) sh.wave_key[wave] = key_max;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) key_max = sh.wave_key[w] > key_max ? sh.wave_key[w] : key_max;
+    const float top = value_of_key<T>(key_max);
+    float part = 0.0f;
+    for (uint32_t base = tid * 8u; base < voc; base += step) {
+        uint32_t h[8];
+        const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (e < n) part += expf((T::one(static_cast<uint16_t>(h[e])) - top) / temperature);
+        }
+    }
+    part = wave_sum(part);
+    if (lane == 0) sh.sum_slots[wave] = part;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) total += sh.sum_slots[w];
+
+    // walk 1 (random_sample.cc:97-109): where the running sum reaches topp
+    wide_walk<T, VEC, 0>(sh, probs, voc, key_max, top, total, temperature, topp, topk);
+    const uint32_t stop = sh.found != 0 ? sh.entry : topk;// rank of the entry that reached topp
+    const float kept = sh.run;                             // the sum up to and including it, or over all topk entries
+    const uint32_t end = stop + 1 < topk ? stop + 1 : topk;
+    __syncthreads();
+    // walk 2 (random_sample.cc:112-125): the first of those `end` entries whose running sum exceeds random_val * kept
+    wide_walk<T, VEC, 1>(sh, probs, voc, key_max, top, total, temperature, random_val * kept, end);
+    if (sh.found == 0) return;// nothing exceeds it (random_val >= 1): the result stays as it is, as in the reference
+    const uint32_t key = sh.key, occurrence = sh.occurrence;
+
+    // occurrence `occurrence` of `key` in index order
+    const uint32_t share = ((voc + BS - 1) / BS + 7u) & ~7u;// logits per lane, a multiple of 8
+    const uint32_t first = static_cast<uint32_t>(tid) * share;
+    const uint32_t last = first + share < voc ? first + share : voc;
+    uint32_t mine = 0;
+    for (uint32_t base = first; base < last; base += 8) {
+        uint32_t h[8];
+        const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mine += (e < n && base + e < last && key_of<T>(h[e]) == key) ? 1u : 0u;
+    }
+    const uint32_t upto = wave_scan_u32(mine);
+    if (lane == kWave - 1) sh.wave_tot[wave] = upto;
+    __syncthreads();
+    uint32_t before = upto - mine;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) before += w < wave ? sh.wave_tot[w] : 0u;
+    if (occurrence >= before && occurrence < before + mine) {
+        uint32_t seen = before;
+        for (uint32_t base = first; base < last; base += 8) {
+            uint32_t h[8];
+            const int n = load_codes<VEC>(probs, voc, base, h);
+            for (int e = 0; e < 8; ++e) {
+                if (e < n && base + e < last && key_of<T>(h[e]) == key) {
+                    if (seen == occurrence) {
+                        result[0] = base + e;
+                        return;
+                    }
+                    ++seen;
+                }
+            }
+        }
+    }
+}
+
 template<typename T, bool VEC>
 __global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const uint16_t *probs, uint32_t voc,
                                                           float random_val, float topp, uint32_t topk, float temperature) {
@@ -694,6 +920,8 @@ void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
         auto *lists = reinterpret_cast<unsigned long long *>(c.heads + kRandomSampleMaxGroups);
         random_sample_partial<T, VEC><<<c.groups, kRandomSamplePartLanes, 0, s>>>(c.heads, lists, c.probs, c.voc, c.vecs, c.topk, c.temperature);
         random_sample_merge<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature, c.heads, lists, c.groups);
+    } else if (form == 2 && c.topk > static_cast<uint32_t>(KMAX)) {
+        random_sample_wide<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature);
     } else if (form == 2) {
         random_sample_topk<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature);
     }
@@ -741,6 +969,9 @@ infiniopStatus_t scratch_address(int device_id, void **address) {
 // share the array: two of them in flight at once, on any streams, race.
 infiniopStatus_t amdRandomSampleNoAlloc(RandomSampleAmdDescriptor_t desc, void *result, void const *probs, float random_val,
                                         float topp, int topk, float temperature, void *stream) {
+    if (result == nullptr || probs == nullptr) {
+        return STATUS_BAD_PARAM;
+    }
     if (desc->voc > kRandomSampleNoAllocMaxVoc) {
         std::fprintf(stderr, "infiniop[amd-gpu]: RandomSampleNoAlloc serves at most %u logits, the descriptor has %u; "
                              "use infiniopRandomSample with a workspace\n", kRandomSampleNoAllocMaxVoc, desc->voc);
@@ -774,9 +1005,6 @@ infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspa
     uint32_t k = 0;
     if (sample) {
         k = static_cast<uint32_t>(topk) > desc->voc ? desc->voc : static_cast<uint32_t>(topk);
-        if (k > static_cast<uint32_t>(kRandomSampleMaxTopk)) {
-            return STATUS_BAD_PARAM;
-        }
     }
     AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -67,13 +67,49 @@ __device__ __forceinline__ float load_w1(const void *w, int kind, uint64_t j) {
     return W16<BF16Rne>::one(w, j);
 }
 
+// ---- the sum of squares of a row, in one order whatever the launch shape ------
+// Every vector of 8 elements gives one partial (pairwise inside the vector);
+// 64 consecutive vectors are added by the wavefront's cross-lane tree
+// (amd::wave_sum); those chunk sums are added in ascending order.  A row's
+// sum therefore does not depend on how many lanes serve it or how many vectors
+// a lane holds, and RMSNorm gives the same bits through every kernel below -
+// which is what lets the fused Add + RMSNorm reproduce the two separate calls
+// bit for bit while choosing its own launch shape.  Lane l of wavefront w
+// holds vector k * 64 * WAVES + 64 * w + l in s[k]; absent vectors give 0.
+// `slots` is LDS with room for NV * WAVES floats that nobody else uses until
+// the next barrier.
+template<int WAVES, int NV>
+__device__ __forceinline__ float row_sum(const float (&s)[NV], float *slots) {
+    float c[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) c[k] = wave_sum(s[k]);
+    float total = 0.0f;
+    if constexpr (WAVES == 1) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) total += c[k];
+    } else {
+        const int wave = threadIdx.x / kWave;
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) slots[k * WAVES + wave] = c[k];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < NV * WAVES; ++j) total += slots[j];
+    }
+    return total;
+}
+
+// One vector's sum of squares: pairwise.
+__device__ __forceinline__ float squares8(const float (&f)[8]) {
+    const float s01 = f[0] * f[0] + f[1] * f[1], s23 = f[2] * f[2] + f[3] * f[3];
+    const float s45 = f[4] * f[4] + f[5] * f[5], s67 = f[6] * f[6] + f[7] * f[7];
+    return (s01 + s23) + (s45 + s67);
+}
+
 __device__ __forceinline__ float inv_rms(float sum_sq, uint64_t d, float eps) {
     const float mean_eps = sum_sq / static_cast<float>(d) + eps;
-#ifdef RMS_DIAG_F32
-    return __builtin_amdgcn_rsqf(mean_eps);
-#else
     return static_cast<float>(1.0 / sqrt(static_cast<double>(mean_eps)));
-#endif
 }
 
 // ---- rows that fit in registers -----------------------------------------------
@@ -126,7 +162,7 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                      uint64_t first_mul, uint64_t hop, uint64_t span, Residual<ADD> res) {
     constexpr int WAVES = BS / kWave;
-    __shared__ float red[2 * WAVES];
+    __shared__ float red[2 * NV * WAVES];// two sets of chunk sums, used in turn: one barrier per row is enough
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
     f32x4 *w_lo = reinterpret_cast<f32x4 *>(dyn_lds);
     const uint32_t nvec = d / 8;
@@ -206,23 +242,14 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
                 if (EXACT || v < nvec) cr.st16(v * 16, cur[k]);
             }
         }
-        float part = 0.0f;
+        float part[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             float f[8];
             widen8<T>(cur[k], f);
-            if constexpr (!EXACT) {
-                if (k * BS + threadIdx.x >= nvec) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) f[i] = 0.0f;
-                }
-            }
-            // pairwise inside the vector, then onto the running partial
-            const float s01 = f[0] * f[0] + f[1] * f[1], s23 = f[2] * f[2] + f[3] * f[3];
-            const float s45 = f[4] * f[4] + f[5] * f[5], s67 = f[6] * f[6] + f[7] * f[7];
-            part += (s01 + s23) + (s45 + s67);
+            part[k] = EXACT || k * BS + threadIdx.x < nvec ? squares8(f) : 0.0f;
         }
-        const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
+        const float k_row = inv_rms(row_sum<WAVES, NV>(part, red + phase * NV * WAVES), d, eps);
 
         const StreamOut<THROUGH> yr(y + static_cast<int64_t>(r) * stride_y);// a row is far shorter than 4 GiB
 #pragma unroll
@@ -231,12 +258,6 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
             if (EXACT || v < nvec) {
                 float f[8], g[8];
                 widen8<T>(cur[k], f);
-#ifdef RMS_DIAG_NOW
-                if constexpr (true) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) g[i] = 1.0f;
-                } else
-#endif
                 if constexpr (WHOME == kWLds) {
                     const f32x4 a = w_lo[v], b = w_hi[v];
                     g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
@@ -295,7 +316,7 @@ __global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t 
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                      Residual<ADD> res) {
     constexpr int WAVES = BS / kWave;
-    __shared__ float red[R * WAVES];
+    __shared__ float red[R * NV * WAVES];
     const uint32_t nvec = d / 8;
     const uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * R;
     const int rows_here = n - row0 < static_cast<uint64_t>(R) ? static_cast<int>(n - row0) : R;
@@ -348,7 +369,7 @@ __global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t 
         }
     }
 
-    float part[R];
+    float part[R][NV];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if constexpr (ADD) {// the row becomes a + b, rounded as Add rounds, and goes out to c
@@ -365,41 +386,39 @@ __global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t 
                 if (r < rows_here && (EXACT || v < nvec)) cr.st16(v * 16, xv[r][k]);
             }
         }
-        part[r] = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             float f[8];
             widen8<T>(xv[r][k], f);
-            if constexpr (!EXACT) {
-                if (k * BS + threadIdx.x >= nvec) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) f[i] = 0.0f;
-                }
-            }
-            const float s01 = f[0] * f[0] + f[1] * f[1], s23 = f[2] * f[2] + f[3] * f[3];
-            const float s45 = f[4] * f[4] + f[5] * f[5], s67 = f[6] * f[6] + f[7] * f[7];
-            part[r] += (s01 + s23) + (s45 + s67);
+            part[r][k] = EXACT || k * BS + threadIdx.x < nvec ? squares8(f) : 0.0f;
         }
-        part[r] = wave_sum(part[r]);
     }
-    if constexpr (WAVES > 1) {
-        const int wave = threadIdx.x / kWave;
-        if ((threadIdx.x & (kWave - 1)) == 0) {
+    // the R rows' chunk sums go through LDS side by side and share one barrier
+    float total[R];
+    if constexpr (WAVES == 1) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) red[r * WAVES + wave] = part[r];
+        for (int r = 0; r < R; ++r) total[r] = row_sum<1, NV>(part[r], red);
+    } else {
+        const int wave = threadIdx.x / kWave;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const float c = wave_sum(part[r][k]);
+                if ((threadIdx.x & (kWave - 1)) == 0) red[(r * NV + k) * WAVES + wave] = c;
+            }
         }
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            float total = 0.0f;
+            total[r] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < WAVES; ++i) total += red[r * WAVES + i];
-            part[r] = total;
+            for (int j = 0; j < NV * WAVES; ++j) total[r] += red[r * NV * WAVES + j];
         }
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const float k_row = inv_rms(part[r], d, eps);
+        const float k_row = inv_rms(total[r], d, eps);
         const StreamOut<THROUGH> yr(y + static_cast<int64_t>(row0 + r) * stride_y);
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -489,41 +508,54 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
             py, px, w, w_kind, n, d, desc.stride_y, desc.stride_x, desc.epsilon, res);
         return;
     }
+    // Large outputs are written through L2 (see StreamOut).
+    const bool through = n * d * sizeof(uint16_t) >= kWriteThroughBytes;
 
-    const bool through_once = n * d * sizeof(uint16_t) >= kWriteThroughBytes;
-    if (const long r1 = amd::tune("RMS_ONCE", 0); r1 != 0 && nvec <= 4096) {// experiment: one pass in dispatch order, r1 rows per workgroup
-        const uint64_t grid1 = ceil_div(n, static_cast<uint64_t>(r1));
-        const bool thr = amd::tune("RMS_THROUGH", through_once ? 1 : 0) != 0;
+    // Which form.  Measured on MI355X, 128 MiB of bf16 rows with fp32 weights
+    // (and [8192, 8192] for the fused form), one pass (R rows per workgroup,
+    // weights in registers) against looping workgroups (weights in LDS):
+    //   d =  512:  41.2 us one pass, R = 1          46.9 us looping
+    //   d = 1024:  46.7 us one pass, R = 2 (59.0 with R = 1)   51.2 us looping
+    //   d = 2048:  44.4 us one pass, R = 2 (47.0 with R = 1)   47.9 us looping
+    //   d = 4096:  45.5 us one pass, R = 1 (46.4 with R = 2)   46.6 us looping
+    //   d = 8192:  45.6-50.3 us one pass            44.6 us looping
+    //   d = 8192, fused Add: 86.5 us one pass with 1024 lanes, 88.1-89.7 with 256 or 512   89.0 us looping
+    //   d >= 16384: looping (a row's weights are 64 KiB and more: too many registers)
+    // One pass re-reads the weight row through L2 once per R rows - at d = 8192
+    // that is twice the bytes of the row itself - which is what it loses to
+    // the looping form there; the fused form moves twice the data per weight.
 #define RMS_ONCE_GO(BS, NV, R, E, TH)                                                                              \
-    rms_norm_once<T, BS, NV, R, E, TH, ADD><<<static_cast<unsigned>(grid1), BS, 0, stream>>>(                      \
+    rms_norm_once<T, BS, NV, R, E, TH, ADD><<<static_cast<unsigned>(ceil_div(n, R)), BS, 0, stream>>>(              \
         py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res)
-#define RMS_ONCE_R(BS, NV, R)                                                                                      \
+#define RMS_ONCE(BS, NV, R)                                                                                        \
     do {                                                                                                           \
         const bool exact = nvec == static_cast<uint64_t>(BS) * NV;                                                 \
-        if (exact && thr) RMS_ONCE_GO(BS, NV, R, true, true);                                                      \
+        if (exact && through) RMS_ONCE_GO(BS, NV, R, true, true);                                                  \
         else if (exact) RMS_ONCE_GO(BS, NV, R, true, false);                                                       \
-        else if (thr) RMS_ONCE_GO(BS, NV, R, false, true);                                                         \
+        else if (through) RMS_ONCE_GO(BS, NV, R, false, true);                                                     \
         else RMS_ONCE_GO(BS, NV, R, false, false);                                                                 \
     } while (0)
-#define RMS_ONCE(BS, NV)                                                                                           \
-    do {                                                                                                           \
-        if (r1 == 1) RMS_ONCE_R(BS, NV, 1);                                                                        \
-        else RMS_ONCE_R(BS, NV, 2);                                                                                \
-    } while (0)
-        const long bs1 = amd::tune("RMS_BS", 0);
-        if (nvec <= 64) RMS_ONCE(64, 1);
-        else if (nvec <= 256) RMS_ONCE(256, 1);
-        else if (nvec <= 512) RMS_ONCE(256, 2);
-        else if (nvec <= 1024 && bs1 == 512) RMS_ONCE(512, 2);
-        else if (nvec <= 1024 && bs1 == 1024) RMS_ONCE(1024, 1);
-        else if (nvec <= 1024) RMS_ONCE(256, 4);
-        else if (nvec <= 2048) RMS_ONCE(512, 4);
-        else RMS_ONCE(1024, 4);
-#undef RMS_ONCE
-#undef RMS_ONCE_R
-#undef RMS_ONCE_GO
+    if (nvec <= 64) {
+        RMS_ONCE(64, 1, 1);
         return;
     }
+    if (nvec <= 256) {
+        RMS_ONCE(256, 1, 2);
+        return;
+    }
+    if (nvec <= 512) {
+        RMS_ONCE(256, 2, 1);
+        return;
+    }
+    if constexpr (ADD) {
+        if (nvec == 1024) {
+            if (through) RMS_ONCE_GO(1024, 1, 1, true, true);
+            else RMS_ONCE_GO(1024, 1, 1, true, false);
+            return;
+        }
+    }
+#undef RMS_ONCE
+#undef RMS_ONCE_GO
 
     // A workgroup that serves several rows fetches the weights once: into LDS
     // as fp32 when the row leaves room for at least two workgroups per compute
@@ -536,8 +568,7 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // slack while staging the weights only 512 times.  Shorter rows put fewer
     // bytes in flight per workgroup, so they get proportionally more of them.
     uint64_t per_cu = ceil_div(32 * 1024, d * sizeof(uint16_t));
-    per_cu = per_cu < 2 ? 2 : (per_cu > 16 ? 16 : per_cu);
-    per_cu = static_cast<uint64_t>(amd::tune("RMS_PER_CU", static_cast<long>(per_cu)));
+    per_cu = per_cu < 2 ? 2 : per_cu;
     int home = kWLds;
     if (lds_bytes <= lds_limit && lds_bytes <= 64 * 1024) {
         const uint64_t fit = (160 * 1024) / (lds_bytes + 256);// 160 KiB of LDS per compute unit
@@ -546,23 +577,18 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         home = kWGlobal;
     }
     uint64_t grid = static_cast<uint64_t>(desc.cu_count) * per_cu;
-    if (n <= grid || amd::tune("RMS_ONESHOT", 0)) {
+    if (n <= grid) {
         grid = n;
         home = kWGlobal;// one row per workgroup: staging would only add a pass
     }
-    // rows of a workgroup: blockIdx.x, + grid, + 2*grid, ...
-    uint64_t first_mul = 1, hop = grid, span = n;
-    if (const long r = amd::tune("RMS_BLOCKED", 0); r > 0 && home == kWLds) {// experiment: r consecutive rows per workgroup
-        grid = ceil_div(n, static_cast<uint64_t>(r));
-        first_mul = span = static_cast<uint64_t>(r);
-        hop = 1;
-    }
+    // rows of a workgroup: blockIdx.x, + grid, + 2 * grid, ...  (Consecutive
+    // rows per workgroup measure 2-13 % slower at [8192, 8192].)
+    const uint64_t first_mul = 1, hop = grid, span = n;
 
-    // Large outputs are written through L2; the kernels that re-read the
-    // weights from memory per row exist in one form only (inexact row length,
-    // plain non-temporal stores): they serve one-row workgroups and rows too
-    // long for LDS, where neither refinement is measurable.
-    const bool through = n * d * sizeof(uint16_t) >= kWriteThroughBytes;
+    // The kernels that re-read the weights from memory per row exist in one
+    // form only (inexact row length, plain non-temporal stores): they serve
+    // one-row workgroups and rows too long for LDS, where neither refinement
+    // is measurable.
 #define RMS_GO(BS, NV, HOME, LDS, EXACT, THROUGH)                                                                      \
     rms_norm_rows<T, BS, NV, HOME, EXACT, THROUGH, ADD><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(             \
         py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res)
@@ -576,10 +602,7 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         else RMS_GO(BS, NV, kWLds, lds_bytes, false, false);                                                           \
     } while (0)
 
-    if (nvec <= 64) RMS_LAUNCH(64, 1);
-    else if (nvec <= 256) RMS_LAUNCH(256, 1);
-    else if (nvec <= 512) RMS_LAUNCH(256, 2);
-    else if (nvec <= 1024) RMS_LAUNCH(256, 4);// d = 8192: 512x2 measures the same, 1024x1 is 8 % slower
+    if (nvec <= 1024) RMS_LAUNCH(256, 4);// d = 8192: 512x2 measures the same, 1024x1 is 8 % slower
     else if (nvec <= 2048) RMS_LAUNCH(512, 4);
     else if (nvec <= 4096) RMS_LAUNCH(1024, 4);
     else RMS_LAUNCH(1024, 8);

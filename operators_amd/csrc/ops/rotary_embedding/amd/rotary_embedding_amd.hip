@@ -109,13 +109,15 @@ __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *
 }
 
 // One pass, one tile of BS work items per workgroup, in the order the
-// dispatcher hands workgroups out.  The position is requested first, then the
-// data, then - as soon as the position is there, while the data is still on
-// its way (loads return in issue order) - the table rows.  UNI: a token's work
-// items are a multiple of BS, so a workgroup lies inside one token and its
-// position and table base are found with scalar arithmetic and scalar loads.
-// The head count is a multiple of HPT (every lane's heads exist): nothing is
-// predicated, so no load can sink into a branch behind the wait for another.
+// dispatcher hands workgroups out.  UNI: a token's work items are a multiple
+// of BS, so a workgroup lies inside one token and its position and table base
+// are found with scalar arithmetic and scalar loads, which run beside the
+// vector loads of the data.  Otherwise every lane loads its token's position
+// itself, after the data loads: asked for first, the position delays the data
+// behind it (k [8192, 8, 128] bf16 with 4 heads per lane: 10.6 us position
+// first, 8.7 us position last).  The head count is a multiple of HPT (every
+// lane's heads exist): nothing is predicated, so no load can sink into a
+// branch behind the wait for another.
 template<typename T, int BS, int HPT, bool BUFST, bool UNI>
 __global__ __launch_bounds__(BS) void rope_once(uint16_t *__restrict__ t, const uint64_t *__restrict__ pos,
                                                 const float *__restrict__ sin_t, const float *__restrict__ cos_t,
@@ -134,7 +136,8 @@ __global__ __launch_bounds__(BS) void rope_once(uint16_t *__restrict__ t, const 
     }
     const uint32_t g = rem / vecs_per_head;
     const uint32_t cv = rem - g * vecs_per_head;
-    const uint64_t p = pos[token];
+    uint64_t p;
+    if constexpr (UNI) p = pos[token];
 
     uint16_t *base = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(cv) * 8;
     u32x4 tv[HPT];
@@ -143,6 +146,7 @@ __global__ __launch_bounds__(BS) void rope_once(uint16_t *__restrict__ t, const 
         const uint32_t h = g + i * groups;
         tv[i] = ld16_stream(base + static_cast<int64_t>(h) * stride_head);
     }
+    if constexpr (!UNI) p = pos[token];
     __builtin_amdgcn_sched_barrier(0);// the data loads leave before anything waits for the position
 
     const uint64_t row = p * head_dim + static_cast<uint64_t>(cv) * 8;
@@ -207,38 +211,43 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
                        static_cast<uint64_t>(d.stride_token) < (1ull << 23) &&
                        d.heads * static_cast<uint64_t>(d.stride_head) < (1ull << 30) && d.head_dim < (1ull << 24);
 
-    // Heads per lane.  Two things pull against each other: every lane fetches
-    // the 64 bytes of table values of its column group whatever the number of
-    // heads it rotates with them, so few heads per lane multiply the table
-    // traffic through L2; many heads per lane leave few lanes.  A token whose
-    // lanes fill a workgroup exactly (UNI) is best when the head count allows
-    // it; a handful of heads goes to one lane per column group.  Measured on
-    // MI355X, one pass (rope_once), 256 lanes:
-    //   q [8192,64,128] bf16 in [8192,80,128]:  2/4/8 heads per lane 43.4 / 43.4 / 46.6 us
-    //                                           (45.5 us for workgroups looping over tokens with prefetch)
-    //   k [8192,8,128] bf16:                    2/4/8 heads per lane 10.5 / 10.6 / 8.65 us (9.05 the position loaded last)
-    //   [4096,32,128] fp16 in [4096,96,128]:    2/4/8 heads per lane 14.1 / 14.4 / 14.3 us
-    // Workgroups of 64 or 128 lanes measure the same or worse (k: 8.6, q: 44.7-48.7 us).
+    // Heads per lane.  Every lane fetches the 64 bytes of table values of its
+    // column group whatever the number of heads it rotates with them, so few
+    // heads per lane multiply the table traffic through L2, and many heads per
+    // lane leave few lanes.  Measured on MI355X (us; one pass, 256 lanes; "uni"
+    // = a token's lanes fill whole workgroups):
+    //   heads per lane                          2          4          8        16
+    //   q [8192,64,128] bf16, 128 MiB        43.6 uni   43.3 uni   46.2      46.4
+    //   k [8192,8,128] bf16, 16 MiB          10.9        8.7        8.7       -
+    //   [4096,32,128] fp16, 32 MiB, random   14.0 uni   14.2       13.2      12.9
+    //   positions
+    // (q with workgroups looping over tokens with prefetch: 45.5; workgroups of
+    // 64 or 128 lanes: the same or worse at every shape.)  So: tensors that
+    // keep the memory system busy for tens of microseconds take the layout in
+    // which a token fills a workgroup; smaller ones, whose time is mostly
+    // launch and latency, put as many heads on a lane as divide the count.
+    const bool large = d.tokens * d.heads * d.head_dim * sizeof(uint16_t) >= kWriteThroughBytes;
     int hpt = 1;
-    for (int cand : {8, 4, 2}) {// the largest that divides the head count and still leaves a workgroup's worth of lanes per token
-        if (d.heads % cand == 0 && (d.heads / cand) * vph >= kBlock) {
-            hpt = cand;
-            break;
-        }
-    }
-    if (hpt == 1) {// fewer lanes than a workgroup per token whatever is chosen: as many heads per lane as divide the count
-        for (int cand : {8, 4, 2}) {
-            if (d.heads % cand == 0) {
+    if (large) {
+        for (int cand : {8, 4, 2}) {// the most heads per lane that still leave a workgroup's worth of lanes per token
+            if (d.heads % cand == 0 && (d.heads / cand) * vph >= kBlock) {
                 hpt = cand;
                 break;
             }
         }
     }
-    if (const long forced = amd::tune("ROPE_HPT", 0); forced > 0 && d.heads % forced == 0) hpt = static_cast<int>(forced);
+    if (hpt == 1) {
+        for (int cand : {16, 8, 4, 2}) {
+            if (d.heads % cand == 0 && (large ? cand <= 8 : true)) {
+                hpt = cand;
+                break;
+            }
+        }
+    }
     const uint64_t groups = d.heads / hpt;
     const uint64_t ipt = groups * vph;
     const uint64_t total = d.tokens * ipt;
-    if (sizeof(Idx) == 4 && total < (1ull << 31) && amd::tune("ROPE_ONCE", 1)) {
+    if (sizeof(Idx) == 4 && total < (1ull << 31)) {
         const bool uni = ipt % kBlock == 0;
         const unsigned grid = static_cast<unsigned>(ceil_div(total, kBlock));
         const bool b1 = bufst && static_cast<uint64_t>(kWave) * static_cast<uint64_t>(d.stride_token) * 2 +
@@ -255,7 +264,8 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
         else if (uni) ROPE_ONCE_GO(HPT, false, true);    \
         else ROPE_ONCE_GO(HPT, false, false);            \
     } while (0)
-        if (hpt == 8) ROPE_ONCE_BU(8);
+        if (hpt == 16) ROPE_ONCE_BU(16);
+        else if (hpt == 8) ROPE_ONCE_BU(8);
         else if (hpt == 4) ROPE_ONCE_BU(4);
         else if (hpt == 2) ROPE_ONCE_BU(2);
         else ROPE_ONCE_BU(1);

@@ -269,6 +269,9 @@ RANDOM_SAMPLE_CASES = [
     (640, 1.0, 0.9, 6, 1.0, "normal"),            # random_val = 1: nothing is written
     (640, 0.3, 0.0, 1, 1.0, "nan_inside"), (640, 0.3, 0.0, 1, 1.0, "nan_first"), (640, 0.3, 0.9, 1, 1.0, "neg_zero_first"),
     (900, 0.5, 0.9, 7, 1.0, "with_inf"),
+    # more candidates than any fixed-size list: the reference clamps topk to the vocabulary and nothing else
+    (5000, 0.42, 0.9, 1025, 1.0, "normal"), (32000, 0.77, 0.95, 4096, 0.8, "normal"), (8192, 0.63, 1.0, 8192, 2.0, "normal"),
+    (3000, 0.15, 0.99, 5000, 1.0, "uniform"), (16384, 0.9, 0.999, 16384, 1.0, "uniform"),
 ]
 
 

@@ -111,8 +111,6 @@ def test_against_oracle_with_ties(ctx):
         codes = x.view(np.uint16)
         args = (float(rng.random()), float(rng.choice([0.0, 0.5, 0.9, 1.0])), int(rng.choice([1, 2, 4, 10, 50, 300, 1024, 5000])),
                 float(rng.choice([0.5, 1.0, 2.0])))
-        if min(args[2], voc) > 1024 and args[1] > 0:
-            continue  # refused, see test_limits
         want = oracle.random_sample(codes, *args)
         got = gpu_sample(ctx, codes, *args)
         if not same_choice(codes, got, want):
@@ -160,10 +158,10 @@ def test_limits(ctx):
     result = torch.zeros(1, dtype=torch.int64, device="cuda").view(torch.uint64)
     with RandomSamplePlan(ctx, result, probs) as plan:
         assert 0 < plan.workspace_size < 200 * 1024
-        plan(result, probs, 0.5, 0.9, 1024, 1.0)          # the largest candidate count
+        plan(result, probs, 0.5, 0.9, 1024, 1.0)          # the largest candidate count ranked in LDS
+        plan(result, probs, 0.5, 0.9, 1025, 1.0)          # beyond it: the histogram walk, no limit on topk
+        plan(result, probs, 0.5, 0.9, 2 ** 31 - 1, 1.0)   # clamped to the vocabulary, as in the reference
         torch.cuda.synchronize()
-        with pytest.raises(InfiniopError):
-            plan(result, probs, 0.5, 0.9, 1025, 1.0)
         plan(result, probs, 0.5, 0.0, 100000, 1.0)        # greedy form: topk is not looked at
         torch.cuda.synchronize()
     # random_val = 1: the reference writes nothing, neither does the kernel
@@ -229,3 +227,56 @@ def test_large_vocabulary(ctx):
             want = oracle.random_sample(x, *args)
             got = gpu_sample(ctx, x, *args)
             assert same_choice(x, got, want), (voc, args, got, want)
+
+
+@pytest.mark.parametrize("voc,topk", [(1025, 1025), (5000, 1025), (5000, 5000), (8191, 3000), (20000, 100000), (34000, 2048)])
+def test_more_candidates_than_lds_ranks_distinct_logits(ctx, voc, topk):
+    """topk beyond 1024 (the reference has no limit, random_sample.cc:67-74): no
+    two logits equal, so the index itself must be the oracle's - for top-p
+    values that stop the walk early, late and never.
+
+    The draw compares a running sum of thousands of fp16 probabilities with a
+    limit; the GPU's expf and the order in which it adds up the softmax
+    denominator differ from the host's in the last bit, which can move one
+    probability by an fp16 unit and with it the crossing point by one rank.
+    For the nearly flat distributions (hundreds to thousands of entries kept)
+    a result one rank away from the oracle's is therefore accepted, at most
+    once per case; the peaked ones must agree exactly."""
+    rng = np.random.default_rng(500 + voc + topk)
+    pool = np.arange(0x0400, 0x4801, dtype=np.uint16)  # every normal fp16 code up to 8.0, so that the distribution is not one spike
+    pool = np.concatenate([pool, pool | 0x8000])
+    codes = rng.choice(pool, voc, replace=False)
+    order = np.argsort(-oracle.decode(codes, "f16"), kind="stable")
+    rank = np.empty(voc, np.int64)
+    rank[order] = np.arange(voc)
+    bad, near = [], []
+    for rv, topp, temp, flat in [(0.37, 0.9, 1.0, False), (0.999, 1.0, 2.0, True), (0.05, 0.5, 0.7, False), (0.93, 0.9999, 5.0, True),
+                                 (0.5, 1e-4, 1.0, False), (0.71, 1.0, 50.0, True)]:
+        want = oracle.random_sample(codes, rv, topp, topk, temp)
+        got = gpu_sample(ctx, codes, rv, topp, topk, temp)
+        if got == want:
+            continue
+        if flat and got is not None and want is not None and abs(int(rank[got]) - int(rank[want])) <= 1:
+            near.append((rv, topp, temp, got, want))
+        else:
+            bad.append((rv, topp, temp, got, want))
+    assert not bad, bad
+    assert len(near) <= 1, near
+
+
+def test_more_candidates_than_lds_ranks_with_ties(ctx):
+    """The reference test's own distribution (uniform [0, 1) in fp16: a few
+    thousand distinct values) with topk up to the whole vocabulary: an index
+    holding the same logit as the oracle's."""
+    rng = np.random.default_rng(91)
+    bad = []
+    for trial in range(24):
+        voc = int(rng.choice([2000, 4096, 16000]))
+        x = rng.random(voc, dtype=np.float32).astype(np.float16) if trial % 2 else (rng.standard_normal(voc, dtype=np.float32) * 3).astype(np.float16)
+        codes = x.view(np.uint16)
+        args = (float(rng.random()), float(rng.choice([0.3, 0.9, 1.0])), int(rng.choice([1025, 1500, 4096, voc, 10 ** 6])), float(rng.choice([0.5, 1.0, 3.0])))
+        want = oracle.random_sample(codes, *args)
+        got = gpu_sample(ctx, codes, *args)
+        if not same_choice(codes, got, want):
+            bad.append((trial, voc, args, got, want))
+    assert not bad, bad[:5]

@@ -259,9 +259,10 @@ def test_null_output_pointer_is_memory_not_allocated(fake_handle):
 
 
 def test_random_sample_host_rules_beyond_the_reference(fake_handle):
-    """A strided or empty logits vector is refused at create time; more than
-    1024 candidates (after clamping topk to the vocabulary) and null pointers
-    are refused at stage 4 before anything touches the device."""
+    """A strided or empty logits vector is refused at create time; null
+    pointers are refused at stage 4 before anything touches the device, and
+    the entry point without workspace refuses vocabularies beyond its limit
+    the same way.  topk has no upper limit (the reference has none)."""
     lib = oa.open_lib()
     handle, _keep = fake_handle
 
@@ -280,5 +281,9 @@ def test_random_sample_host_rules_beyond_the_reference(fake_handle):
     assert st == 0
     f = ctypes.c_float
     assert lib.infiniopRandomSample(d, None, 0, None, None, f(0.5), f(0.9), 4, f(1.0), None) == 2
-    assert lib.infiniopRandomSample(d, None, 0, 8, 8, f(0.5), f(0.9), 1025, f(1.0), None) == 2
+    assert lib.infiniopRandomSampleNoAlloc(d, None, None, f(0.5), f(0.9), 4, f(1.0), None) == 2
+    assert lib.infiniopDestroyRandomSampleDescriptor(d) == 0
+    st, d = create(("u64", (1,), None), ("f16", ((1 << 20) + 1,), None))
+    assert st == 0
+    assert lib.infiniopRandomSampleNoAlloc(d, 8, 8, f(0.5), f(0.9), 4, f(1.0), None) == 2  # more logits than its lists serve
     assert lib.infiniopDestroyRandomSampleDescriptor(d) == 0
