@@ -395,6 +395,7 @@ def ops_table(ctx, args, gen):
         "S3 random_sample f16 voc 151936, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 50, gen, "random_sample") for _ in range(MAX_SETS)],
         "S4 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8, no workspace (one workgroup)": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample", False) for _ in range(MAX_SETS)],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1b causal_softmax bf16 [32,4096,4096] (the Attention row's softmax on its own)": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, bf16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
         # Not an operator of the library: a plain device-to-device copy of known

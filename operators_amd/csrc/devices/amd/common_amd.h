@@ -68,17 +68,6 @@ inline uint64_t max_grid_1d(unsigned lanes) { return 0xFFFFFFFFull / lanes; }
 // more are 1-3 % faster written through.
 constexpr uint64_t kWriteThroughBytes = 64ull << 20;
 
-// Launch-shape experiments: a build with -DINFINIOP_AMD_TUNE reads integer
-// knobs from the environment; the normal build folds every knob to its default.
-#ifdef INFINIOP_AMD_TUNE
-inline long tune(const char *name, long dflt) {
-    const char *v = std::getenv(name);
-    return v != nullptr ? std::atol(v) : dflt;
-}
-#else
-constexpr long tune(const char *, long dflt) { return dflt; }
-#endif
-
 }// namespace amd
 
 #endif

@@ -15,6 +15,7 @@
 // without being read.
 #include "../../../devices/amd/kernel_amd.h"
 #include "causal_softmax_amd.h"
+#include <algorithm>
 
 namespace {
 
@@ -38,19 +39,25 @@ __device__ __forceinline__ float exp_nonpositive(float d) {
 constexpr float kLeanExpLimit = -126.0f;
 
 // The library exponential for the rare arguments outside that range (-inf,
-// very long tails, NaN).  Deliberately not inlined: it is almost never
-// executed, and four inlined copies per kernel cost instruction-cache space
-// that the common path needs.
-__device__ __attribute__((noinline)) float exp_any(float d) { return expf(d); }
+// very long tails, NaN), eight at a time through memory.  Deliberately not
+// inlined, and deliberately fed through a small array of its own: a call per
+// element inside the kernels would make every value that is live across it
+// compete for the few registers a callee preserves, and the common path would
+// pay for that with half its occupancy.
+__device__ __attribute__((noinline)) void exp_any8(float *v, float mx) {
+    for (int e = 0; e < 8; ++e) v[e] = expf(v[e] - mx);
+}
 
-// One workgroup of BS lanes per row at a time; lane l owns vectors l, l+BS, ...
-// (NV of them, 8 elements each), so total <= 8*BS*NV.  Workgroups stride over
-// the batch*seq rows (neighbouring rows keep nearly the same number of
-// columns, so the stride balances the causal triangle) and always have the
-// next row's loads in flight.  Loads are unconditional - a lane whose vector
-// lies in the masked part re-reads the row's last kept vector, which the
-// memory pipeline merges into one request - so that the compiler can count
-// the loads in flight and wait for the current row only.
+// One workgroup of BS lanes per row; lane l owns vectors l, l+BS, ... (NV of
+// them, 8 elements each), so total <= 8*BS*NV.  A workgroup takes one row at a
+// time and starts the next one only after it has stored the last: that keeps
+// the register count low enough for three to five wavefronts per SIMD, and it
+// is those other wavefronts that cover a row's load latency and arithmetic.
+// (A form that kept the next row's loads in flight needed twice the registers
+// and measured 3-30 % slower at every row length from 1024 to 32768 columns.)
+// Loads are unconditional: a lane whose vector lies in the masked part
+// re-reads the row's last kept vector, which the memory pipeline merges into
+// one request.
 template<typename T, int BS, int NV, bool THROUGH>
 __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
                                                           int64_t stride_b, int64_t stride_i) {
@@ -87,88 +94,86 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
             dst[k] = ld16_stream(row.ptr + static_cast<uint64_t>(v < last_vec ? v : last_vec) * 8);
         }
     };
+    // The one vector of a row that straddles the mask (when the kept length is
+    // not a multiple of 8) is dealt with apart from the others, inside
+    // wavefront-uniform branches that are taken once per row: its kept
+    // elements enter the maximum and minimum one by one, the exponentials of
+    // its masked elements (whatever they came to) are replaced by zero before
+    // the sum, and its masked outputs are forced to zero before the store (a
+    // row that turned to NaN would otherwise leak into them).  Everything else
+    // runs without a per-element test.
     auto finish_row = [&](const Row &row, const u32x4(&cur)[NV], int phase) {
         const uint32_t keep = row.keep;
         const uint32_t keep_vecs = (keep + 7) / 8;
-        // Maximum and minimum of the kept part.  fp16 rows are compared two
-        // elements at a time in their own format (v_pk_max_f16 / v_pk_min_f16
-        // ignore a NaN operand like fmaxf / fminf do); the boundary vector,
-        // whose tail is masked, and bf16 rows go element by element in fp32.
-        float f[NV][8];
+        const uint32_t tail = keep & 7u;// kept elements of the straddling vector, 0 when there is none
         float mx = neg_inf, mn = __builtin_inff();
-        if constexpr (T::kPackedMinMax) {
-            typename T::pair mx2 = T::splat(neg_inf), mn2 = T::splat(__builtin_inff());
+        [[maybe_unused]] typename T::pair mx2, mn2;
+        if constexpr (T::kPackedMinMax) mx2 = T::splat(neg_inf), mn2 = T::splat(__builtin_inff());
 #pragma unroll
-            for (int k = 0; k < NV; ++k) {
-                const uint32_t v = k * BS + threadIdx.x;
-                if (v >= keep_vecs) continue;// wholly masked: nothing to reduce, zeros are stored below
-                if (v * 8 + 8 > keep) {
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = k * BS + threadIdx.x;
+            const bool straddles = tail != 0 && v + 1 == keep_vecs;
+            if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                if (straddles) {
                     float b[8];
                     widen8<T>(cur[k], b);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
-                        if (v * 8 + e < keep) mx = fmaxf(mx, b[e]), mn = fminf(mn, b[e]);
-                    }
-                } else {
-                    const uint32_t w[4] = {cur[k].x, cur[k].y, cur[k].z, cur[k].w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        mx2 = T::max2(mx2, T::as_pair(w[i]));
-                        mn2 = T::min2(mn2, T::as_pair(w[i]));
+                        if (static_cast<uint32_t>(e) < tail) mx = fmaxf(mx, b[e]), mn = fminf(mn, b[e]);
                     }
                 }
             }
-            mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
-            mn = fminf(mn, fminf(T::first(mn2), T::second(mn2)));
-        } else {
+            if (v >= keep_vecs || straddles) continue;// wholly masked: nothing to reduce, zeros are stored below
+            if constexpr (T::kPackedMinMax) {
+                const uint32_t w[4] = {cur[k].x, cur[k].y, cur[k].z, cur[k].w};
 #pragma unroll
-            for (int k = 0; k < NV; ++k) {
-                const uint32_t v = k * BS + threadIdx.x;
-                if (v >= keep_vecs) continue;
+                for (int i = 0; i < 4; ++i) {
+                    mx2 = T::max2(mx2, T::as_pair(w[i]));
+                    mn2 = T::min2(mn2, T::as_pair(w[i]));
+                }
+            } else {
                 float b[8];
                 widen8<T>(cur[k], b);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    if (v * 8 + e < keep) mx = fmaxf(mx, b[e]), mn = fminf(mn, b[e]);
-                }
+                for (int e = 0; e < 8; ++e) mx = fmaxf(mx, b[e]), mn = fminf(mn, b[e]);
             }
+        }
+        if constexpr (T::kPackedMinMax) {
+            mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
+            mn = fminf(mn, fminf(T::first(mn2), T::second(mn2)));
         }
         mx = block_max<WAVES>(mx, red, phase);
 
-        // d = x - max <= 0.  The masked tail of the boundary vector takes d = 0
-        // here and is zeroed after the exponential.  Anything below the lean
-        // exponential's range (-inf inputs, very long tails) sends the wavefront
-        // through the library routine; NaN passes through either form as NaN.
-        // The smallest d of this lane is its minimum less the row's maximum.
-#pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
-            if (v >= keep_vecs) continue;
-            widen8<T>(cur[k], f[k]);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) f[k][e] -= mx;
-            if (v * 8 + 8 > keep) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) f[k][e] = v * 8 + e < keep ? f[k][e] : 0.0f;
-            }
-        }
+        // d = x - max <= 0.  Anything below the lean exponential's range (-inf
+        // inputs, very long tails) sends the wavefront through the library
+        // routine; NaN passes through either form as NaN.  The smallest d of
+        // this lane is its minimum less the row's maximum.
         const float lowest = mn - mx;// +inf - max for a lane without kept elements: passes the test below
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
+        float f[NV][8];
         float part = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = k * BS + threadIdx.x;
             if (v >= keep_vecs) continue;
+            widen8<T>(cur[k], f[k]);
             if (lean) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) f[k][e] = exp_nonpositive(f[k][e]);
+                for (int e = 0; e < 8; ++e) f[k][e] = exp_nonpositive(f[k][e] - mx);
             } else {
+                float slow[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) f[k][e] = exp_any(f[k][e]);
+                for (int e = 0; e < 8; ++e) slow[e] = f[k][e];
+                exp_any8(slow, mx);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[k][e] = slow[e];
             }
-            if (v * 8 + 8 > keep) {
+            const bool straddles = tail != 0 && v + 1 == keep_vecs;
+            if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                if (straddles) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) f[k][e] = v * 8 + e < keep ? f[k][e] : 0.0f;
+                    for (int e = 0; e < 8; ++e) f[k][e] = static_cast<uint32_t>(e) < tail ? f[k][e] : 0.0f;
+                }
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) part += f[k][e];
@@ -187,11 +192,19 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
                     const float q = f[k][e] * rcp;// e / sum: one residual step makes the quotient correctly rounded in all but rare cases
                     o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, f[k][e]), rcp, q);
                 }
-                if (v * 8 + 8 > keep) {// boundary vector: its masked tail is zero even when the row turned to NaN
+                u32x4 packed = narrow8_unit_range<T>(o);
+                const bool straddles = tail != 0 && v + 1 == keep_vecs;
+                if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                    if (straddles) {// its masked tail is zero whatever the row turned into
+                        uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) o[e] = v * 8 + e < keep ? o[e] : 0.0f;
+                        for (int e = 0; e < 8; ++e) {
+                            if (static_cast<uint32_t>(e) >= tail) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                        }
+                        packed = u32x4{w[0], w[1], w[2], w[3]};
+                    }
                 }
-                out.st16(v * 16, narrow8_unit_range<T>(o));
+                out.st16(v * 16, packed);
             } else if (v < nvec) {
                 out.st16(v * 16, u32x4{0, 0, 0, 0});
             }
@@ -200,28 +213,16 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
 
     uint64_t r = blockIdx.x;
     if (r >= rows) return;
-    u32x4 xa[NV], xb[NV];
-    Row ra = here(), rb = ra;
-    load_row(ra, xa);
+    int phase = 0;// alternates the LDS slots, so that one barrier per reduction is enough
     while (true) {
-        if (r + hop >= rows) {
-            finish_row(ra, xa, 0);
-            break;
-        }
-        advance();
-        rb = here();
-        load_row(rb, xb);
-        finish_row(ra, xa, 0);
+        u32x4 x[NV];
+        const Row row = here();
+        load_row(row, x);
+        finish_row(row, x, phase);
+        phase ^= 1;
         r += hop;
-        if (r + hop >= rows) {
-            finish_row(rb, xb, 1);
-            break;
-        }
+        if (r >= rows) return;
         advance();
-        ra = here();
-        load_row(ra, xa);
-        finish_row(rb, xb, 1);
-        r += hop;
     }
 }
 
@@ -255,25 +256,21 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
     // Rows of up to 4096 elements are taken by single wavefronts (no barrier, no
-    // LDS), longer ones by 256-1024 lanes.
-    // Measured on MI355X at [32, 4096, 4096] fp16: one row per wavefront is
-    // 6-13 % faster than 128, 256 or 512 lanes per row.  The grid of the
-    // single-wavefront form is several times what the chip holds at once
-    // (16 such wavefronts per compute unit), so the dispatcher evens out the
-    // triangular load while each workgroup still prefetches across its few
-    // rows: 32 workgroups per unit 314 us, 64 288, 96 281, 128 277, 256 278,
-    // one workgroup per row 293.
-    // Both forms get a grid several times what is resident.  Short rows: 128
-    // workgroups per unit at 4096 elements, 512 for 2048 and shorter
-    // ([128, 2048, 2048]: 274 us with 512, 302 with 128).  Long rows: 64 per
-    // unit ([8, 8192, 8192]: 272 us against 300 with 8; [2, 16384, 16384]: 268
-    // against 289).
-    uint64_t per_cu = 64;
-    if (nvec <= 512) {
-        per_cu = nvec > 256 ? 128 : 512;
-    }
-    const uint64_t cap = static_cast<uint64_t>(d.cu_count) * per_cu;
-    const unsigned grid = static_cast<unsigned>(rows < cap ? rows : cap);
+    // LDS), longer ones by 256-1024 lanes.  Measured on MI355X, fp16 / bf16:
+    //   [32, 4096, 4096]   one workgroup per row 264 / 261-266 us (76 %), 256 workgroups per
+    //                      compute unit 267 / 267-274, 64 per unit 293 / 292-299; 128 or 256
+    //                      lanes per row 264-288 / 261-270
+    //   [128, 2048, 2048]  one per row 261 / 258-266, 512 per unit 263 / 262-265
+    //   [512, 1024, 1024]  one per row 262 / 253-264, 512 per unit 285 / 283-285
+    //   [2048, 512, 512]   one per row 396 / 362, 512 per unit 361 / 332
+    //   [8, 8192, 8192]    one per row 268 / 256-265, 64 per unit 272-274 / 270-274
+    //   [2, 16384, 16384]  one per row 277-280, 64 per unit 282-284
+    // so every row gets a workgroup of its own - the dispatcher then evens out
+    // the causal triangle by itself - except rows of 512 elements and fewer,
+    // where a workgroup's start costs as much as its row.
+    const uint64_t cap = nvec <= 64 ? static_cast<uint64_t>(d.cu_count) * 512 : rows;
+    const uint64_t limit = amd::max_grid_1d(1024);// the kernel strides over what the grid does not cover
+    const unsigned grid = static_cast<unsigned>(std::min({rows, cap, limit}));
 
     const bool vec_ok = d.total % 8 == 0 && nvec <= 4096 && d.seq < (1ull << 31) && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);
     if (!vec_ok) {
@@ -281,13 +278,13 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         return;
     }
     const bool through = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
-#define CS_LAUNCH(BS, NV)                                                                                                          \
-    do {                                                                                                                           \
-        if (through)                                                                                                               \
-            causal_softmax_rows<T, BS, NV, true><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),                  \
+#define CS_LAUNCH(BS, NV)                                                                                                      \
+    do {                                                                                                                       \
+        if (through)                                                                                                           \
+            causal_softmax_rows<T, BS, NV, true><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),              \
                                                                           static_cast<uint32_t>(d.total), d.stride_b, d.stride_i); \
-        else                                                                                                                       \
-            causal_softmax_rows<T, BS, NV, false><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),                 \
+        else                                                                                                                   \
+            causal_softmax_rows<T, BS, NV, false><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),             \
                                                                            static_cast<uint32_t>(d.total), d.stride_b, d.stride_i); \
     } while (0)
     if (nvec <= 64) CS_LAUNCH(64, 1);
