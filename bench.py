@@ -91,6 +91,34 @@ class Launch:
             raise RuntimeError(f"{self.name}: status {st}")
 
 
+class CopyYardstick:
+    """A plain device-to-device copy that moves `nbytes` in all (half read,
+    half written) through the HIP runtime's own hipMemcpyAsync: what the
+    platform achieves on the same byte count with no arithmetic and no access
+    pattern to speak of, fixed launch cost included.  A yardstick beside the
+    operators' rows, not a part of the library."""
+
+    _hip = None
+
+    def __init__(self, nbytes):
+        import torch
+
+        if CopyYardstick._hip is None:
+            CopyYardstick._hip = ctypes.CDLL("libamdhip64.so")
+            CopyYardstick._hip.hipMemcpyAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
+            CopyYardstick._hip.hipMemcpyAsync.restype = ctypes.c_int
+        self.half = max(16, nbytes // 2 // 16 * 16)
+        self.src = torch.empty(self.half, dtype=torch.uint8, device="cuda").random_(0, 256)
+        self.dst = torch.empty(self.half, dtype=torch.uint8, device="cuda")
+        self.nbytes = 2 * self.half
+        self.name = "copy"
+
+    def __call__(self, stream):
+        st = CopyYardstick._hip.hipMemcpyAsync(self.dst.data_ptr(), self.src.data_ptr(), self.half, 3, stream)  # 3 = device to device
+        if st != 0:
+            raise RuntimeError(f"hipMemcpyAsync: error {st}")
+
+
 def _randn(shape, dtype, gen):
     import torch
 
@@ -341,6 +369,13 @@ def op_entry(name, config, sets, steps, warmup, repeats):
            "calls_per_run": steps, "runs": repeats, "warmup_calls": warmup}
     if getattr(sets[0], "latency_bound", False):
         row.update({"bound": "latency", "frac_of_peak": None})
+    elif not sets[0].flops and repeats > 1:
+        # the same byte count as a plain runtime copy, timed the same way
+        copies = [CopyYardstick(nbytes) for _ in sets]
+        copy_runs = sorted(time_rotating([[c] for c in copies], steps, warmup if rep == 0 else 0)[1] / steps for rep in range(repeats))
+        copy_us = copy_runs[len(copy_runs) // 2] * 1e6
+        row.update({"copy_same_bytes_us": round(copy_us, 3), "speed_vs_copy": round(copy_us / (per_call * 1e6), 4)})
+        del copies
     if sets[0].flops:
         tflops = sets[0].flops / per_call / 1e12
         row.update({"bound": "mfma", "flops": sets[0].flops, "tflop_per_s": round(tflops, 1),
@@ -394,6 +429,7 @@ def ops_table(ctx, args, gen):
         "S2 random_sample f16 voc 32000, greedy": lambda: [make_random_sample(ctx, 32000, 1, gen, "random_sample") for _ in range(MAX_SETS)],
         "S3 random_sample f16 voc 151936, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 50, gen, "random_sample") for _ in range(MAX_SETS)],
         "S4 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8, no workspace (one workgroup)": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample", False) for _ in range(MAX_SETS)],
+        "S5 random_sample f16 voc 151936, top-k = voc (more than 1024 candidates), top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 151936, gen, "random_sample") for _ in range(MAX_SETS)],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
         "N1b causal_softmax bf16 [32,4096,4096] (the Attention row's softmax on its own)": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, bf16, gen, "causal_softmax") for _ in range(2)],
     }
@@ -521,6 +557,7 @@ def cpu_per_op(T):
     out["S4 random_sample"] = dict(out["S1 random_sample"])  # the same call, served by one workgroup on the GPU
     run("S2 random_sample", "f16", lambda: oracle.random_sample(l9[:32000], 0.37, 0.0, 1, 0.8), lambda: ref.random_sample(l9[:32000], 0.37, 0.0, 1, 0.8))
     run("S3 random_sample", "f16", lambda: oracle.random_sample(l9, 0.37, 0.9, 50, 0.8), lambda: ref.random_sample(l9, 0.37, 0.9, 50, 0.8))
+    # S5 (top-k = the whole vocabulary) has no CPU column: the reference's selection loop is O(topk * voc), about 100 s per call here
     return out
 
 
