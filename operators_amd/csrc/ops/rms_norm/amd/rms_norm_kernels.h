@@ -570,19 +570,20 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // unit, else it re-reads them from memory like a one-row workgroup does.
     const uint64_t lds_bytes = d * sizeof(float);
     const uint64_t lds_limit = static_cast<uint64_t>(desc.lds_per_block) - 1024;
-    // With the next row always in flight, one workgroup per compute unit already
-    // reaches the bandwidth this access pattern allows (measured at [8192, 8192]
-    // bf16: 1, 2, 3 and 4 per unit all give 73.3-74.0 % of peak); 2 keeps some
-    // slack while staging the weights only 512 times.  Shorter rows put fewer
-    // bytes in flight per workgroup, so they get proportionally more of them.
-    uint64_t per_cu = ceil_div(32 * 1024, d * sizeof(uint16_t));
-    per_cu = per_cu < 2 ? 2 : per_cu;
+    // How many workgroups per compute unit.  With the next row always in flight
+    // a workgroup keeps two rows' worth of loads outstanding, and what measures
+    // best is 20-32 KiB of them per compute unit, not more: bf16 rows with fp32
+    // weights, 128 MiB in all, 1 / 2 / 3 / 4 workgroups per unit -
+    //   d =  5120:  49.4 / 44.9 / 46.6 / 47.4 us      d = 10240:  45.6 / 47.0 / 48.3 / 48.3 us
+    //   d =  6144:  45.8 / 45.4 / 47.1 / 47.9 us      d = 12288:  45.3 / 46.9 / 47.2 / 47.1 us
+    //   d =  7168:  45.6 / 47.0 / 46.3 / 47.4 us      d = 16384:  46.7 / 46.7 us
+    //   d =  8192:  44.6 / 44.8 / 45.2 / 45.5 us
+    // so rows of up to 12 KiB get two workgroups per unit and longer ones one.
+    uint64_t per_cu = d * sizeof(uint16_t) > 12 * 1024 ? 1 : 2;
     int home = kWLds;
-    if (lds_bytes <= lds_limit && lds_bytes <= 64 * 1024) {
-        const uint64_t fit = (160 * 1024) / (lds_bytes + 256);// 160 KiB of LDS per compute unit
-        per_cu = fit < per_cu ? fit : per_cu;
-    } else {
+    if (lds_bytes > lds_limit || lds_bytes > 64 * 1024) {
         home = kWGlobal;
+        per_cu = 2;
     }
     uint64_t grid = static_cast<uint64_t>(desc.cu_count) * per_cu;
     if (n <= grid) {
@@ -602,15 +603,44 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res)
 #define RMS_LAUNCH(BS, NV)                                                                                             \
     do {                                                                                                               \
-        const bool exact = !ADD && nvec == static_cast<uint64_t>(BS) * NV; /* the fused form keeps one variant */      \
         if (home != kWLds) RMS_GO(BS, NV, kWGlobal, 0, false, false);                                                  \
-        else if (exact && through) RMS_GO(BS, NV, kWLds, lds_bytes, !ADD, true);                                       \
-        else if (exact) RMS_GO(BS, NV, kWLds, lds_bytes, !ADD, false);                                                 \
         else if (through) RMS_GO(BS, NV, kWLds, lds_bytes, false, true);                                               \
         else RMS_GO(BS, NV, kWLds, lds_bytes, false, false);                                                           \
     } while (0)
 
-    if (nvec <= 1024) RMS_LAUNCH(256, 4);// d = 8192: 512x2 measures the same, 1024x1 is 8 % slower
+    // Row lengths of common models get a shape that fits them exactly, two or
+    // three vectors per lane where that measures best (us per 128 MiB of bf16
+    // rows, against the general ladder below):
+    //   d =  5120: 320 x 2  47.5 (256 x 4: 48.4, 640 x 1: 51.5)   d = 10240: 640 x 2  47.1 (512 x 4: 49.7)
+    //   d =  6144: 256 x 3  46.8 (256 x 4: 48.5, 384 x 2: 47.6)   d = 12288: 512 x 3  46.4 (512 x 4: 48.9, 768 x 2: 47.2)
+    //   d =  7168: 896 x 1  46.1 (256 x 4: 48.0, 448 x 2: 47.5)   d = 14336: 896 x 2  48.0 (512 x 4: 48.3)
+    //   d =  8192: 512 x 2  43.4-44.7 (256 x 4: 44.3-44.8, 1024 x 1: 44.2-45.0)
+    //   d = 16384: 512 x 4  46.4 (1024 x 2: 47.5)
+    // The fused form keeps the ladder, whose kernels predicate the vectors a
+    // row does not have: one variant per shape.
+    if constexpr (!ADD) {
+        if (home == kWLds) {
+#define RMS_EXACT(BS, NV)                                        \
+    do {                                                         \
+        if (through) RMS_GO(BS, NV, kWLds, lds_bytes, true, true); \
+        else RMS_GO(BS, NV, kWLds, lds_bytes, true, false);      \
+        return;                                                  \
+    } while (0)
+            switch (nvec) {
+                case 640: RMS_EXACT(320, 2);
+                case 768: RMS_EXACT(256, 3);
+                case 896: RMS_EXACT(896, 1);
+                case 1024: RMS_EXACT(512, 2);
+                case 1280: RMS_EXACT(640, 2);
+                case 1536: RMS_EXACT(512, 3);
+                case 1792: RMS_EXACT(896, 2);
+                case 2048: RMS_EXACT(512, 4);
+                default: break;
+            }
+#undef RMS_EXACT
+        }
+    }
+    if (nvec <= 1024) RMS_LAUNCH(256, 4);
     else if (nvec <= 2048) RMS_LAUNCH(512, 4);
     else if (nvec <= 4096) RMS_LAUNCH(1024, 4);
     else RMS_LAUNCH(1024, 8);

@@ -46,7 +46,11 @@ def test_golden_odd_sizes(ctx):
 
 
 @pytest.mark.parametrize("dt,wdt", [("f16", "f16"), ("f16", "f32"), ("bf16", "f32"), ("bf16", "bf16")])
-@pytest.mark.parametrize("n,d", [(16, 2048), (3, 8), (700, 512), (9, 4096), (5, 8192), (1100, 8192), (3, 16384), (2, 32768), (2, 65536), (2, 70000), (4, 1023)])
+@pytest.mark.parametrize("n,d", [(16, 2048), (3, 8), (700, 512), (9, 4096), (5, 8192), (1100, 8192), (3, 16384), (2, 32768), (2, 65536), (2, 70000), (4, 1023),
+                                 # widths of common models, more rows than workgroups (the looping kernels with their exact launch shapes)
+                                 (1100, 5120), (1030, 6144), (600, 7168), (520, 10240), (300, 12288), (290, 14336), (280, 16384),
+                                 # and two of them with an output large enough to be written through L2
+                                 (5600, 6144), (4700, 7168)])
 def test_against_oracle(ctx, dt, wdt, n, d):
     rng = np.random.default_rng(n * 7 + d)
     x = oracle.encode(rng.standard_normal((n, d)).astype(np.float32), dt)
