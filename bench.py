@@ -430,6 +430,7 @@ def ops_table(ctx, args, gen):
         "S3 random_sample f16 voc 151936, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 50, gen, "random_sample") for _ in range(MAX_SETS)],
         "S4 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8, no workspace (one workgroup)": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample", False) for _ in range(MAX_SETS)],
         "S5 random_sample f16 voc 151936, top-k = voc (more than 1024 candidates), top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 151936, gen, "random_sample") for _ in range(MAX_SETS)],
+        "Q1 rms_norm bf16 [524288,128] w f32 (a per-head norm: 8192 tokens x 64 heads)": lambda: [make_rms_norm(ctx, 524288, 128, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * 524288 * 128, nset))],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
         "N1b causal_softmax bf16 [32,4096,4096] (the Attention row's softmax on its own)": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, bf16, gen, "causal_softmax") for _ in range(2)],
     }

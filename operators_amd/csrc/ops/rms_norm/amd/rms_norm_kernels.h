@@ -438,6 +438,63 @@ __global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t 
     }
 }
 
+// ---- short rows: several rows per wavefront ---------------------------------------
+// Rows of up to 256 elements (the per-head norms of attention: head_dim 64-256)
+// would leave most of a wavefront idle at one row each.  Here P = 8, 16 or 32
+// lanes serve a row, one vector per lane, and a wavefront takes 64 / P
+// consecutive rows; the sum of squares is the first steps of the wavefront
+// tree (amd::wave_sum), stopped at the group's width, which adds the same
+// values in the same order as the full tree would with zeros in the absent
+// lanes - so these rows, too, give the bits every other form gives.
+template<int P>
+__device__ __forceinline__ float segment_sum(float v) {
+    static_assert(P == 8 || P == 16 || P == 32, "lanes per row");
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));// quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));// quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));// row_half_mirror
+    if constexpr (P >= 16) {
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));// row_mirror
+    }
+    if constexpr (P == 32) v += __shfl_xor(v, 16);// the neighbouring row of 16 lanes
+    return v;
+}
+
+template<typename T, int P, bool THROUGH, bool ADD>
+__global__ __launch_bounds__(kWave) void rms_norm_short(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
+                                                        uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
+                                                        Residual<ADD> res) {
+    constexpr uint32_t RPW = kWave / P;// rows per wavefront
+    const uint32_t nvec = d / 8;
+    const uint32_t sub = threadIdx.x % P, rr = threadIdx.x / P;
+    const uint32_t lv = sub < nvec ? sub : 0;
+    float g[8];
+    load_w8(w, w_kind, lv, g);
+    for (uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * RPW; row0 < n; row0 += static_cast<uint64_t>(gridDim.x) * RPW) {
+        const uint64_t row = row0 + rr;
+        const bool have = row < n && sub < nvec;
+        const uint64_t lr = row < n ? row : row0;// absent rows re-read the first one; nothing of them is stored
+        u32x4 xv = ld16_stream(x + static_cast<int64_t>(lr) * stride_x + static_cast<uint64_t>(lv) * 8);
+        if constexpr (ADD) {// the row becomes a + b, rounded as Add rounds, and goes out to c
+            const u32x4 bv = ld16_stream(res.b + static_cast<int64_t>(lr) * res.stride_b + static_cast<uint64_t>(lv) * 8);
+            float p[8], q[8];
+            widen8<T>(xv, p);
+            widen8<T>(bv, q);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) p[i] += q[i];
+            xv = narrow8<T>(p);
+            const StreamOut<THROUGH> cr(res.c + static_cast<int64_t>(row0) * res.stride_c);
+            if (have) cr.st16(rr * static_cast<uint32_t>(res.stride_c) * 2 + sub * 16, xv);
+        }
+        float f[8];
+        widen8<T>(xv, f);
+        const float k_row = inv_rms(segment_sum<P>(sub < nvec ? squares8(f) : 0.0f), d, eps);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
+        const StreamOut<THROUGH> yr(y + static_cast<int64_t>(row0) * stride_y);
+        if (have) yr.st16(rr * static_cast<uint32_t>(stride_y) * 2 + sub * 16, narrow8<T>(f));
+    }
+}
+
 // ---- any row length, any alignment ----------------------------------------------
 // Two passes over the row with element accesses; the second pass re-reads x,
 // which the first pass left in cache for rows of ordinary length.
@@ -543,20 +600,46 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         else if (through) RMS_ONCE_GO(BS, NV, R, false, true);                                                     \
         else RMS_ONCE_GO(BS, NV, R, false, false);                                                                 \
     } while (0)
-    if (nvec <= 64) {
+    // Rows of up to 256 elements, 8 consecutive ones within reach of a 32-bit
+    // byte offset from the first: 2-8 rows per wavefront.
+    bool near = desc.stride_y >= 0 && desc.stride_y < (1 << 26);
+    if constexpr (ADD) near = near && res.stride_c >= 0 && res.stride_c < (1 << 26);
+    if (nvec <= 32 && near) {
+        const unsigned lanes = nvec <= 8 ? 8 : (nvec <= 16 ? 16 : 32);
+        const uint64_t want = ceil_div(n, kWave / lanes), cap = amd::max_grid_1d(kWave);
+        const unsigned grid = static_cast<unsigned>(want < cap ? want : cap);
+#define RMS_SHORT(P)                                                                                                   \
+    do {                                                                                                               \
+        if (through)                                                                                                   \
+            rms_norm_short<T, P, true, ADD><<<grid, kWave, 0, stream>>>(py, px, w, w_kind, n, static_cast<uint32_t>(d), \
+                                                                        desc.stride_y, desc.stride_x, desc.epsilon, res); \
+        else                                                                                                           \
+            rms_norm_short<T, P, false, ADD><<<grid, kWave, 0, stream>>>(py, px, w, w_kind, n, static_cast<uint32_t>(d), \
+                                                                         desc.stride_y, desc.stride_x, desc.epsilon, res); \
+    } while (0)
+        if (lanes == 8) RMS_SHORT(8);
+        else if (lanes == 16) RMS_SHORT(16);
+        else RMS_SHORT(32);
+#undef RMS_SHORT
+        return;
+    }
+    // A one-pass grid has a workgroup per R rows; beyond what one launch can
+    // hold the looping kernels below take over.
+    const auto once_fits = [&](unsigned lanes, unsigned rows) { return ceil_div(n, rows) <= amd::max_grid_1d(lanes); };
+    if (nvec <= 64 && once_fits(64, 1)) {
         RMS_ONCE(64, 1, 1);
         return;
     }
-    if (nvec <= 256) {
+    if (nvec > 64 && nvec <= 256 && once_fits(256, 2)) {
         RMS_ONCE(256, 1, 2);
         return;
     }
-    if (nvec <= 512) {
+    if (nvec > 256 && nvec <= 512 && once_fits(256, 1)) {
         RMS_ONCE(256, 2, 1);
         return;
     }
     if constexpr (ADD) {
-        if (nvec == 1024) {
+        if (nvec == 1024 && once_fits(1024, 1)) {
             if (through) RMS_ONCE_GO(1024, 1, 1, true, true);
             else RMS_ONCE_GO(1024, 1, 1, true, false);
             return;

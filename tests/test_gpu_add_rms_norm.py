@@ -52,7 +52,11 @@ def check_y(got, want, dt, what, max_frac=5e-3):
 
 
 @pytest.mark.parametrize("dt,wdt", [("f16", "f16"), ("f16", "f32"), ("bf16", "f32"), ("bf16", "bf16")])
-@pytest.mark.parametrize("n,d", [(16, 2048), (3, 8), (700, 512), (9, 4096), (1100, 8192), (3, 16384), (2, 65536), (2, 70000), (4, 1023)])
+@pytest.mark.parametrize("n,d", [(16, 2048), (3, 8), (700, 512), (9, 4096), (1100, 8192), (3, 16384), (2, 65536), (2, 70000), (4, 1023),
+                                 # short rows, several to a wavefront (per-head norms), with ragged last wavefronts
+                                 (5001, 128), (1003, 64), (777, 256), (333, 72), (50, 200),
+                                 # widths of common models on the looping kernels
+                                 (600, 5120), (530, 7168), (300, 12288)])
 def test_against_oracle_and_against_the_two_separate_calls(ctx, dt, wdt, n, d):
     a, b, w = inputs(n, d, dt, wdt, n * 11 + d)
     want_c, want_y = oracle.add_rms_norm(a, b, w, 1e-5, dt, wdt)

@@ -50,7 +50,10 @@ def test_golden_odd_sizes(ctx):
                                  # widths of common models, more rows than workgroups (the looping kernels with their exact launch shapes)
                                  (1100, 5120), (1030, 6144), (600, 7168), (520, 10240), (300, 12288), (290, 14336), (280, 16384),
                                  # and two of them with an output large enough to be written through L2
-                                 (5600, 6144), (4700, 7168)])
+                                 (5600, 6144), (4700, 7168),
+                                 # short rows, several to a wavefront (per-head norms): full and ragged last wavefronts, rows that
+                                 # do not fill their lanes, an output large enough to be written through L2
+                                 (5001, 128), (4096, 128), (1003, 64), (777, 256), (333, 72), (101, 16), (50, 200), (270000, 128)])
 def test_against_oracle(ctx, dt, wdt, n, d):
     rng = np.random.default_rng(n * 7 + d)
     x = oracle.encode(rng.standard_normal((n, d)).astype(np.float32), dt)
@@ -70,6 +73,11 @@ def test_row_strides_of_x_and_y_are_independent(ctx):
     want = oracle.rms_norm(x, w, 1e-5, "f16", "f32")
     check(run(ctx, x, w, 1e-5, "f16", "f32", x_stride=4096, y_stride=2304), want, "f16", "strided rows")
     check(run(ctx, x, w, 1e-5, "f16", "f32", x_stride=2049, y_stride=2051), want, "f16", "odd row strides")
+    # short rows (several to a wavefront): one head of 128 out of every 640 elements, written 256 apart
+    x = oracle.encode(rng.standard_normal((1001, 128)).astype(np.float32), "bf16")
+    w = oracle.encode(rng.uniform(0.5, 1.5, 128).astype(np.float32), "f32")
+    want = oracle.rms_norm(x, w, 1e-6, "bf16", "f32")
+    check(run(ctx, x, w, 1e-6, "bf16", "f32", x_stride=640, y_stride=256), want, "bf16", "strided short rows")
 
 
 def test_in_place(ctx):
