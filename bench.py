@@ -415,6 +415,7 @@ def ops_table(ctx, args, gen):
         f"C5 rms_norm bf16 [{T},8192] w f32": lambda: [make_rms_norm(ctx, T, 8192, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * T * 8192, nset))],
         f"C5 rope_q bf16 [{T},64,128] in [{T},80,128]": lambda: rope_sets(T, 80, 0, 64, bf16, T, 5e5, False),
         f"C5 rope_k bf16 [{T},8,128] in [{T},80,128]": lambda: rope_sets(T, 80, 64, 8, bf16, T, 5e5, False),
+        f"C5b rope_qk bf16 [{T},72,128] in [{T},80,128] (q and k of the fused buffer as one 72-head view, one call)": lambda: rope_sets(T, 80, 0, 72, bf16, T, 5e5, False),
         f"C5 swiglu bf16 [{T},28672] fused gate/up": lambda: [make_swiglu(ctx, T, 28672, bf16, True, gen, "swiglu") for _ in range(max(2, nset // 2))],
         f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(sets_needed(6 * T * 8192, nset))],
         # beyond the four-operator path: attention scores of 32 heads, 4096 x 4096, in place
