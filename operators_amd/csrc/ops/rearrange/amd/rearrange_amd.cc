@@ -91,6 +91,13 @@ infiniopStatus_t amdCreateRearrangeDescriptor(AmdHandle_t handle, RearrangeAmdDe
         return STATUS_BAD_TENSOR_SHAPE;
     }
     desc->ndim = n;
+    // The kernels number the rows with dimension 0 varying fastest; any
+    // numbering copies the same bytes.  They are numbered in the tensors' own
+    // dimension order, which for a transposing copy follows the source's
+    // addresses and scatters the writes.  The other way round - rows numbered
+    // by destination address, the source gathered - measured slower on MI355X:
+    // bf16 [8192, 64, 128] out of [8192, 80, 128] -> [64, 8192, 128] 49.6 us
+    // against 43.7 us.
     for (int k = 0; k < n; ++k) {// innermost outer dimension first
         desc->shape[k] = shp[n - 1 - k];
         desc->dst_stride[k] = sd[n - 1 - k];
