@@ -194,16 +194,19 @@ def make_random_sample(ctx, voc, topk, gen, name, use_workspace=True):
     return launch
 
 
-def make_rearrange(ctx, tokens, heads, dtype, gen, name):
-    """[token, head, 128] heads of a fused qkv buffer -> contiguous [head, token, 128] (a cache write / head transpose)."""
+def make_rearrange(ctx, tokens, heads, dtype, gen, name, back=False):
+    """[token, head, 128] heads of a fused qkv buffer -> contiguous [head, token, 128] (a cache write / head transpose);
+    `back`: the other way round, head-major results back into [token, head, 128] of a wider buffer."""
     import torch
 
     from operators_amd.ops import RearrangePlan
 
     qkv = _randn((tokens, heads + 16, 128), dtype, gen)
     src = qkv[:, :heads, :]
-    cache = torch.empty((heads, tokens, 128), dtype=dtype, device="cuda")
+    cache = _randn((heads, tokens, 128), dtype, gen) if back else torch.empty((heads, tokens, 128), dtype=dtype, device="cuda")
     dst = cache.permute(1, 0, 2)  # same logical shape as src, strides (128, tokens*128, 1)
+    if back:
+        src, dst = dst, src
     plan = RearrangePlan(ctx, dst, src)
     return Launch(name, ctx.lib.infiniopRearrange, (plan.desc, dst.data_ptr(), src.data_ptr()), 2 * src.numel() * src.element_size(), (plan, qkv, cache))
 
@@ -420,6 +423,7 @@ def ops_table(ctx, args, gen):
         f"C5 add bf16 [{T},8192]": lambda: [make_add(ctx, T, 8192, bf16, False, gen, "add") for _ in range(sets_needed(6 * T * 8192, nset))],
         # beyond the four-operator path: attention scores of 32 heads, 4096 x 4096, in place
         f"N2 rearrange bf16 [{T},64,128] of [{T},80,128] -> [64,{T},128]": lambda: [make_rearrange(ctx, T, 64, bf16, gen, "rearrange") for _ in range(sets_needed(4 * T * 64 * 128, nset))],
+        f"N2b rearrange bf16 [64,{T},128] -> [{T},64,128] of [{T},80,128] (the way back)": lambda: [make_rearrange(ctx, T, 64, bf16, gen, "rearrange", True) for _ in range(sets_needed(4 * T * 64 * 128, nset))],
         f"F1 add_rms_norm bf16 [{T},8192] w f32 (fused Add + RMSNorm)": lambda: [make_add_rms_norm(ctx, T, 8192, bf16, torch.float32, gen, "add_rms_norm") for _ in range(sets_needed(6 * T * 8192, nset))],
         # GEMM-bound rows (a library GEMM; priced against the MFMA peak): the gate/up projection and the whole MLP of a Llama-70B layer
         f"M1 matmul bf16 [{T},8192] x [8192,57344]": lambda: [make_matmul(ctx, T, 8192, 57344, bf16, gen, "matmul") for _ in range(2)],

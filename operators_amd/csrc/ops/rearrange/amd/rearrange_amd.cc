@@ -93,11 +93,17 @@ infiniopStatus_t amdCreateRearrangeDescriptor(AmdHandle_t handle, RearrangeAmdDe
     desc->ndim = n;
     // The kernels number the rows with dimension 0 varying fastest; any
     // numbering copies the same bytes.  They are numbered in the tensors' own
-    // dimension order, which for a transposing copy follows the source's
-    // addresses and scatters the writes.  The other way round - rows numbered
-    // by destination address, the source gathered - measured slower on MI355X:
-    // bf16 [8192, 64, 128] out of [8192, 80, 128] -> [64, 8192, 128] 49.6 us
-    // against 43.7 us.
+    // dimension order.  Sorting the dimensions by destination stride (writes
+    // in address order, the source gathered) or by source stride (the
+    // reverse) was measured on MI355X with the head transpose of attention,
+    // bf16 [8192, 64, 128] inside [8192, 80, 128] <-> dense [64, 8192, 128]:
+    // into the dense tensor 43.4 us as is and 49.6 us by destination order;
+    // back out of it 42.3 us as is and 58.6 us by source order.  In both the
+    // tensors' own order walks the 64 heads of a token first - 16 KiB in one
+    // piece on the wide side, 2 MiB steps on the dense side - and the sorted
+    // order walks tokens first, 20 KiB steps on the wide side, which is what
+    // costs.  No rule based on one tensor's strides alone gets both right, so
+    // the order is left as the caller wrote it.
     for (int k = 0; k < n; ++k) {// innermost outer dimension first
         desc->shape[k] = shp[n - 1 - k];
         desc->dst_stride[k] = sd[n - 1 - k];
