@@ -100,6 +100,23 @@ __device__ __forceinline__ float row_sum(const float (&s)[NV], float *slots) {
     return total;
 }
 
+// The same sum for a lane count known only at launch (waves >= 2).  (Fetching
+// the chunk sums with one LDS read, one per lane, and adding them out of that
+// register lane by lane measured 1-8 % slower than this loop of LDS reads.)
+template<int NV>
+__device__ __forceinline__ float row_sum_any(const float (&s)[NV], float *slots, uint32_t waves) {
+    const uint32_t wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const float c = wave_sum(s[k]);
+        if ((threadIdx.x & (kWave - 1)) == 0) slots[k * waves + wave] = c;
+    }
+    __syncthreads();
+    float total = 0.0f;
+    for (uint32_t j = 0; j < NV * waves; ++j) total += slots[j];
+    return total;
+}
+
 // One vector's sum of squares: pairwise, each pair as one product and one
 // fused multiply-add (the library is compiled with contraction off for RoPE's
 // sake; here fusing costs nothing - the sum's order already differs from the
@@ -164,11 +181,14 @@ struct Residual<true> {
 namespace {
 
 template<typename T, int BS, int NV, int WHOME, bool EXACT, bool THROUGH, bool ADD>
-__global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
+__global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                      uint64_t first_mul, uint64_t hop, uint64_t span, Residual<ADD> res) {
-    constexpr int WAVES = BS / kWave;
-    __shared__ float red[2 * NV * WAVES];// two sets of chunk sums, used in turn: one barrier per row is enough
+    // BS = 0: the lane count is the launch's (any multiple of 64 up to 1024)
+    constexpr int MAX_WAVES = (BS != 0 ? BS : 1024) / kWave;
+    const uint32_t bs = BS != 0 ? BS : blockDim.x;
+    [[maybe_unused]] const uint32_t waves = bs / kWave;
+    __shared__ float red[2 * NV * MAX_WAVES];// two sets of chunk sums, used in turn: one barrier per row is enough
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
     f32x4 *w_lo = reinterpret_cast<f32x4 *>(dyn_lds);
     const uint32_t nvec = d / 8;
@@ -179,14 +199,14 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
         const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
+            const uint32_t v = k * bs + threadIdx.x;
             dst[k] = ld16_stream(xr + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
         }
         if constexpr (ADD) {
             const uint16_t *br = res.b + static_cast<int64_t>(row) * res.stride_b;
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                const uint32_t v = k * BS + threadIdx.x;
+                const uint32_t v = k * bs + threadIdx.x;
                 dst_b[k] = ld16_stream(br + static_cast<uint64_t>(EXACT || v < nvec ? v : 0) * 8);
             }
         }
@@ -210,14 +230,14 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
             float g[NV][8];
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                const uint32_t v = k * BS + threadIdx.x;
+                const uint32_t v = k * bs + threadIdx.x;
                 W::load8(w, EXACT || v < nvec ? v : 0, g[k]);
             }
             if (more) load_row(row + hop, xn, bn);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                const uint32_t v = k * BS + threadIdx.x;
+                const uint32_t v = k * bs + threadIdx.x;
                 if (EXACT || v < nvec) {
                     w_lo[v] = f32x4{g[k][0], g[k][1], g[k][2], g[k][3]};
                     w_hi[v] = f32x4{g[k][4], g[k][5], g[k][6], g[k][7]};
@@ -238,7 +258,7 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
             const StreamOut<THROUGH> cr(res.c + static_cast<int64_t>(r) * res.stride_c);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                const uint32_t v = k * BS + threadIdx.x;
+                const uint32_t v = k * bs + threadIdx.x;
                 float p[8], q[8];
                 widen8<T>(cur[k], p);
                 widen8<T>(cur_b[k], q);
@@ -253,14 +273,14 @@ __global__ __launch_bounds__(BS) void rms_norm_rows(uint16_t *y, const uint16_t 
         for (int k = 0; k < NV; ++k) {
             float f[8];
             widen8<T>(cur[k], f);
-            part[k] = EXACT || k * BS + threadIdx.x < nvec ? squares8(f) : 0.0f;
+            part[k] = EXACT || k * bs + threadIdx.x < nvec ? squares8(f) : 0.0f;
         }
-        const float k_row = inv_rms(row_sum<WAVES, NV>(part, red + phase * NV * WAVES), d, eps);
+        const float k_row = inv_rms((BS != 0 ? row_sum<MAX_WAVES, NV>(part, red + phase * NV * MAX_WAVES) : row_sum_any<NV>(part, red + phase * NV * MAX_WAVES, waves)), d, eps);
 
         const StreamOut<THROUGH> yr(y + static_cast<int64_t>(r) * stride_y);// a row is far shorter than 4 GiB
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
+            const uint32_t v = k * bs + threadIdx.x;
             if (EXACT || v < nvec) {
                 float f[8], g[8];
                 widen8<T>(cur[k], f);
@@ -580,7 +600,8 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // (and [8192, 8192] for the fused form), one pass (R rows per workgroup,
     // weights in registers) against looping workgroups (weights in LDS):
     //   d =  512:  41.2 us one pass, R = 1          46.9 us looping
-    //   d = 1024:  46.7 us one pass, R = 2 (59.0 with R = 1)   51.2 us looping
+    //   d =  768:  43.9 us one pass with 128 lanes, R = 2 (45.6 with R = 4; 54.8 with 256 lanes)
+    //   d = 1024:  43.8 us one pass with 128 lanes, R = 2 (45.1 with R = 4); 45.5-46.7 with 256 lanes, R = 2 (59.0 with R = 1)   51.2 us looping
     //   d = 2048:  44.4 us one pass, R = 2 (47.0 with R = 1)   47.9 us looping
     //   d = 4096:  45.5 us one pass, R = 1 (46.4 with R = 2)   46.6 us looping
     //   d = 8192:  45.6-50.3 us one pass            44.6 us looping
@@ -630,7 +651,11 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         RMS_ONCE(64, 1, 1);
         return;
     }
-    if (nvec > 64 && nvec <= 256 && once_fits(256, 2)) {
+    if (nvec > 64 && nvec <= 128 && once_fits(128, 2)) {
+        RMS_ONCE(128, 1, 2);
+        return;
+    }
+    if (nvec > 128 && nvec <= 256 && once_fits(256, 2)) {
         RMS_ONCE(256, 1, 2);
         return;
     }
@@ -691,34 +716,58 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         else RMS_GO(BS, NV, kWLds, lds_bytes, false, false);                                                           \
     } while (0)
 
-    // Row lengths of common models get a shape that fits them exactly, two or
-    // three vectors per lane where that measures best (us per 128 MiB of bf16
-    // rows, against the general ladder below):
-    //   d =  5120: 320 x 2  47.5 (256 x 4: 48.4, 640 x 1: 51.5)   d = 10240: 640 x 2  47.1 (512 x 4: 49.7)
-    //   d =  6144: 256 x 3  46.8 (256 x 4: 48.5, 384 x 2: 47.6)   d = 12288: 512 x 3  46.4 (512 x 4: 48.9, 768 x 2: 47.2)
-    //   d =  7168: 896 x 1  46.1 (256 x 4: 48.0, 448 x 2: 47.5)   d = 14336: 896 x 2  48.0 (512 x 4: 48.3)
-    //   d =  8192: 512 x 2  43.4-44.7 (256 x 4: 44.3-44.8, 1024 x 1: 44.2-45.0)
-    //   d = 16384: 512 x 4  46.4 (1024 x 2: 47.5)
-    // The fused form keeps the ladder, whose kernels predicate the vectors a
-    // row does not have: one variant per shape.
+    // Row lengths of common models get a launch shape that fits them exactly
+    // (lanes x vectors per lane = the row), two or three vectors per lane
+    // where that measures best (us per 128 MiB of bf16 rows; the last figure
+    // of each line is the general ladder below, which predicates the vectors
+    // a row does not have):
+    //   d =  5120: 320 x 2  47.5   640 x 1  51.5                  256 x 4  48.4
+    //   d =  6144: 256 x 3  46.8   384 x 2  47.6                  256 x 4  48.5
+    //   d =  7168: 896 x 1  46.1   448 x 2  47.5                  256 x 4  48.0
+    //   d =  8192: 512 x 2  43.4-44.7   1024 x 1  44.2-45.0       256 x 4  44.3-44.8
+    //   d = 10240: 640 x 2  47.1                                  512 x 4  49.7
+    //   d = 12288: 512 x 3  46.4   768 x 2  47.2                  512 x 4  48.9
+    //   d = 14336: 896 x 2  48.0                                  512 x 4  48.3
+    //   d = 16384: 512 x 4  46.4   1024 x 2  47.5
+    // Any other multiple of 512 elements gets its exact shape from the same
+    // kernel with the lane count taken from the launch (d = 4608: 46.6 against
+    // 48.2 on the ladder; d = 9216: 45.6 against 50.3), which at the widths
+    // above is 0.5-2.5 % slower than the kernels compiled for them.  The fused
+    // form keeps the ladder: an exact shape gained it nothing (d = 5120: 96.6
+    // against 97.6).
     if constexpr (!ADD) {
-        if (home == kWLds) {
-#define RMS_EXACT(BS, NV)                                        \
-    do {                                                         \
-        if (through) RMS_GO(BS, NV, kWLds, lds_bytes, true, true); \
-        else RMS_GO(BS, NV, kWLds, lds_bytes, true, false);      \
-        return;                                                  \
+        if (home == kWLds && nvec % kWave == 0) {
+#define RMS_EXACT(BS, NV, LANES)                                                                                       \
+    do {                                                                                                               \
+        if (through)                                                                                                   \
+            rms_norm_rows<T, BS, NV, kWLds, true, true, ADD><<<static_cast<unsigned>(grid), LANES, lds_bytes, stream>>>( \
+                py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res); \
+        else                                                                                                           \
+            rms_norm_rows<T, BS, NV, kWLds, true, false, ADD><<<static_cast<unsigned>(grid), LANES, lds_bytes, stream>>>( \
+                py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res); \
+        return;                                                                                                        \
     } while (0)
             switch (nvec) {
-                case 640: RMS_EXACT(320, 2);
-                case 768: RMS_EXACT(256, 3);
-                case 896: RMS_EXACT(896, 1);
-                case 1024: RMS_EXACT(512, 2);
-                case 1280: RMS_EXACT(640, 2);
-                case 1536: RMS_EXACT(512, 3);
-                case 1792: RMS_EXACT(896, 2);
-                case 2048: RMS_EXACT(512, 4);
+                case 640: RMS_EXACT(320, 2, 320);
+                case 768: RMS_EXACT(256, 3, 256);
+                case 896: RMS_EXACT(896, 1, 896);
+                case 1024: RMS_EXACT(512, 2, 512);
+                case 1280: RMS_EXACT(640, 2, 640);
+                case 1536: RMS_EXACT(512, 3, 512);
+                case 1792: RMS_EXACT(896, 2, 896);
+                case 2048: RMS_EXACT(512, 4, 512);
                 default: break;
+            }
+            const uint64_t m = nvec / kWave;
+            for (int cand : {2, 3, 4, 1}) {
+                const unsigned lanes = static_cast<unsigned>(kWave * m / cand);
+                if (m % cand != 0 || lanes < 256 || lanes > 1024) continue;
+                switch (cand) {
+                    case 1: RMS_EXACT(0, 1, lanes);
+                    case 2: RMS_EXACT(0, 2, lanes);
+                    case 3: RMS_EXACT(0, 3, lanes);
+                    default: RMS_EXACT(0, 4, lanes);
+                }
             }
 #undef RMS_EXACT
         }

@@ -49,6 +49,8 @@ def test_golden_odd_sizes(ctx):
 @pytest.mark.parametrize("n,d", [(16, 2048), (3, 8), (700, 512), (9, 4096), (5, 8192), (1100, 8192), (3, 16384), (2, 32768), (2, 65536), (2, 70000), (4, 1023),
                                  # widths of common models, more rows than workgroups (the looping kernels with their exact launch shapes)
                                  (1100, 5120), (1030, 6144), (600, 7168), (520, 10240), (300, 12288), (290, 14336), (280, 16384),
+                                 # other multiples of 512 (the kernel whose lane count is the launch's): 576 x 1, 576 x 2, 704 x 2, 832 x 1 lanes x vectors
+                                 (1100, 4608), (300, 9216), (280, 11264), (290, 6656),
                                  # and two of them with an output large enough to be written through L2
                                  (5600, 6144), (4700, 7168),
                                  # short rows, several to a wavefront (per-head norms): full and ragged last wavefronts, rows that
