@@ -123,12 +123,19 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         // with 64 lanes and 42.1 us with 256; 8 KiB rows (8 wavefronts each) 57.5
         // against 42.1 us, 2 KiB rows 61.0 against 46.3 us.
         const bool wave_rows = kBlock == kWave && upr >= 16 * kWave;
-        const int lanes = wave_rows ? kWave : 256;
+        // Rows that fill 128-lane workgroups better than 256-lane ones get those: 128 MiB of bf16 rows out
+        // of a buffer twice as wide, 2816 elements per row (352 units) 43.3 us against 51.5 us, 3072 per row
+        // 42.8 against 50.0, 6912 per row 42.7 against 45.1; nothing between them where both fit equally.
+        const bool half = !wave_rows && ceil_div(upr, 128) * 128 < ceil_div(upr, 256) * 256;
+        const int lanes = wave_rows ? kWave : (half ? 128 : 256);
         const dim3 grid(static_cast<unsigned>(ceil_div(upr, lanes)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
         const bool bufst = BYTES == 16 && large && desc.row_bytes < (1ull << 32);
         if (wave_rows) {
             if (bufst) rearrange_rows<BYTES, BYTES == 16, kWave><<<grid, kWave, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
             else rearrange_rows<BYTES, false, kWave><<<grid, kWave, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+        } else if (half) {
+            if (bufst) rearrange_rows<BYTES, BYTES == 16, 128><<<grid, 128, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
+            else rearrange_rows<BYTES, false, 128><<<grid, 128, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
         } else {
             if (bufst) rearrange_rows<BYTES, BYTES == 16, 256><<<grid, 256, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
             else rearrange_rows<BYTES, false, 256><<<grid, 256, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
