@@ -21,7 +21,7 @@ bounded sample of the same workload; `ops` lists every operator/configuration
 with its own time, bandwidth and fraction of the 8 TB/s peak: per row one cold
 first call (buffers never touched before; includes one-time code loading where
 the kernel has not run yet in the process), then at least 20 warm-up calls and
-5 runs of at least 40 calls each between two events, rotating over buffer
+5 runs of at least 200 calls each (40 for the GEMM-bound rows) between two events, rotating over buffer
 sets; `us_per_call` is the median run, `us_min`/`us_max` the fastest and
 slowest.
 """
@@ -453,12 +453,14 @@ def ops_table(ctx, args, gen):
         if args.only and args.only not in label:
             continue
         sets = build()
-        # the table proper: 20 warm-up calls, 5 runs of >= 40 calls, median; a single
-        # named row (profiling) runs exactly what was asked for, once
+        # the table proper: 20 warm-up calls, 5 runs of >= 200 calls (>= 40 for the GEMM-bound
+        # rows, which take milliseconds each), median; a single named row (profiling) runs exactly
+        # what was asked for, once
         if args.only:
             rows.append(op_entry(sets[0].name, label, sets, args.steps, args.warmup, 1))
         else:
-            rows.append(op_entry(sets[0].name, label, sets, max(args.steps, 40), max(args.warmup, 20), 5))
+            calls = 40 if sets[0].flops else 200
+            rows.append(op_entry(sets[0].name, label, sets, max(args.steps, calls), max(args.warmup, 20), 5))
         del sets
         torch.cuda.empty_cache()
     return rows
