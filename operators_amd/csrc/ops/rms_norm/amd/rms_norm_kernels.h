@@ -180,7 +180,7 @@ struct Residual<true> {
 };
 namespace {
 
-template<typename T, int BS, int NV, int WHOME, bool EXACT, bool THROUGH, bool ADD>
+template<typename T, int BS, int NV, int WHOME, bool EXACT, bool THROUGH, bool ADD, bool AHEAD = true>
 __global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                      uint64_t first_mul, uint64_t hop, uint64_t span, Residual<ADD> res) {
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y
     const uint64_t last = row + span < n ? row + span : n;
     u32x4 xv[NV], xn[NV], bv[NB], bn[NB];
     load_row(row, xv, bv);// in flight while the weights are fetched below
-    bool more = row + hop < last;// this workgroup owns a row after the current one
+    bool more = AHEAD && row + hop < last;// this workgroup owns a row after the current one, and fetches it ahead
 
     if constexpr (WHOME == kWLds) {
         // All of this lane's weight loads are issued before the first is
@@ -306,6 +306,16 @@ __global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y
     // way - so that the loop is entered with the memory operations in the
     // order every later pass leaves them in, and the waits inside it count
     // the younger operations instead of draining the queue.
+    if constexpr (!AHEAD) {// one register set: a row is fetched only after the one before it has been stored
+        int phase = 0;
+        while (true) {
+            finish_row(row, xv, bv, phase);
+            phase ^= 1;
+            row += hop;
+            if (row >= last) return;
+            load_row(row, xv, bv);
+        }
+    }
     if (!more) {
         finish_row(row, xv, bv, 0);
         return;
@@ -706,8 +716,13 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // form only (inexact row length, plain non-temporal stores): they serve
     // one-row workgroups and rows too long for LDS, where neither refinement
     // is measurable.
+    // Two register sets (the next row fetched ahead) fit the 128 registers a
+    // lane of a 1024-lane workgroup may have up to 4 vectors per lane, 2 in
+    // the fused form; beyond that the second set would live in scratch
+    // memory, and those shapes work through one row at a time.
 #define RMS_GO(BS, NV, HOME, LDS, EXACT, THROUGH)                                                                      \
-    rms_norm_rows<T, BS, NV, HOME, EXACT, THROUGH, ADD><<<static_cast<unsigned>(grid), BS, LDS, stream>>>(             \
+    rms_norm_rows<T, BS, NV, HOME, EXACT, THROUGH, ADD, (BS * NV * (ADD ? 2 : 1) <= 4096)>                             \
+        <<<static_cast<unsigned>(grid), BS, LDS, stream>>>(                                                            \
         py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res)
 #define RMS_LAUNCH(BS, NV)                                                                                             \
     do {                                                                                                               \
