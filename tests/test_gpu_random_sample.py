@@ -280,3 +280,55 @@ def test_more_candidates_than_lds_ranks_with_ties(ctx):
         if not same_choice(codes, got, want):
             bad.append((trial, voc, args, got, want))
     assert not bad, bad[:5]
+
+
+def test_more_candidates_few_distinct_logits(ctx):
+    """The walk over more than 1024 candidates takes 64 keys at a time while the
+    running sum stays below 1.0 and entry by entry beyond it.  Distributions
+    that put both to work: every logit equal (one key holding the whole
+    vocabulary: the entry inside the key comes from a division), two and
+    three levels, one dominant logit (the running sum is 1.0 after the first
+    entry and everything after it adds nothing or a last unit), logits so far
+    apart that most probabilities are zero, and the entry limit (topk) falling
+    inside a key.  All ties, so the logit at the drawn index must be the
+    oracle's; where the oracle leaves the result unwritten, so must the GPU."""
+    rng = np.random.default_rng(7)
+    f = lambda *v: np.asarray(v, np.float16).view(np.uint16)  # noqa: E731
+    bad = []
+    cases = []
+    for voc in (1500, 4100, 9000):
+        cases.append(("all equal", np.full(voc, f(0.25)[0], np.uint16)))
+        cases.append(("two levels", rng.choice(f(1.0, -1.0), voc)))
+        cases.append(("three levels", rng.choice(f(2.0, 1.5, -3.0), voc, p=[0.01, 0.09, 0.9])))
+        one = np.full(voc, f(-20.0)[0], np.uint16)
+        one[voc // 3] = f(12.0)[0]
+        cases.append(("one dominant", one))
+        far = rng.choice(f(30.0, 0.0, -40.0), voc, p=[0.002, 0.5, 0.498])
+        cases.append(("far apart", far))
+        cases.append(("eight values", rng.choice(f(0.0, 0.5, 1.0, 1.5, 2.0, 2.5, 3.0, 3.5), voc)))
+    for what, codes in cases:
+        voc = codes.size
+        for rv, topp, topk, temp in [(0.37, 0.9, voc, 1.0), (0.999, 1.0, voc, 1.0), (0.0, 1.0, voc, 0.5), (0.6, 0.5, 1025, 2.0),
+                                     (0.95, 1.0, voc - 7, 1.0), (0.5, 1e-3, voc, 1.0), (0.9999, 0.99, 2 * voc, 4.0), (1.0, 1.0, voc, 1.0)]:
+            want = oracle.random_sample(codes, rv, topp, topk, temp)
+            got = gpu_sample(ctx, codes, rv, topp, topk, temp)
+            if not same_choice(codes, got, want):
+                bad.append((what, voc, (rv, topp, topk, temp), got, want))
+    assert not bad, bad[:6]
+
+
+def test_more_candidates_bf16_still_adds_entry_by_entry(ctx):
+    """bf16 probabilities are finer than the 2^-24 units the fast walk counts
+    in, so bf16 logits keep the one-by-one chain: against the oracle's bf16
+    extension on tie-heavy inputs."""
+    rng = np.random.default_rng(8)
+    bad = []
+    for voc in (1400, 5000):
+        x = rng.integers(-24, 24, voc).astype(np.float32) / 4
+        codes = oracle.encode(x, "bf16")
+        for rv, topp, topk, temp in [(0.37, 0.9, voc, 1.0), (0.99, 1.0, voc, 2.0), (0.2, 0.6, 2000, 0.7)]:
+            want = oracle.random_sample(codes, rv, topp, topk, temp, "bf16")
+            got = gpu_sample(ctx, codes, rv, topp, topk, temp, dt="bf16")
+            if not same_choice(codes, got, want, "bf16"):
+                bad.append((voc, (rv, topp, topk, temp), got, want))
+    assert not bad, bad
