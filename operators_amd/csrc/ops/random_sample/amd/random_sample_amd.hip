@@ -92,6 +92,55 @@ __device__ __forceinline__ int load_codes(const uint16_t *p, uint32_t voc, uint3
     return n;
 }
 
+// A pass of `lanes` lanes over the logits [begin, end) (begin a multiple of
+// 8): lane `me` takes the 8-logit vectors me, me + lanes, ... of the range and
+// calls body(base, codes, n) for each (n < 8 only for the vector that holds
+// the end).  With a 16-byte aligned array the loads of U vectors are issued
+// together before the first is used: a workgroup that walks a few hundred KB
+// alone is bound by the latency of each round of loads, not by bandwidth
+// (151 936 logits, 1024 lanes: 19 rounds of one load against 3 rounds of 8).
+template<bool VEC, int U, typename F>
+__device__ __forceinline__ void sweep_logits(const uint16_t *probs, uint32_t begin, uint32_t end, uint32_t me, uint32_t lanes, F &&body) {
+    if constexpr (VEC) {
+        const uint32_t full = begin + (end - begin) / 8u * 8u;// end of the whole vectors
+        if (full > begin) {
+            const uint32_t last = full - 8u;
+            for (uint32_t base0 = begin + me * 8u; base0 < full; base0 += lanes * 8u * U) {
+                u32x4 v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t b = base0 + static_cast<uint32_t>(u) * lanes * 8u;
+                    v[u] = ld16(probs + (b < full ? b : last));// a vector past the range re-reads the last one and is dropped below
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t b = base0 + static_cast<uint32_t>(u) * lanes * 8u;
+                    if (b < full) {
+                        const uint32_t h[8] = {v[u].x & 0xFFFFu, v[u].x >> 16, v[u].y & 0xFFFFu, v[u].y >> 16,
+                                               v[u].z & 0xFFFFu, v[u].z >> 16, v[u].w & 0xFFFFu, v[u].w >> 16};
+                        body(b, h, 8);
+                    }
+                }
+            }
+        }
+        if (full < end && me == ((full - begin) / 8u) % lanes) {// the partial vector, by the lane whose turn it is
+            uint32_t h[8];
+            const int n = static_cast<int>(end - full);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[e] = e < n ? probs[full + e] : 0u;
+            body(full, h, n);
+        }
+    } else {
+        for (uint32_t base = begin + me * 8u; base < end; base += lanes * 8u) {
+            uint32_t h[8];
+            const int n = end - base < 8u ? static_cast<int>(end - base) : 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[e] = e < n ? probs[base + e] : 0u;
+            body(base, h, n);
+        }
+    }
+}
+
 // Sum over the 64 lanes with DPP adds (the lane pattern of amd::wave_sum):
 // four steps inside each row of 16 lanes, then row broadcasts 15 and 31; the
 // total lands in lane 63 and is read back to every lane through an SGPR.
@@ -472,6 +521,7 @@ struct WideShared {
     float run;
     uint32_t n;
     uint32_t exact;// the running sum is still a whole number of units of 2^-24, at most 1.0
+    int64_t range_top;// the key range hist and p_of describe now, by its top key; -1: none
 };
 
 // One walk over the sorted sequence.  MODE 0: stop at the first entry whose
@@ -494,29 +544,31 @@ __device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs,
     __syncthreads();
     for (int64_t hi = key_max; hi >= 0; hi -= kWideBins) {
         if (sh.done != 0) break;// uniform: written before the last barrier
-        for (int b = tid; b < kWideBins; b += BS) sh.hist[b] = 0;
-        __syncthreads();
-        for (uint32_t base = tid * 8u; base < voc; base += BS * 8u) {
-            uint32_t h[8];
-            const int n = load_codes<VEC>(probs, voc, base, h);
+        if (sh.range_top != hi) {// uniform; the second walk finds the first walk's last range still there
+            __syncthreads();// everyone has read range_top
+            for (int b = tid; b < kWideBins; b += BS) sh.hist[b] = 0;
+            if (tid == 0) sh.range_top = hi;
+            __syncthreads();
+            sweep_logits<VEC, 8>(probs, 0, voc, tid, BS, [&](uint32_t, const uint32_t(&h)[8], int n) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                if (e < n) {
-                    const uint32_t below = static_cast<uint32_t>(hi) - key_of<T>(h[e]);// wraps for keys above the range
-                    if (below < static_cast<uint32_t>(kWideBins)) atomicAdd(&sh.hist[below], 1u);
+                for (int e = 0; e < 8; ++e) {
+                    if (e < n) {
+                        const uint32_t below = static_cast<uint32_t>(hi) - key_of<T>(h[e]);// wraps for keys above the range
+                        if (below < static_cast<uint32_t>(kWideBins)) atomicAdd(&sh.hist[below], 1u);
+                    }
                 }
+            });
+            __syncthreads();
+            for (int b = tid; b < kWideBins; b += BS) {
+                float p = 0.0f;
+                if (sh.hist[b] != 0 && static_cast<int64_t>(b) <= hi) {
+                    const float x = value_of_key<T>(static_cast<uint32_t>(hi - b));
+                    p = T::one(T::narrow1(expf((x - top) / temperature) / total));
+                }
+                sh.p_of[b] = p;
             }
+            __syncthreads();
         }
-        __syncthreads();
-        for (int b = tid; b < kWideBins; b += BS) {
-            float p = 0.0f;
-            if (sh.hist[b] != 0 && static_cast<int64_t>(b) <= hi) {
-                const float x = value_of_key<T>(static_cast<uint32_t>(hi - b));
-                p = T::one(T::narrow1(expf((x - top) / temperature) / total));
-            }
-            sh.p_of[b] = p;
-        }
-        __syncthreads();
         if (tid < kWave) {
             float run = sh.run;
             uint32_t n = sh.n;
@@ -637,13 +689,11 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
                                                           float random_val, float topp, uint32_t topk, float temperature) {
     __shared__ WideShared sh;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t step = BS * 8u;
+    if (tid == 0) sh.range_top = -1;
 
     // the largest key, then the denominator in the accumulation order of the other one-workgroup form
     uint32_t key_max = 0;
-    for (uint32_t base = tid * 8u; base < voc; base += step) {
-        uint32_t h[8];
-        const int n = load_codes<VEC>(probs, voc, base, h);
+    sweep_logits<VEC, 8>(probs, 0, voc, tid, BS, [&](uint32_t, const uint32_t(&h)[8], int n) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             if (e < n) {
@@ -651,7 +701,7 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
                 key_max = k > key_max ? k : key_max;
             }
         }
-    }
+    });
     key_max = wave_max_u32(key_max);
     if (lane == 0) sh.wave_key[wave] = key_max;
     __syncthreads();
@@ -659,14 +709,12 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
     for (int w = 0; w < WAVES; ++w) key_max = sh.wave_key[w] > key_max ? sh.wave_key[w] : key_max;
     const float top = value_of_key<T>(key_max);
     float part = 0.0f;
-    for (uint32_t base = tid * 8u; base < voc; base += step) {
-        uint32_t h[8];
-        const int n = load_codes<VEC>(probs, voc, base, h);
+    sweep_logits<VEC, 8>(probs, 0, voc, tid, BS, [&](uint32_t, const uint32_t(&h)[8], int n) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             if (e < n) part += expf((T::one(static_cast<uint16_t>(h[e])) - top) / temperature);
         }
-    }
+    });
     part = wave_sum(part);
     if (lane == 0) sh.sum_slots[wave] = part;
     __syncthreads();
@@ -685,38 +733,50 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
     if (sh.found == 0) return;// nothing exceeds it (random_val >= 1): the result stays as it is, as in the reference
     const uint32_t key = sh.key, occurrence = sh.occurrence;
 
-    // occurrence `occurrence` of `key` in index order
-    const uint32_t share = ((voc + BS - 1) / BS + 7u) & ~7u;// logits per lane, a multiple of 8
-    const uint32_t first = static_cast<uint32_t>(tid) * share;
-    const uint32_t last = first + share < voc ? first + share : voc;
+    // Occurrence `occurrence` of `key` in index order.  Every wavefront takes one contiguous sixteenth of the
+    // logits, 64 neighbouring vectors at a time, and counts the key in it; the wavefront whose part holds the
+    // occurrence goes through its part once more, in order, and the lane that holds it writes the index.
+    const uint32_t part_len = ((voc + WAVES - 1) / WAVES + 7u) & ~7u;// logits per wavefront, a multiple of 8
+    const uint32_t first = static_cast<uint32_t>(wave) * part_len < voc ? static_cast<uint32_t>(wave) * part_len : voc;
+    const uint32_t last = first + part_len < voc ? first + part_len : voc;
     uint32_t mine = 0;
-    for (uint32_t base = first; base < last; base += 8) {
-        uint32_t h[8];
-        const int n = load_codes<VEC>(probs, voc, base, h);
+    sweep_logits<VEC, 8>(probs, first, last, lane, kWave, [&](uint32_t, const uint32_t(&h)[8], int n) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) mine += (e < n && base + e < last && key_of<T>(h[e]) == key) ? 1u : 0u;
-    }
-    const uint32_t upto = wave_scan_u32(mine);
-    if (lane == kWave - 1) sh.wave_tot[wave] = upto;
+        for (int e = 0; e < 8; ++e) mine += (e < n && key_of<T>(h[e]) == key) ? 1u : 0u;
+    });
+    mine = wave_sum_u32(mine);
+    if (lane == 0) sh.wave_tot[wave] = mine;
     __syncthreads();
-    uint32_t before = upto - mine;
+    uint32_t before = 0;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) before += w < wave ? sh.wave_tot[w] : 0u;
-    if (occurrence >= before && occurrence < before + mine) {
-        uint32_t seen = before;
-        for (uint32_t base = first; base < last; base += 8) {
-            uint32_t h[8];
-            const int n = load_codes<VEC>(probs, voc, base, h);
-            for (int e = 0; e < 8; ++e) {
-                if (e < n && base + e < last && key_of<T>(h[e]) == key) {
-                    if (seen == occurrence) {
-                        result[0] = base + e;
-                        return;
+    if (occurrence < before || occurrence >= before + mine) return;// uniform over the wavefront
+    uint32_t seen = before;
+    for (uint32_t base0 = first; base0 < last; base0 += kWave * 8u) {// 64 neighbouring vectors, in index order
+        const uint32_t base = base0 + static_cast<uint32_t>(lane) * 8u;
+        uint32_t h[8];
+        const int n = base < last ? load_codes<VEC>(probs, last, base, h) : 0;
+        uint32_t hits = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hits += (e < n && key_of<T>(h[e]) == key) ? 1u : 0u;
+        const uint32_t upto = wave_scan_u32(hits);
+        const uint32_t here = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(upto), kWave - 1));
+        if (occurrence < seen + here) {
+            uint32_t at = seen + upto - hits;// matches before this lane's vector
+            if (occurrence >= at && occurrence < at + hits) {
+                for (int e = 0; e < 8; ++e) {
+                    if (e < n && key_of<T>(h[e]) == key) {
+                        if (at == occurrence) {
+                            result[0] = base + e;
+                            return;
+                        }
+                        ++at;
                     }
-                    ++seen;
                 }
             }
+            return;
         }
+        seen += here;
     }
 }
 
