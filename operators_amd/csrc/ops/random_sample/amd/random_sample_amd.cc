@@ -52,15 +52,28 @@ infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampl
 
 // The reference's back ends sort in a workspace of voc * 12 (CPU) or voc * 20
 // bytes plus what their sorting library allocates per call (CUDA).  Here the
-// workspace only carries the candidates from the first launch of the
-// two-launch form to the second: one header and 512 candidates of 8 bytes per
-// workgroup, under 200 KiB whatever the vocabulary; small vocabularies need
-// none.  A call that comes without it is served by one workgroup.
-uint64_t amdRandomSampleWorkspaceBytes(const RandomSampleAmdDescriptor &d) {
+// workspace carries what a first launch spread over the chip leaves for the
+// workgroup that draws: for up to 256 candidates one header and 512 candidates
+// of 8 bytes per workgroup (under 200 KiB whatever the vocabulary); for more,
+// the headers and a count for every 16-bit key (257 KiB).  Small vocabularies
+// need none.  A call that comes without it is served by one workgroup.
+uint64_t amdRandomSampleListBytes(const RandomSampleAmdDescriptor &d) {
     if (d.groups == 0) {
         return 0;
     }
     return kRandomSampleMaxGroups * sizeof(RandomSamplePart) + static_cast<uint64_t>(d.groups) * kRandomSamplePartCap * sizeof(uint64_t);
+}
+
+uint64_t amdRandomSampleHistogramBytes(const RandomSampleAmdDescriptor &d) {
+    if (d.groups == 0) {
+        return 0;
+    }
+    return kRandomSampleMaxGroups * sizeof(RandomSamplePart) + static_cast<uint64_t>(kRandomSampleKeys) * sizeof(uint32_t);
+}
+
+uint64_t amdRandomSampleWorkspaceBytes(const RandomSampleAmdDescriptor &d) {
+    const uint64_t lists = amdRandomSampleListBytes(d), histogram = amdRandomSampleHistogramBytes(d);
+    return lists > histogram ? lists : histogram;
 }
 
 infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t desc, uint64_t *size) {

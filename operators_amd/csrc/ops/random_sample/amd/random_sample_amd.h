@@ -20,6 +20,8 @@ constexpr int kRandomSampleMaxGroups = 48;
 constexpr int kRandomSamplePartTopk = 256;
 // vocabularies below this are sampled by one workgroup in one launch
 constexpr uint32_t kRandomSampleSplitVoc = 4096;
+// keys of the histogram form: every 16-bit code has one
+constexpr uint32_t kRandomSampleKeys = 1u << 16;
 // largest vocabulary the entry point without workspace and allocation serves
 constexpr uint32_t kRandomSampleNoAllocMaxVoc = 1u << 20;
 
@@ -43,6 +45,10 @@ typedef RandomSampleAmdDescriptor *RandomSampleAmdDescriptor_t;
 
 infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampleAmdDescriptor_t *desc_ptr,
                                                  infiniopTensorDescriptor_t result, infiniopTensorDescriptor_t probs);
+// bytes of workspace the two forms that use one need: candidate lists (topk <= 256), a histogram of all 16-bit
+// keys (more candidates); the descriptor asks for the larger
+uint64_t amdRandomSampleListBytes(const RandomSampleAmdDescriptor &desc);
+uint64_t amdRandomSampleHistogramBytes(const RandomSampleAmdDescriptor &desc);
 uint64_t amdRandomSampleWorkspaceBytes(const RandomSampleAmdDescriptor &desc);
 infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t desc, uint64_t *size);
 infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspace, uint64_t workspace_size,

@@ -516,6 +516,8 @@ struct WideShared {
     uint32_t wave_key[WAVES];
     float sum_slots[WAVES];
     uint32_t wave_tot[WAVES];
+    uint32_t part_key[kRandomSampleMaxGroups];// per part of the logits: its largest key and its
+    float part_sum[kRandomSampleMaxGroups];   // sum of expf((x - its largest) / temperature)
     // state of a walk, written by the first wavefront
     uint32_t done, found, entry, key, occurrence;
     float run;
@@ -530,8 +532,8 @@ struct WideShared {
 // exceeds `threshold` (found = 1, key/occurrence name it), or after `limit_n`.
 // Leaves the running sum in sh.run.  All lanes call it.
 template<typename T, bool VEC, int MODE>
-__device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs, uint32_t voc, uint32_t key_max, float top,
-                                          float total, float temperature, float threshold, uint32_t limit_n) {
+__device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs, uint32_t voc, const uint32_t *counts, uint32_t key_max,
+                                          float top, float total, float temperature, float threshold, uint32_t limit_n) {
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     if (tid == 0) {
         sh.done = limit_n == 0 ? 1u : 0u;
@@ -546,18 +548,22 @@ __device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs,
         if (sh.done != 0) break;// uniform: written before the last barrier
         if (sh.range_top != hi) {// uniform; the second walk finds the first walk's last range still there
             __syncthreads();// everyone has read range_top
-            for (int b = tid; b < kWideBins; b += BS) sh.hist[b] = 0;
             if (tid == 0) sh.range_top = hi;
-            __syncthreads();
-            sweep_logits<VEC, 8>(probs, 0, voc, tid, BS, [&](uint32_t, const uint32_t(&h)[8], int n) {
+            if (counts != nullptr) {// counted by an earlier launch: key k's count is counts[k]
+                for (int b = tid; b < kWideBins; b += BS) sh.hist[b] = static_cast<int64_t>(b) <= hi ? counts[hi - b] : 0u;
+            } else {
+                for (int b = tid; b < kWideBins; b += BS) sh.hist[b] = 0;
+                __syncthreads();
+                sweep_logits<VEC, 8>(probs, 0, voc, tid, BS, [&](uint32_t, const uint32_t(&h)[8], int n) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    if (e < n) {
-                        const uint32_t below = static_cast<uint32_t>(hi) - key_of<T>(h[e]);// wraps for keys above the range
-                        if (below < static_cast<uint32_t>(kWideBins)) atomicAdd(&sh.hist[below], 1u);
+                    for (int e = 0; e < 8; ++e) {
+                        if (e < n) {
+                            const uint32_t below = static_cast<uint32_t>(hi) - key_of<T>(h[e]);// wraps for keys above the range
+                            if (below < static_cast<uint32_t>(kWideBins)) atomicAdd(&sh.hist[below], 1u);
+                        }
                     }
-                }
-            });
+                });
+            }
             __syncthreads();
             for (int b = tid; b < kWideBins; b += BS) {
                 float p = 0.0f;
@@ -684,52 +690,144 @@ __device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs,
     }
 }
 
+// The softmax denominator is formed part by part: the logits are cut into
+// `groups` parts of 2048 * vecs, each part's sum is taken relative to the
+// part's own largest logit by 256 lanes (sequentially per lane, then the
+// wavefront tree, then the four wavefronts in order), and the parts are
+// rescaled to the overall maximum and added in a fixed order.  The split form
+// gives every part to a workgroup of its own in an earlier launch; one
+// workgroup alone takes four parts at a time, 256 lanes each - the same
+// arithmetic in the same order, so both forms get the same denominator, to
+// the bit, and with it the same probabilities and the same draw.
 template<typename T, bool VEC>
+__device__ __forceinline__ void part_max_and_sum(const uint16_t *probs, uint32_t voc, uint32_t start, uint32_t vecs, float temperature,
+                                                 bool active, uint32_t t, uint32_t *key_slots, float *sum_slots, uint32_t *counts,
+                                                 uint32_t &key_max, float &sum) {
+    constexpr uint32_t PL = kRandomSamplePartLanes;
+    const uint32_t lane = t & (kWave - 1), w = t / kWave;
+    uint32_t km = 0;
+    if (active) {
+        for (uint32_t v = 0; v < vecs; ++v) {
+            const uint32_t base = start + (v * PL + t) * 8u;
+            if (base < voc) {
+                uint32_t h[8];
+                const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (e < n) {
+                        const uint32_t k = key_of<T>(h[e]);
+                        km = k > km ? k : km;
+                        if (counts != nullptr) atomicAdd(&counts[k], 1u);
+                    }
+                }
+            }
+        }
+        km = wave_max_u32(km);
+        if (lane == 0) key_slots[w] = km;
+    }
+    __syncthreads();
+    float part = 0.0f;
+    if (active) {
+#pragma unroll
+        for (uint32_t i = 0; i < PL / kWave; ++i) km = key_slots[i] > km ? key_slots[i] : km;
+        const float top = value_of_key<T>(km);
+        for (uint32_t v = 0; v < vecs; ++v) {
+            const uint32_t base = start + (v * PL + t) * 8u;
+            if (base < voc) {
+                uint32_t h[8];
+                const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (e < n) part += expf((T::one(static_cast<uint16_t>(h[e])) - top) / temperature);
+                }
+            }
+        }
+        part = wave_sum(part);
+        if (lane == 0) sum_slots[w] = part;
+    }
+    __syncthreads();
+    key_max = km;
+    sum = 0.0f;
+    if (active) {
+#pragma unroll
+        for (uint32_t i = 0; i < PL / kWave; ++i) sum += sum_slots[i];
+    }
+}
+
+// First launches of the split form: clear the counts, then one workgroup per
+// part of the logits counts every key and leaves its part's maximum and sum.
+__global__ __launch_bounds__(256) void random_sample_clear(u32x4 *counts) {
+    counts[blockIdx.x * 256u + threadIdx.x] = u32x4{0, 0, 0, 0};
+}
+
+template<typename T, bool VEC>
+__global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_count(RandomSamplePart *heads, uint32_t *counts, const uint16_t *probs,
+                                                                                uint32_t voc, uint32_t vecs, float temperature) {
+    __shared__ uint32_t key_slots[kRandomSamplePartLanes / kWave];
+    __shared__ float sum_slots[kRandomSamplePartLanes / kWave];
+    uint32_t key_max;
+    float sum;
+    part_max_and_sum<T, VEC>(probs, voc, blockIdx.x * (kRandomSamplePartLanes * 8u * vecs), vecs, temperature, true, threadIdx.x,
+                             key_slots, sum_slots, counts, key_max, sum);
+    if (threadIdx.x == 0) heads[blockIdx.x] = RandomSamplePart{0, key_max, sum, 0};
+}
+
+// SPLIT: the parts' maxima and sums come from `heads` and the counts of all
+// keys from `counts`, both left by the launches above; otherwise this
+// workgroup works them out itself (counts: a range of keys at a time, in LDS).
+template<typename T, bool VEC, bool SPLIT>
 __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const uint16_t *probs, uint32_t voc,
-                                                          float random_val, float topp, uint32_t topk, float temperature) {
+                                                          float random_val, float topp, uint32_t topk, float temperature,
+                                                          const RandomSamplePart *heads, const uint32_t *counts, uint32_t groups, uint32_t vecs) {
     __shared__ WideShared sh;
+    __shared__ uint32_t key_slots[BS / kWave];
+    __shared__ float sum_slots4[BS / kWave];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     if (tid == 0) sh.range_top = -1;
 
-    // the largest key, then the denominator in the accumulation order of the other one-workgroup form
-    uint32_t key_max = 0;
-    sweep_logits<VEC, 8>(probs, 0, voc, tid, BS, [&](uint32_t, const uint32_t(&h)[8], int n) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if (e < n) {
-                const uint32_t k = key_of<T>(h[e]);
-                key_max = k > key_max ? k : key_max;
+    if constexpr (SPLIT) {
+        if (static_cast<uint32_t>(tid) < groups) {
+            sh.part_key[tid] = heads[tid].key_max;
+            sh.part_sum[tid] = heads[tid].sum;
+        }
+    } else {
+        constexpr uint32_t PL = kRandomSamplePartLanes, SIDE = BS / PL;// parts taken side by side
+        const uint32_t side = tid / PL, t = tid % PL;
+        for (uint32_t g0 = 0; g0 < groups; g0 += SIDE) {
+            const uint32_t g = g0 + side;
+            uint32_t key_max;
+            float sum;
+            part_max_and_sum<T, VEC>(probs, voc, g * (PL * 8u * vecs), vecs, temperature, g < groups, t,
+                                     key_slots + side * (PL / kWave), sum_slots4 + side * (PL / kWave), nullptr, key_max, sum);
+            if (g < groups && t == 0) {
+                sh.part_key[g] = key_max;
+                sh.part_sum[g] = sum;
             }
         }
-    });
-    key_max = wave_max_u32(key_max);
-    if (lane == 0) sh.wave_key[wave] = key_max;
+    }
     __syncthreads();
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) key_max = sh.wave_key[w] > key_max ? sh.wave_key[w] : key_max;
+    // the overall maximum and the denominator rescaled to it, in a fixed order (groups <= 48: one wavefront's work)
+    uint32_t key_max = 0;
+    for (uint32_t g = 0; g < groups; ++g) key_max = sh.part_key[g] > key_max ? sh.part_key[g] : key_max;
     const float top = value_of_key<T>(key_max);
-    float part = 0.0f;
-    sweep_logits<VEC, 8>(probs, 0, voc, tid, BS, [&](uint32_t, const uint32_t(&h)[8], int n) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if (e < n) part += expf((T::one(static_cast<uint16_t>(h[e])) - top) / temperature);
-        }
-    });
-    part = wave_sum(part);
-    if (lane == 0) sh.sum_slots[wave] = part;
+    if (tid < kWave) {
+        float part = 0.0f;
+        if (static_cast<uint32_t>(tid) < groups) part = sh.part_sum[tid] * expf((value_of_key<T>(sh.part_key[tid]) - top) / temperature);
+        part = wave_sum(part);
+        if (tid == 0) sh.sum_slots[0] = part;
+    }
     __syncthreads();
-    float total = 0.0f;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) total += sh.sum_slots[w];
+    const float total = sh.sum_slots[0];
+    const uint32_t *const from = SPLIT ? counts : nullptr;
 
     // walk 1 (random_sample.cc:97-109): where the running sum reaches topp
-    wide_walk<T, VEC, 0>(sh, probs, voc, key_max, top, total, temperature, topp, topk);
+    wide_walk<T, VEC, 0>(sh, probs, voc, from, key_max, top, total, temperature, topp, topk);
     const uint32_t stop = sh.found != 0 ? sh.entry : topk;// rank of the entry that reached topp
     const float kept = sh.run;                             // the sum up to and including it, or over all topk entries
     const uint32_t end = stop + 1 < topk ? stop + 1 : topk;
     __syncthreads();
     // walk 2 (random_sample.cc:112-125): the first of those `end` entries whose running sum exceeds random_val * kept
-    wide_walk<T, VEC, 1>(sh, probs, voc, key_max, top, total, temperature, random_val * kept, end);
+    wide_walk<T, VEC, 1>(sh, probs, voc, from, key_max, top, total, temperature, random_val * kept, end);
     if (sh.found == 0) return;// nothing exceeds it (random_val >= 1): the result stays as it is, as in the reference
     const uint32_t key = sh.key, occurrence = sh.occurrence;
 
@@ -1058,21 +1156,34 @@ struct RandomSampleCall {
     float random_val, topp;
     uint32_t topk;
     float temperature;
-    RandomSamplePart *heads;// the workspace, when the two-launch form is to be used
+    void *workspace;// what a first launch leaves for the drawing workgroup goes here; null: one workgroup does the whole call
     uint32_t groups, vecs;
 };
 
-// form 2: sampling, 1: greedy, 0: nothing to launch
+// form 2: sampling, 1: greedy, 0: nothing to launch.  Sampling with up to
+// kRandomSamplePartTopk candidates ranks them in LDS (candidate lists through
+// the workspace, or one workgroup alone); with more it walks the histogram of
+// keys (counts through the workspace, or one workgroup alone).
 template<typename T, bool VEC>
 void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
+    auto *heads = static_cast<RandomSamplePart *>(c.workspace);
     if (form == 1) {
         random_sample_greedy<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc);
-    } else if (form == 2 && c.heads != nullptr) {
-        auto *lists = reinterpret_cast<unsigned long long *>(c.heads + kRandomSampleMaxGroups);
-        random_sample_partial<T, VEC><<<c.groups, kRandomSamplePartLanes, 0, s>>>(c.heads, lists, c.probs, c.voc, c.vecs, c.topk, c.temperature);
-        random_sample_merge<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature, c.heads, lists, c.groups);
-    } else if (form == 2 && c.topk > static_cast<uint32_t>(KMAX)) {
-        random_sample_wide<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature);
+    } else if (form == 2 && c.topk > static_cast<uint32_t>(kRandomSamplePartTopk)) {
+        if (heads != nullptr) {
+            auto *counts = reinterpret_cast<uint32_t *>(heads + kRandomSampleMaxGroups);
+            random_sample_clear<<<kRandomSampleKeys / (256 * 4), 256, 0, s>>>(reinterpret_cast<u32x4 *>(counts));
+            random_sample_count<T, VEC><<<c.groups, kRandomSamplePartLanes, 0, s>>>(heads, counts, c.probs, c.voc, c.vecs, c.temperature);
+            random_sample_wide<T, VEC, true><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature,
+                                                              heads, counts, c.groups, c.vecs);
+        } else {
+            random_sample_wide<T, VEC, false><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature,
+                                                               nullptr, nullptr, c.groups, c.vecs);
+        }
+    } else if (form == 2 && heads != nullptr) {
+        auto *lists = reinterpret_cast<unsigned long long *>(heads + kRandomSampleMaxGroups);
+        random_sample_partial<T, VEC><<<c.groups, kRandomSamplePartLanes, 0, s>>>(heads, lists, c.probs, c.voc, c.vecs, c.topk, c.temperature);
+        random_sample_merge<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature, heads, lists, c.groups);
     } else if (form == 2) {
         random_sample_topk<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature);
     }
@@ -1084,8 +1195,10 @@ void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
 // the process ends.  Host code never uses the array's name as an address (on
 // the host it is only a handle for the symbol): the address on a GPU is asked
 // for once, with that GPU current, and kept.
-constexpr uint64_t kScratchBytes = kRandomSampleMaxGroups * sizeof(RandomSamplePart) +
-                                   static_cast<uint64_t>(kRandomSampleMaxGroups) * kRandomSamplePartCap * sizeof(uint64_t);
+constexpr uint64_t kScratchListBytes = kRandomSampleMaxGroups * sizeof(RandomSamplePart) +
+                                       static_cast<uint64_t>(kRandomSampleMaxGroups) * kRandomSamplePartCap * sizeof(uint64_t);
+constexpr uint64_t kScratchCountBytes = kRandomSampleMaxGroups * sizeof(RandomSamplePart) + static_cast<uint64_t>(kRandomSampleKeys) * sizeof(uint32_t);
+constexpr uint64_t kScratchBytes = kScratchListBytes > kScratchCountBytes ? kScratchListBytes : kScratchCountBytes;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 constexpr int kMaxGpus = 64;
@@ -1159,11 +1272,16 @@ infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspa
     }
     AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool split = sample && k >= 2 && desc->groups != 0 && k <= static_cast<uint32_t>(kRandomSamplePartTopk) &&
-                       workspace != nullptr && workspace_size >= amdRandomSampleWorkspaceBytes(*desc) &&
-                       (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0;
+    // what the form this call takes needs of the workspace (16-byte aligned: the counts are cleared 16 bytes at a time)
+    const uint64_t needs = k <= static_cast<uint32_t>(kRandomSamplePartTopk) ? amdRandomSampleListBytes(*desc) : amdRandomSampleHistogramBytes(*desc);
+    const bool split = sample && k >= 2 && desc->groups != 0 && workspace != nullptr && workspace_size >= needs &&
+                       (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0;
+    // the parts the denominator is formed in: the first launch's workgroups, or as many of one vector per lane for
+    // vocabularies too small to be split
+    const uint32_t groups = desc->groups != 0 ? desc->groups : static_cast<uint32_t>(amd::ceil_div(desc->voc, kRandomSamplePartLanes * 8u));
+    const uint32_t vecs = desc->groups != 0 ? desc->vecs : 1u;
     const RandomSampleCall call{static_cast<uint64_t *>(result), static_cast<const uint16_t *>(probs), desc->voc, random_val, topp, k,
-                                temperature, split ? static_cast<RandomSamplePart *>(workspace) : nullptr, desc->groups, desc->vecs};
+                                temperature, split ? workspace : nullptr, groups, vecs};
     // greedy unless sampling; a vocabulary of one logit has one candidate of
     // probability 1, which wins unless random_val >= 1, as in the reference's loops
     const int form = (sample && k >= 2) ? 2 : (!sample || random_val < 1.0f) ? 1 : 0;
