@@ -358,11 +358,10 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopDestroyAttentionDescriptor(i
  * Otherwise: the first index of the maximum.  probs: 1-D F16 (reference) or
  * BF16 (extension: probabilities round to nearest even), unit stride;
  * result: U64, one element written.  Equal logits are ordered by ascending
- * index.  topk (after clamping to the vocabulary size) may be at most 1024 in
- * the sampling form, else STATUS_BAD_PARAM.  The workspace (under 200 KiB, 0
- * below 4096 logits) lets the sampling form spread its pass over the logits
- * over the chip; a call without it is served by one workgroup, with the same
- * result.
+ * index.  Any topk is served (it is clamped to the vocabulary size, as in the
+ * reference).  The workspace (262 912 bytes, 0 below 4096 logits) lets the
+ * sampling form spread its passes over the logits over the chip; a call
+ * without it, or with less, is served by one workgroup, with the same result.
  * ======================================================================== */
 typedef struct RandomSampleDescriptor {
     Device device;
@@ -381,8 +380,9 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopRandomSample(
     void *result, void const *probs, float random_val, float topp, int topk, float temperature, void *stream);
 /* no counterpart in the reference.  For callers that cannot allocate device
  * memory or hand over a workspace (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc): infiniopRandomSample with the
- * candidate lists of its two-launch form kept in an array of 197 376 bytes
+ * loops, harnesses that forbid hipMalloc): infiniopRandomSample with what its
+ * first launches leave for the drawing workgroup (candidate lists, or a count
+ * per 16-bit key) kept in an array of 262 912 bytes
  * that the library holds on every GPU it runs on until the process ends.  The
  * call allocates nothing.  Same results as infiniopRandomSample with a
  * workspace.  Descriptors of more than 1 048 576 logits answer

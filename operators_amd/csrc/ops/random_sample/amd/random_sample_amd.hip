@@ -16,14 +16,18 @@
 //  * the first wavefront forms the sequential running sums once, as a
 //    branch-free chain with the addends in registers, and takes the top-p and
 //    random_val decisions with ballots over them.
-// Two forms.  One workgroup of 1024 lanes does all of it from the logits in
-// one launch (topk_full; 32 000 logits take it several times as long as the
-// two-launch form: one compute unit's instruction rate is the limit).  With the workspace the descriptor asks for,
-// topk <= 256 and 4096 logits or more, a first launch spreads the pass over the
-// logits over up to 48 workgroups, each of which drops everything that cannot
-// be in the overall topk, and a second launch of one workgroup finishes from
-// the few hundred survivors (6.9 + 10.3 us for 32 000 logits, 9.7 + 14.0 us
-// for 151 936).
+// That is the form for up to 256 candidates (topk after clamping).  One
+// workgroup of 1024 lanes does all of it from the logits in one launch
+// (topk_full; 32 000 logits take it several times as long as the two-launch
+// form: one compute unit's instruction rate is the limit).  With the workspace
+// the descriptor asks for and 4096 logits or more, a first launch spreads the
+// pass over the logits over up to 48 workgroups, each of which drops
+// everything that cannot be in the overall topk, and a second launch of one
+// workgroup finishes from the few hundred survivors (6.9 + 10.3 us for 32 000
+// logits, 9.7 + 14.0 us for 151 936).
+// More candidates than that - any number, the reference has no limit - are
+// not ranked at all: the running sums are formed over a histogram of the keys
+// (further down).
 //
 // Two things differ from the CPU path and are visible to a caller:
 //  * equal logits: the CPU's selection sort leaves equal values in an order
@@ -454,25 +458,39 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
 
 // ---- more candidates than LDS ranks: sampling without a sorted list -----------
 // The reference keeps any topk up to the vocabulary size (random_sample.cc:
-// 67-74 only clamps it).  Beyond KMAX candidates nothing is compacted or
+// 67-74 only clamps it).  Beyond 256 candidates nothing is compacted or
 // ranked.  Equal logits have equal probabilities, so the sorted sequence the
 // reference walks is fully described by how often every 16-bit code occurs: a
 // histogram over the ordered keys, walked from the largest key down, adding
-// each key's probability as many times as the key occurs - the same sequential
-// fp32 additions, the same comparisons.  One workgroup:
-//   1. the largest key and the softmax denominator (two passes over the logits);
+// each key's probability as many times as the key occurs - the same fp32
+// running sums, the same comparisons:
+//   1. the largest key and the softmax denominator, part by part (see
+//      part_max_and_sum);
 //   2. walk 1 finds where the running sum reaches topp (or the topk-th entry)
 //      and with it the sum of the kept prefix; walk 2 finds the entry whose
 //      running sum exceeds random_val times that sum.  A walk takes the key
-//      space in ranges of kWideBins keys from the top: count the logits of the
-//      range into an LDS histogram, compute every occupied key's probability
-//      in parallel, then the first wavefront adds them up in order.  Walks
-//      stop as soon as their question is answered - for ordinary top-p values
-//      within the first range;
-//   3. the answer is "occurrence r of key K": every lane counts K in its
-//      contiguous share of the logits, a prefix sum finds the share holding
-//      occurrence r, and that lane looks it up.  Equal logits are thereby
-//      ordered by ascending index, as in the other forms.
+//      space in ranges of kWideBins keys from the top: the counts of the
+//      range's keys into LDS, every occupied key's probability in parallel,
+//      then the first wavefront goes through them in order.  Walks stop as
+//      soon as their question is answered - for ordinary top-p values within
+//      the first range - and the second walk starts on the range the first
+//      one left in LDS;
+//   3. the answer is "occurrence r of key K": every wavefront counts K in its
+//      contiguous sixteenth of the logits, and the wavefront whose part holds
+//      occurrence r goes through it once more in order.  Equal logits are
+//      thereby ordered by ascending index, as in the other form.
+// With the workspace, two launches before the one workgroup that draws take
+// what can be spread over the chip: the counts of all 65 536 keys (cleared,
+// then one atomic add per logit) and every part's maximum and sum; the walks
+// then read a range's counts instead of passing over the logits, and once a
+// walk has left the first range it steps over whole ranges in which nothing
+// can happen (wide_range_totals) - a top-p of 1 with top-k off, plain
+// sampling from the whole distribution, costs little more than a peaked one.
+// Without the workspace the one workgroup counts a range at a time itself.
+// 151 936 fp16 logits, top-k off, MI355X, with the workspace: 54 us at top-p
+// 0.9 (4.5 clear + 19.7 count + 28.8 draw), 112 us at top-p 1; without:
+// 87 us and 0.41 ms.  (Before the measures described here and below: 223 us
+// and 5.9 ms.)
 // The additions need not be made one by one.  An fp16 probability is a whole
 // number of units of 2^-24 (the spacing of fp16 subnormals), and so is every
 // sum of them; below 1.0 an fp32 holds any such number exactly (at most 24
@@ -483,12 +501,12 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
 // key at which the comparison turns, one integer division for the entry
 // inside that key.  Only a running sum that passes 1.0 (one-hot
 // distributions; bf16 probabilities, which are finer than 2^-24, always) is
-// continued one entry at a time, as the reference adds.  151 936 logits,
-// top-k off, on MI355X: 223 -> 123 us at top-p 0.9, 760 -> 131 us at top-p
-// 0.99, 5.9 ms -> 0.47 ms for a distribution so flat that the walk covers the
-// whole vocabulary (what is left is the passes over the logits, one per
-// range of keys and walk).
+// continued one entry at a time, as the reference adds.  On its own this
+// took 151 936 logits with top-k off from 223 to 123 us at top-p 0.9, from 760
+// to 131 us at top-p 0.99 and from 5.9 ms to 0.47 ms for a distribution so
+// flat that the walk covers the whole vocabulary.
 constexpr int kWideBins = 4096;
+constexpr int kWideRanges = static_cast<int>(kRandomSampleKeys) / kWideBins;
 constexpr uint32_t kOneUnits = 1u << 24;     // 1.0 in units of 2^-24
 constexpr uint32_t kManyUnits = 1u << 25;    // stands for "more than 1.0" in a prefix sum of 64 terms
 
@@ -524,7 +542,77 @@ struct WideShared {
     uint32_t n;
     uint32_t exact;// the running sum is still a whole number of units of 2^-24, at most 1.0
     int64_t range_top;// the key range hist and p_of describe now, by its top key; -1: none
+    // per range of kWideBins keys from the top: what all its entries add to the running sum, in units (kManyUnits:
+    // more than the exact walk handles), and how many entries it has; filled on demand
+    unsigned long long range_sum[kWideRanges];
+    uint32_t range_units[kWideRanges], range_count[kWideRanges];
+    uint32_t ranges_known;
 };
+
+// What every range of keys adds to the running sum and to the entry count,
+// from the counts of all keys (split form, exact units only).  A walk that has
+// left the first range behind asks for this once and then steps over every
+// range in which nothing can happen - a top-p of 1 sends the first walk
+// through the whole vocabulary only to learn the sum - instead of fetching
+// and walking it.  Lane l takes the 64 keys from 64 * l up (they lie in at
+// most two ranges); a key's probability is formed exactly as the walk forms
+// it, except that keys so far below the top that it must truncate to zero
+// (expf(d) / total < 2^-24, the smallest fp16) are not exponentiated.
+template<typename T>
+__device__ __attribute__((noinline)) void wide_range_totals(WideShared &sh, const uint32_t *counts, uint32_t key_max, float top, float total,
+                                                          float temperature) {
+    const uint32_t tid = threadIdx.x;
+    if (tid < static_cast<uint32_t>(kWideRanges)) {
+        sh.range_sum[tid] = 0;
+        sh.range_count[tid] = 0;
+    }
+    __syncthreads();
+    const uint32_t k0 = tid * 64u;
+    if (k0 <= key_max) {
+        const float zero_below = logf(total) - 17.0f;
+        const uint32_t r_far = (key_max - k0) / kWideBins;// the range of the lowest key; the highest is in it or in the one before
+        unsigned long long sum_far = 0, sum_near = 0;
+        uint32_t cnt_far = 0, cnt_near = 0;
+#pragma unroll 1
+        for (int half = 0; half < 2; ++half) {// 32 keys' counts in flight at a time: the calling kernel has 128 registers a lane
+        u32x4 c[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c[i] = *reinterpret_cast<const u32x4 *>(counts + k0 + 32 * half + 4 * i);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t four[4] = {c[i].x, c[i].y, c[i].z, c[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t k = k0 + 32 * half + 4 * i + j, n = four[j];
+                if (n != 0 && k <= key_max) {
+                    const float d = (value_of_key<T>(k) - top) / temperature;
+                    uint32_t units = 0;
+                    if (!(d < zero_below)) {
+                        const float p = T::one(T::narrow1(expf(d) / total));
+                        units = p <= 1.0f ? static_cast<uint32_t>(p * 16777216.0f) : kManyUnits;
+                    }
+                    unsigned long long add = static_cast<unsigned long long>(n) * units;
+                    add = add > kManyUnits ? kManyUnits : add;
+                    if ((key_max - k) / kWideBins == r_far) sum_far += add, cnt_far += n;
+                    else sum_near += add, cnt_near += n;
+                }
+            }
+        }
+        }
+        if (cnt_far != 0) {
+            atomicAdd(&sh.range_sum[r_far], sum_far);
+            atomicAdd(&sh.range_count[r_far], cnt_far);
+        }
+        if (cnt_near != 0) {// r_far >= 1 here
+            atomicAdd(&sh.range_sum[r_far - 1], sum_near);
+            atomicAdd(&sh.range_count[r_far - 1], cnt_near);
+        }
+    }
+    __syncthreads();
+    if (tid < static_cast<uint32_t>(kWideRanges)) sh.range_units[tid] = sh.range_sum[tid] > kManyUnits ? kManyUnits : static_cast<uint32_t>(sh.range_sum[tid]);
+    if (tid == 0) sh.ranges_known = 1;
+    __syncthreads();
+}
 
 // One walk over the sorted sequence.  MODE 0: stop at the first entry whose
 // running sum reaches `threshold` (found = 1, entry = its rank), or after
@@ -546,6 +634,22 @@ __device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs,
     __syncthreads();
     for (int64_t hi = key_max; hi >= 0; hi -= kWideBins) {
         if (sh.done != 0) break;// uniform: written before the last barrier
+        if (ExactUnits<T>::value && counts != nullptr && hi != static_cast<int64_t>(key_max) && sh.exact != 0) {
+            // past the first range, with every key's count at hand: step over this range if nothing happens in it
+            if (sh.ranges_known == 0) wide_range_totals<T>(sh, counts, key_max, top, total, temperature);
+            const int r = static_cast<int>((static_cast<int64_t>(key_max) - hi) / kWideBins);
+            const uint32_t adds = sh.range_units[r], entries = sh.range_count[r];
+            const uint32_t units_run = static_cast<uint32_t>(sh.run * 16777216.0f), n = sh.n;
+            if (adds < kManyUnits && units_run + adds <= kOneUnits && units_run + adds < thr && n + entries < limit_n) {
+                __syncthreads();// everyone has read the state
+                if (tid == 0) {
+                    sh.run = static_cast<float>(units_run + adds) * (1.0f / 16777216.0f);
+                    sh.n = n + entries;
+                }
+                __syncthreads();
+                continue;
+            }
+        }
         if (sh.range_top != hi) {// uniform; the second walk finds the first walk's last range still there
             __syncthreads();// everyone has read range_top
             if (tid == 0) sh.range_top = hi;
@@ -783,7 +887,10 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
     __shared__ uint32_t key_slots[BS / kWave];
     __shared__ float sum_slots4[BS / kWave];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    if (tid == 0) sh.range_top = -1;
+    if (tid == 0) {
+        sh.range_top = -1;
+        sh.ranges_known = 0;
+    }
 
     if constexpr (SPLIT) {
         if (static_cast<uint32_t>(tid) < groups) {
@@ -849,32 +956,59 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) before += w < wave ? sh.wave_tot[w] : 0u;
     if (occurrence < before || occurrence >= before + mine) return;// uniform over the wavefront
+    // in index order, 64 neighbouring vectors at a time; the loads of eight such rounds are issued together
+    constexpr int U = 8;
+    const uint32_t whole = first + (last - first) / 8u * 8u;// end of this part's whole vectors
     uint32_t seen = before;
-    for (uint32_t base0 = first; base0 < last; base0 += kWave * 8u) {// 64 neighbouring vectors, in index order
-        const uint32_t base = base0 + static_cast<uint32_t>(lane) * 8u;
-        uint32_t h[8];
-        const int n = base < last ? load_codes<VEC>(probs, last, base, h) : 0;
-        uint32_t hits = 0;
+    for (uint32_t base0 = first; base0 < whole; base0 += kWave * 8u * U) {
+        u32x4 v[U];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) hits += (e < n && key_of<T>(h[e]) == key) ? 1u : 0u;
-        const uint32_t upto = wave_scan_u32(hits);
-        const uint32_t here = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(upto), kWave - 1));
-        if (occurrence < seen + here) {
-            uint32_t at = seen + upto - hits;// matches before this lane's vector
-            if (occurrence >= at && occurrence < at + hits) {
-                for (int e = 0; e < 8; ++e) {
-                    if (e < n && key_of<T>(h[e]) == key) {
-                        if (at == occurrence) {
-                            result[0] = base + e;
-                            return;
+        for (int u = 0; u < U; ++u) {
+            const uint32_t base = base0 + (static_cast<uint32_t>(u) * kWave + lane) * 8u;
+            const uint32_t at = base < whole ? base : first;// past the end: any vector of the part, dropped below
+            if constexpr (VEC) {
+                v[u] = ld16(probs + at);
+            } else {
+                v[u] = u32x4{probs[at] | (static_cast<uint32_t>(probs[at + 1]) << 16), probs[at + 2] | (static_cast<uint32_t>(probs[at + 3]) << 16),
+                             probs[at + 4] | (static_cast<uint32_t>(probs[at + 5]) << 16), probs[at + 6] | (static_cast<uint32_t>(probs[at + 7]) << 16)};
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t base = base0 + (static_cast<uint32_t>(u) * kWave + lane) * 8u;
+            const uint32_t h[8] = {v[u].x & 0xFFFFu, v[u].x >> 16, v[u].y & 0xFFFFu, v[u].y >> 16,
+                                   v[u].z & 0xFFFFu, v[u].z >> 16, v[u].w & 0xFFFFu, v[u].w >> 16};
+            uint32_t hits = 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) hits += (base < whole && key_of<T>(h[e]) == key) ? 1u : 0u;
+            const uint32_t upto = wave_scan_u32(hits);
+            const uint32_t here = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(upto), kWave - 1));
+            if (occurrence < seen + here) {// uniform: it is in this round
+                uint32_t at = seen + upto - hits;// matches before this lane's vector
+                if (occurrence >= at && occurrence < at + hits) {
+                    for (int e = 0; e < 8; ++e) {
+                        if (key_of<T>(h[e]) == key) {
+                            if (at == occurrence) result[0] = base + e;
+                            ++at;
                         }
-                        ++at;
                     }
                 }
+                return;
             }
-            return;
+            seen += here;
         }
-        seen += here;
+    }
+    // what is left is the vector that holds the end of the logits
+    if (lane == 0) {
+        for (uint32_t i = whole; i < last; ++i) {
+            if (key_of<T>(probs[i]) == key) {
+                if (seen == occurrence) {
+                    result[0] = i;
+                    return;
+                }
+                ++seen;
+            }
+        }
     }
 }
 
