@@ -1360,10 +1360,12 @@ infiniopStatus_t scratch_address(int device_id, void **address) {
 }// namespace
 
 // RandomSample without a caller-provided workspace and without any allocation:
-// the candidate lists of the two-launch form live in this library's own array
-// on the GPU.  Same results as amdRandomSample with a workspace.  Nothing in
-// the array has to be cleared between calls (the first launch writes every
-// header and every list entry the second one reads).  All calls on one GPU
+// what the first launches leave for the drawing workgroup lives in this
+// library's own array on the GPU.  Same results as amdRandomSample with a
+// workspace.  Nothing in the array has to be cleared between calls by the host
+// (the first launch writes every header and every list entry the last one
+// reads; the counts of the histogram form are cleared by a kernel of the call
+// itself).  All calls on one GPU
 // share the array: two of them in flight at once, on any streams, race.
 infiniopStatus_t amdRandomSampleNoAlloc(RandomSampleAmdDescriptor_t desc, void *result, void const *probs, float random_val,
                                         float topp, int topk, float temperature, void *stream) {
@@ -1391,9 +1393,11 @@ infiniopStatus_t amdRandomSampleNoAlloc(RandomSampleAmdDescriptor_t desc, void *
 
 // Stage 4 of RandomSample.  With topp > 0 and topk > 1 it samples, otherwise
 // it returns the first index of the maximum, as the reference does
-// (random_sample.cc:160-166).  The workspace is used by the two-launch form
-// only; without it (null, too small, misaligned), for more than 256
-// candidates and for small vocabularies one workgroup does the whole call.
+// (random_sample.cc:160-166).  The workspace carries what a first launch
+// spread over the chip leaves for the workgroup that draws: candidate lists
+// for up to 256 candidates, a count per key for more.  Without it (null, too
+// small for the form the call takes, misaligned) and for small vocabularies
+// one workgroup does the whole call, with the same result.
 infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspace, uint64_t workspace_size, void *result,
                                  void const *probs, float random_val, float topp, int topk, float temperature, void *stream) {
     if (result == nullptr || probs == nullptr) {
