@@ -176,7 +176,7 @@ def make_causal_softmax(ctx, heads, seq, total, dtype, gen, name):
     return Launch(name, ctx.lib.infiniopCausalSoftmax, (plan.desc, None, 0, y.data_ptr()), nbytes, (plan, y))
 
 
-def make_random_sample(ctx, voc, topk, gen, name, use_workspace=True):
+def make_random_sample(ctx, voc, topk, gen, name, use_workspace=True, topp=0.9, temperature=0.8):
     """One draw from `voc` fp16 logits ~ N(0, 3): top-p 0.9, top-k `topk`, temperature 0.8 (greedy when topk is 1).
     Without the workspace the library serves the call with one workgroup."""
     import torch
@@ -188,7 +188,7 @@ def make_random_sample(ctx, voc, topk, gen, name, use_workspace=True):
     plan = RandomSamplePlan(ctx, result, logits, use_workspace)
     f = ctypes.c_float
     ws = plan.workspace.data_ptr() if plan.workspace is not None else None
-    args = (plan.desc, ws, plan.workspace_size, result.data_ptr(), logits.data_ptr(), f(0.37), f(0.9 if topk > 1 else 0.0), topk, f(0.8))
+    args = (plan.desc, ws, plan.workspace_size, result.data_ptr(), logits.data_ptr(), f(0.37), f(topp if topk > 1 else 0.0), topk, f(temperature))
     launch = Launch(name, ctx.lib.infiniopRandomSample, args, voc * 2 + 8, (plan, logits, result))
     launch.latency_bound = True  # a few hundred KB at most: the time is a chain of dependent steps, not traffic
     return launch
@@ -434,7 +434,8 @@ def ops_table(ctx, args, gen):
         "S2 random_sample f16 voc 32000, greedy": lambda: [make_random_sample(ctx, 32000, 1, gen, "random_sample") for _ in range(MAX_SETS)],
         "S3 random_sample f16 voc 151936, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 50, gen, "random_sample") for _ in range(MAX_SETS)],
         "S4 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8, no workspace (one workgroup)": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample", False) for _ in range(MAX_SETS)],
-        "S5 random_sample f16 voc 151936, top-k = voc (more than 1024 candidates), top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 151936, gen, "random_sample") for _ in range(MAX_SETS)],
+        "S5 random_sample f16 voc 151936, top-k off (= voc: the histogram form), top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 151936, 151936, gen, "random_sample") for _ in range(MAX_SETS)],
+        "S6 random_sample f16 voc 151936, top-k off, top-p 1, temperature 1 (plain sampling from the whole distribution)": lambda: [make_random_sample(ctx, 151936, 151936, gen, "random_sample", True, 1.0, 1.0) for _ in range(MAX_SETS)],
         "Q1 rms_norm bf16 [524288,128] w f32 (a per-head norm: 8192 tokens x 64 heads)": lambda: [make_rms_norm(ctx, 524288, 128, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * 524288 * 128, nset))],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
         "N1b causal_softmax bf16 [32,4096,4096] (the Attention row's softmax on its own)": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, bf16, gen, "causal_softmax") for _ in range(2)],
