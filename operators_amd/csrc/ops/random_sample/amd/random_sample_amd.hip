@@ -16,18 +16,18 @@
 //  * the first wavefront forms the sequential running sums once, as a
 //    branch-free chain with the addends in registers, and takes the top-p and
 //    random_val decisions with ballots over them.
-// That is the form for up to 256 candidates (topk after clamping).  One
-// workgroup of 1024 lanes does all of it from the logits in one launch
-// (topk_full; 32 000 logits take it several times as long as the two-launch
-// form: one compute unit's instruction rate is the limit).  With the workspace
-// the descriptor asks for and 4096 logits or more, a first launch spreads the
-// pass over the logits over up to 48 workgroups, each of which drops
-// everything that cannot be in the overall topk, and a second launch of one
-// workgroup finishes from the few hundred survivors (6.9 + 10.3 us for 32 000
-// logits, 9.7 + 14.0 us for 151 936).
-// More candidates than that - any number, the reference has no limit - are
-// not ranked at all: the running sums are formed over a histogram of the keys
-// (further down).
+// That is the form for up to 256 candidates (topk after clamping) when the
+// caller hands over the workspace the descriptor asks for and there are 4096
+// logits or more: a first launch spreads the pass over the logits over up to
+// 48 workgroups, each of which drops everything that cannot be in the overall
+// topk, and a second launch of one workgroup finishes from the few hundred
+// survivors (6.9 + 10.3 us for 32 000 logits, 9.7 + 14.0 us for 151 936).
+// (One workgroup can do all of it from the logits alone - topk_full, which the
+// second launch falls back to when a list overflows - but takes several times
+// as long: one compute unit's instruction rate is the limit.)
+// More candidates than that - any number, the reference has no limit - and
+// every call without the workspace are not ranked at all: the running sums
+// are formed over a histogram of the keys (further down).
 //
 // Two things differ from the CPU path and are visible to a caller:
 //  * equal logits: the CPU's selection sort leaves equal values in an order
@@ -1012,13 +1012,6 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
     }
 }
 
-template<typename T, bool VEC>
-__global__ __launch_bounds__(BS) void random_sample_topk(uint64_t *result, const uint16_t *probs, uint32_t voc,
-                                                          float random_val, float topp, uint32_t topk, float temperature) {
-    __shared__ TopkShared sh;
-    topk_full<T, VEC>(sh, result, probs, voc, random_val, topp, topk, temperature);
-}
-
 // ---- the same in two launches, the first spread over the chip ---------------
 // First launch: workgroup w of 256 lanes takes the logits
 // [w * 2048 * vecs, (w + 1) * 2048 * vecs) and leaves in the workspace
@@ -1295,15 +1288,20 @@ struct RandomSampleCall {
 };
 
 // form 2: sampling, 1: greedy, 0: nothing to launch.  Sampling with up to
-// kRandomSamplePartTopk candidates ranks them in LDS (candidate lists through
-// the workspace, or one workgroup alone); with more it walks the histogram of
-// keys (counts through the workspace, or one workgroup alone).
+// kRandomSamplePartTopk candidates and the workspace ranks them in LDS
+// (candidate lists from a first launch); with more candidates it walks the
+// histogram of keys (counts from two launches before it); without the
+// workspace one workgroup walks the histogram whatever the candidate count -
+// measured against the one-workgroup ranking form (topk_full, still what the
+// second launch of the list form falls back to), top-k 50, MI355X: 13.9
+// against 18.1 us at 512 logits, 29.6 against 57.1 us at 32 000, 94.9 against
+// 211.5 us at 151 936.
 template<typename T, bool VEC>
 void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
     auto *heads = static_cast<RandomSamplePart *>(c.workspace);
     if (form == 1) {
         random_sample_greedy<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc);
-    } else if (form == 2 && c.topk > static_cast<uint32_t>(kRandomSamplePartTopk)) {
+    } else if (form == 2 && (c.topk > static_cast<uint32_t>(kRandomSamplePartTopk) || heads == nullptr)) {
         if (heads != nullptr) {
             auto *counts = reinterpret_cast<uint32_t *>(heads + kRandomSampleMaxGroups);
             random_sample_clear<<<kRandomSampleKeys / (256 * 4), 256, 0, s>>>(reinterpret_cast<u32x4 *>(counts));
@@ -1314,12 +1312,10 @@ void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
             random_sample_wide<T, VEC, false><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature,
                                                                nullptr, nullptr, c.groups, c.vecs);
         }
-    } else if (form == 2 && heads != nullptr) {
+    } else if (form == 2) {
         auto *lists = reinterpret_cast<unsigned long long *>(heads + kRandomSampleMaxGroups);
         random_sample_partial<T, VEC><<<c.groups, kRandomSamplePartLanes, 0, s>>>(heads, lists, c.probs, c.voc, c.vecs, c.topk, c.temperature);
         random_sample_merge<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature, heads, lists, c.groups);
-    } else if (form == 2) {
-        random_sample_topk<T, VEC><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature);
     }
 }
 
