@@ -527,37 +527,78 @@ __global__ __launch_bounds__(kWave) void rms_norm_short(uint16_t *y, const uint1
 
 // ---- any row length, any alignment ----------------------------------------------
 // Two passes over the row with element accesses; the second pass re-reads x,
-// which the first pass left in cache for rows of ordinary length.
+// which the first pass left in cache for rows of ordinary length.  A lane owns
+// whole groups of 8 elements - the vectors of the kernels above - and rows of
+// up to 65 536 elements are summed in the same order as there (a group's
+// pairwise partial, 64 groups by the wavefront tree, those chunk sums in
+// ascending order), so a row gives the same bits whether its alignment and
+// strides allow the vector kernels or not.  Longer rows, which only this
+// kernel serves, add the chunk sums per wavefront first.
 template<typename T, bool ADD>
 __global__ __launch_bounds__(256) void rms_norm_generic(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                          uint64_t n, uint64_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                          Residual<ADD> res) {
     constexpr int BS = 256, WAVES = BS / kWave;
+    constexpr uint64_t kChunk = 8 * kWave, kMaxChunks = 128;
     __shared__ float red[2 * WAVES];
+    __shared__ float chunk_sum[kMaxChunks];
+    const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const uint64_t chunks = (d + kChunk - 1) / kChunk;
+    const bool in_order = chunks <= kMaxChunks;
     int phase = 0;
     for (uint64_t row = blockIdx.x; row < n; row += gridDim.x, phase ^= 1) {
         const uint16_t *xr = x + static_cast<int64_t>(row) * stride_x;
         uint16_t *yr = y + static_cast<int64_t>(row) * stride_y;
-        float part = 0.0f;
+        const uint16_t *br = nullptr;
+        uint16_t *cr = nullptr;
         if constexpr (ADD) {// first pass forms and stores the sum; the second pass reads it back from c
-            const uint16_t *br = res.b + static_cast<int64_t>(row) * res.stride_b;
-            uint16_t *cr = res.c + static_cast<int64_t>(row) * res.stride_c;
-            for (uint64_t j = threadIdx.x; j < d; j += BS) {
-                const uint16_t sum = T::narrow1(T::one(xr[j]) + T::one(br[j]));
-                cr[j] = sum;
-                const float f = T::one(sum);
-                part += f * f;
+            br = res.b + static_cast<int64_t>(row) * res.stride_b;
+            cr = res.c + static_cast<int64_t>(row) * res.stride_c;
+        }
+        float part = 0.0f;
+        for (uint64_t c = wave; c < chunks; c += WAVES) {
+            const uint64_t j0 = (c * kWave + lane) * 8;
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint64_t j = j0 + e;
+                f[e] = 0.0f;
+                if (j < d) {
+                    if constexpr (ADD) {
+                        const uint16_t sum = T::narrow1(T::one(xr[j]) + T::one(br[j]));
+                        cr[j] = sum;
+                        f[e] = T::one(sum);
+                    } else {
+                        f[e] = T::one(xr[j]);
+                    }
+                }
             }
-            xr = cr;
-        } else {
-            for (uint64_t j = threadIdx.x; j < d; j += BS) {
-                const float f = T::one(xr[j]);
-                part += f * f;
+            const float s = wave_sum(squares8(f));
+            if (in_order) {
+                if (lane == 0) chunk_sum[c] = s;
+            } else {
+                part += s;
             }
         }
-        const float k_row = inv_rms(block_sum<WAVES>(part, red, phase), d, eps);
-        for (uint64_t j = threadIdx.x; j < d; j += BS) {
-            yr[j] = T::narrow1((k_row * T::one(xr[j])) * load_w1(w, w_kind, j));
+        if constexpr (ADD) xr = cr;
+        float total;
+        if (in_order) {
+            __syncthreads();
+            total = 0.0f;
+            for (uint64_t c = 0; c < chunks; ++c) total += chunk_sum[c];
+            __syncthreads();// the next row's chunk sums wait for everyone to have read these
+        } else {
+            // every lane of a wavefront holds the wavefront's sum: one lane of each enters the workgroup's
+            total = block_sum<WAVES>(lane == 0 ? part : 0.0f, red, phase);
+        }
+        const float k_row = inv_rms(total, d, eps);
+        for (uint64_t c = wave; c < chunks; c += WAVES) {
+            const uint64_t j0 = (c * kWave + lane) * 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint64_t j = j0 + e;
+                if (j < d) yr[j] = T::narrow1((k_row * T::one(xr[j])) * load_w1(w, w_kind, j));
+            }
         }
         // y may alias x (and c may alias a or b): every lane re-reads only elements it wrote itself.
     }
