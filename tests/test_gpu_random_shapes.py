@@ -77,6 +77,11 @@ def test_rms_norm_and_fused(ctx, seed):
     torch.cuda.synchronize()
     got_y = to_codes(ty)
     close(got_y, oracle.rms_norm(x, w, eps, dt, wdt), dt, "rms_norm " + what, frac)
+    if seed % 3 == 0:  # in place: the same bits as out of place
+        tx_copy = tx.clone() if sx == d else strided_like(x, (n, d), (sx, 1), dt)[0]
+        ctx.rms_norm(tx_copy, tx_copy, tw, eps)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_codes(tx_copy), got_y), "in place differs: " + what
     # the fused form on the same rows: c = x + b bit for bit Add's, y RMSNorm's of that sum
     tb = to_torch(b, dt)
     tc = torch.empty((n, d), dtype=tx.dtype, device="cuda")
@@ -114,10 +119,12 @@ def test_swiglu(ctx, seed):
     else:  # unrelated row strides
         ta = strided_like(a, (n, di), (di + 8 * int(rng.integers(0, 5)), 1), dt)[0]
         tb = strided_like(b, (n, di), (di + int(rng.choice([0, 8, 5])), 1), dt)[0]
-    tc = torch.empty((n, di), dtype=ta.dtype, device="cuda")
+    # the result into a tensor of its own, or in place over a or over b (the reference's tests do both)
+    where = int(rng.integers(0, 3))
+    tc = torch.empty((n, di), dtype=ta.dtype, device="cuda") if where == 0 else (ta if where == 1 else tb)
     ctx.swiglu(tc, ta, tb)
     torch.cuda.synchronize()
-    close(to_codes(tc), oracle.swiglu(a, b, dt), dt, f"seed {seed}: swiglu [{n},{di}] {dt} layout {layout}")
+    close(to_codes(tc), oracle.swiglu(a, b, dt), dt, f"seed {seed}: swiglu [{n},{di}] {dt} layout {layout} result {where}")
 
 
 @pytest.mark.parametrize("seed", range(40))
@@ -152,6 +159,8 @@ def test_add(ctx, seed):
         b = oracle.encode(rng.standard_normal(sb).astype(np.float32), dt)
     ta, tb = to_torch(a, dt), to_torch(b, dt)
     tc = torch.empty(want_shape, dtype=ta.dtype, device="cuda")
+    if list(sa) == want_shape and rng.random() < 0.3:
+        tc = ta  # in place over the operand that has the result's shape
     ctx.add(tc, ta, tb)
     torch.cuda.synchronize()
     want = oracle.add(a, b, tuple(want_shape), dt)
