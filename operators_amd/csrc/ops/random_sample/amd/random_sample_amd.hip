@@ -488,7 +488,7 @@ __device__ __attribute__((noinline)) void topk_full(TopkShared &sh, uint64_t *re
 // sampling from the whole distribution, costs little more than a peaked one.
 // Without the workspace the one workgroup counts a range at a time itself.
 // 151 936 fp16 logits, top-k off, MI355X, with the workspace: 54 us at top-p
-// 0.9 (4.5 clear + 19.7 count + 28.8 draw), 112 us at top-p 1; without:
+// 0.9 (4.5 clear + 17.7 count + 28.8 draw), 112 us at top-p 1; without:
 // 87 us and 0.41 ms.  (Before the measures described here and below: 223 us
 // and 5.9 ms.)
 // The additions need not be made one by one.  An fp16 probability is a whole
@@ -805,7 +805,7 @@ __device__ __forceinline__ void wide_walk(WideShared &sh, const uint16_t *probs,
 // the bit, and with it the same probabilities and the same draw.
 template<typename T, bool VEC>
 __device__ __forceinline__ void part_max_and_sum(const uint16_t *probs, uint32_t voc, uint32_t start, uint32_t vecs, float temperature,
-                                                 bool active, uint32_t t, uint32_t *key_slots, float *sum_slots, uint32_t *counts,
+                                                 bool active, uint32_t t, uint32_t *key_slots, float *sum_slots,
                                                  uint32_t &key_max, float &sum) {
     constexpr uint32_t PL = kRandomSamplePartLanes;
     const uint32_t lane = t & (kWave - 1), w = t / kWave;
@@ -821,7 +821,6 @@ __device__ __forceinline__ void part_max_and_sum(const uint16_t *probs, uint32_t
                     if (e < n) {
                         const uint32_t k = key_of<T>(h[e]);
                         km = k > km ? k : km;
-                        if (counts != nullptr) atomicAdd(&counts[k], 1u);
                     }
                 }
             }
@@ -859,20 +858,36 @@ __device__ __forceinline__ void part_max_and_sum(const uint16_t *probs, uint32_t
 }
 
 // First launches of the split form: clear the counts, then one workgroup per
-// part of the logits counts every key and leaves its part's maximum and sum.
+// part of the logits leaves its part's maximum and sum while further
+// workgroups count every key.
 __global__ __launch_bounds__(256) void random_sample_clear(u32x4 *counts) {
     counts[blockIdx.x * 256u + threadIdx.x] = u32x4{0, 0, 0, 0};
 }
 
 template<typename T, bool VEC>
 __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_count(RandomSamplePart *heads, uint32_t *counts, const uint16_t *probs,
-                                                                                uint32_t voc, uint32_t vecs, float temperature) {
+                                                                                uint32_t voc, uint32_t groups, uint32_t vecs, float temperature) {
     __shared__ uint32_t key_slots[kRandomSamplePartLanes / kWave];
     __shared__ float sum_slots[kRandomSamplePartLanes / kWave];
+    if (blockIdx.x >= groups) {
+        // The workgroups behind the first `groups` only count: one vector of eight logits per lane, one atomic add
+        // per logit.  It is the atomic adds that this launch waits for: 151 936 of them take 13 us however they are
+        // spread (the sums alone: 4.8 us; counting inside the summing workgroups: 19.2 us in all; like this: 17.7).
+        const uint32_t base = ((blockIdx.x - groups) * kRandomSamplePartLanes + threadIdx.x) * 8u;
+        if (base < voc) {
+            uint32_t h[8];
+            const int n = load_codes<VEC>(probs, voc, base, h);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (e < n) atomicAdd(&counts[key_of<T>(h[e])], 1u);
+            }
+        }
+        return;
+    }
     uint32_t key_max;
     float sum;
     part_max_and_sum<T, VEC>(probs, voc, blockIdx.x * (kRandomSamplePartLanes * 8u * vecs), vecs, temperature, true, threadIdx.x,
-                             key_slots, sum_slots, counts, key_max, sum);
+                             key_slots, sum_slots, key_max, sum);
     if (threadIdx.x == 0) heads[blockIdx.x] = RandomSamplePart{0, key_max, sum, 0};
 }
 
@@ -905,7 +920,7 @@ __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const
             uint32_t key_max;
             float sum;
             part_max_and_sum<T, VEC>(probs, voc, g * (PL * 8u * vecs), vecs, temperature, g < groups, t,
-                                     key_slots + side * (PL / kWave), sum_slots4 + side * (PL / kWave), nullptr, key_max, sum);
+                                     key_slots + side * (PL / kWave), sum_slots4 + side * (PL / kWave), key_max, sum);
             if (g < groups && t == 0) {
                 sh.part_key[g] = key_max;
                 sh.part_sum[g] = sum;
@@ -1305,7 +1320,8 @@ void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
         if (heads != nullptr) {
             auto *counts = reinterpret_cast<uint32_t *>(heads + kRandomSampleMaxGroups);
             random_sample_clear<<<kRandomSampleKeys / (256 * 4), 256, 0, s>>>(reinterpret_cast<u32x4 *>(counts));
-            random_sample_count<T, VEC><<<c.groups, kRandomSamplePartLanes, 0, s>>>(heads, counts, c.probs, c.voc, c.vecs, c.temperature);
+            const unsigned counting = static_cast<unsigned>(amd::ceil_div(c.voc, kRandomSamplePartLanes * 8u));
+            random_sample_count<T, VEC><<<c.groups + counting, kRandomSamplePartLanes, 0, s>>>(heads, counts, c.probs, c.voc, c.groups, c.vecs, c.temperature);
             random_sample_wide<T, VEC, true><<<1, BS, 0, s>>>(c.result, c.probs, c.voc, c.random_val, c.topp, c.topk, c.temperature,
                                                               heads, counts, c.groups, c.vecs);
         } else {
