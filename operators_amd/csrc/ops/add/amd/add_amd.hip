@@ -71,6 +71,7 @@ struct Add32 {
 // ranges beyond what one launch may span: 2^32 work-items.)
 template<typename Op>
 __global__ __launch_bounds__(kWave) void add_flat_vec(u32x4 *c, const u32x4 *a, const u32x4 *b, uint64_t nvec) {
+    AMD_ARGS_NOW(c, a, b, nvec, gridDim.x);
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kWave;
     for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kWave + threadIdx.x; i < nvec; i += step) {
         const u32x4 va = ld16_stream(a + i);
@@ -195,15 +196,15 @@ __global__ __launch_bounds__(kBlock) void add_bcast_rows(u32x4 *c, const typenam
 // [8192, 8192] bf16: 40.9 against 42.7 us.
 // SWAP says the row is operand a (the sum is formed as a + b either way).
 template<typename Op, bool SWAP, bool THROUGH>
-__global__ __launch_bounds__(kWave) void add_rowvec_tiles(u32x4 *c, const u32x4 *full, const u32x4 *vec, uint32_t tiles_per_row, uint64_t ntiles) {
-    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {// more than one pass only beyond what one launch may span
-        const uint32_t ct = static_cast<uint32_t>(tile % tiles_per_row);
-        const u32x4 vv = ld16(vec + ct * kWave + threadIdx.x);
-        const u32x4 vf = ld16_stream(full + tile * kWave + threadIdx.x);
-        const u32x4 r = SWAP ? Op::vec(vv, vf) : Op::vec(vf, vv);
-        if constexpr (THROUGH) StreamOut<true>(c + tile * kWave).st16(threadIdx.x * 16, r);
-        else st16_stream(c + tile * kWave + threadIdx.x, r);
-    }
+__global__ __launch_bounds__(kWave) void add_rowvec_tiles(u32x4 *c, const u32x4 *full, const u32x4 *vec, uint32_t tiles_per_row, FastDiv by_row) {
+    AMD_ARGS_NOW(c, full, vec, tiles_per_row, by_row.mul, by_row.shift);
+    const uint32_t tile = blockIdx.x;// one tile per workgroup: the host takes this form only for what one launch spans
+    const uint32_t ct = tile - fast_quotient(tile, by_row) * tiles_per_row;// tile % tiles_per_row
+    const u32x4 vv = ld16(vec + ct * kWave + threadIdx.x);
+    const u32x4 vf = ld16_stream(full + static_cast<uint64_t>(tile) * kWave + threadIdx.x);
+    const u32x4 r = SWAP ? Op::vec(vv, vf) : Op::vec(vf, vv);
+    if constexpr (THROUGH) StreamOut<true>(c + static_cast<uint64_t>(tile) * kWave).st16(threadIdx.x * 16, r);
+    else st16_stream(c + static_cast<uint64_t>(tile) * kWave + threadIdx.x, r);
 }
 
 // Element form: any strides.
@@ -302,18 +303,19 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         const bool through = (ma == kFull) != (mb == kFull) && n * sizeof(S) >= kWriteThroughBytes && inner_vecs < (1ull << 28);
         bool launched = false;
         // a whole tensor plus one row whose length is a multiple of a wavefront of vectors
-        if (desc.ndim == 2 && inner_vecs % kWave == 0 && inner_vecs < (1ull << 31) &&
+        // (up to what one launch of single-wavefront workgroups spans, 64 GiB of 16-bit output; beyond that the general kernels below)
+        if (desc.ndim == 2 && inner_vecs % kWave == 0 && desc.shape[1] * (inner_vecs / kWave) < max_grid_1d(kWave) &&
             ((ma == kFull && mb == kRuns && desc.b_stride[1] == 0) || (ma == kRuns && mb == kFull && desc.a_stride[1] == 0))) {
             const bool swap = ma == kRuns;
             const u32x4 *full = static_cast<const u32x4 *>(swap ? b : a), *vec = static_cast<const u32x4 *>(swap ? a : b);
             u32x4 *pc = static_cast<u32x4 *>(c);
             const uint32_t tpr = static_cast<uint32_t>(inner_vecs / kWave);
-            const uint64_t ntiles = desc.shape[1] * tpr;
-            const unsigned g = static_cast<unsigned>(ntiles < max_grid_1d(kWave) ? ntiles : max_grid_1d(kWave));
-            if (swap && through) add_rowvec_tiles<Op, true, true><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
-            else if (swap) add_rowvec_tiles<Op, true, false><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
-            else if (through) add_rowvec_tiles<Op, false, true><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
-            else add_rowvec_tiles<Op, false, false><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, ntiles);
+            const unsigned g = static_cast<unsigned>(desc.shape[1] * tpr);
+            const FastDiv by_row = fast_div(tpr);
+            if (swap && through) add_rowvec_tiles<Op, true, true><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, by_row);
+            else if (swap) add_rowvec_tiles<Op, true, false><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, by_row);
+            else if (through) add_rowvec_tiles<Op, false, true><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, by_row);
+            else add_rowvec_tiles<Op, false, false><<<g, kWave, 0, stream>>>(pc, full, vec, tpr, by_row);
             return STATUS_SUCCESS;
         }
 #define ADD_BCAST_CASE(MA, MB)                                        \

@@ -60,7 +60,8 @@ __device__ __attribute__((noinline)) void exp_any8(float *v, float mx) {
 // one request.
 template<typename T, int BS, int NV, bool THROUGH>
 __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
-                                                          int64_t stride_b, int64_t stride_i) {
+                                                          int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
+    AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
     constexpr int WAVES = BS / kWave;
     __shared__ float red[4 * WAVES];// two slot sets for the maxima, two for the sums
     const uint32_t nvec = total / 8;
@@ -74,8 +75,8 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
     // any one time (measured: faster than giving each matrix of the batch its
     // own workgroups); (b, i) is advanced by the constant hop without dividing.
     const uint32_t hop = gridDim.x;
-    const uint32_t hop_b = hop / seq, hop_i = hop - hop_b * seq;
-    uint64_t b = blockIdx.x / seq;
+    const uint32_t hop_b = fast_quotient(hop, by_seq), hop_i = hop - hop_b * seq;// the grid is far below 2^31 rows (see FastDiv)
+    uint64_t b = fast_quotient(blockIdx.x, by_seq);
     uint32_t i = blockIdx.x - static_cast<uint32_t>(b) * seq;
     auto here = [&]() { return Row{y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i, total - seq + i + 1}; };
     auto advance = [&]() {
@@ -278,14 +279,15 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         return;
     }
     const bool through = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
+    const FastDiv by_seq = fast_div(static_cast<uint32_t>(d.seq));
 #define CS_LAUNCH(BS, NV)                                                                                                      \
     do {                                                                                                                       \
         if (through)                                                                                                           \
             causal_softmax_rows<T, BS, NV, true><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),              \
-                                                                          static_cast<uint32_t>(d.total), d.stride_b, d.stride_i); \
+                                                                          static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by_seq); \
         else                                                                                                                   \
             causal_softmax_rows<T, BS, NV, false><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),             \
-                                                                           static_cast<uint32_t>(d.total), d.stride_b, d.stride_i); \
+                                                                           static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by_seq); \
     } while (0)
     if (nvec <= 64) CS_LAUNCH(64, 1);
     else if (nvec <= 128) CS_LAUNCH(64, 2);

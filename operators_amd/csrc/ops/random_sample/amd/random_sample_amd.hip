@@ -194,6 +194,7 @@ __device__ __forceinline__ uint32_t wave_scan_u32(uint32_t v) {
 // where NaN is never greater than anything and a NaN in front is never beaten.
 template<typename T, bool VEC>
 __global__ __launch_bounds__(BS) void random_sample_greedy(uint64_t *result, const uint16_t *probs, uint32_t voc) {
+    AMD_ARGS_NOW(result, probs, voc);
     __shared__ unsigned long long best_of[WAVES];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     unsigned long long best = 0;
@@ -867,6 +868,7 @@ __global__ __launch_bounds__(256) void random_sample_clear(u32x4 *counts) {
 template<typename T, bool VEC>
 __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_count(RandomSamplePart *heads, uint32_t *counts, const uint16_t *probs,
                                                                                 uint32_t voc, uint32_t groups, uint32_t vecs, float temperature) {
+    AMD_ARGS_NOW(heads, counts, probs, voc, groups, vecs, temperature);
     __shared__ uint32_t key_slots[kRandomSamplePartLanes / kWave];
     __shared__ float sum_slots[kRandomSamplePartLanes / kWave];
     if (blockIdx.x >= groups) {
@@ -898,6 +900,7 @@ template<typename T, bool VEC, bool SPLIT>
 __global__ __launch_bounds__(BS) void random_sample_wide(uint64_t *result, const uint16_t *probs, uint32_t voc,
                                                           float random_val, float topp, uint32_t topk, float temperature,
                                                           const RandomSamplePart *heads, const uint32_t *counts, uint32_t groups, uint32_t vecs) {
+    AMD_ARGS_NOW(result, probs, voc, random_val, topp, topk, temperature, heads, counts, groups, vecs);
     __shared__ WideShared sh;
     __shared__ uint32_t key_slots[BS / kWave];
     __shared__ float sum_slots4[BS / kWave];
@@ -1046,6 +1049,7 @@ template<typename T, bool VEC>
 __global__ __launch_bounds__(kRandomSamplePartLanes) void random_sample_partial(RandomSamplePart *heads, unsigned long long *lists,
                                                                                   const uint16_t *probs, uint32_t voc,
                                                                                   uint32_t vecs, uint32_t topk, float temperature) {
+    AMD_ARGS_NOW(heads, lists, probs, voc, vecs, topk, temperature);
     constexpr int PBS = kRandomSamplePartLanes, PW = PBS / kWave;
     __shared__ __attribute__((aligned(16))) uint32_t lane_rank_key[PBS];
     __shared__ uint32_t bound_slot, max_slot, data_lanes;
@@ -1161,6 +1165,7 @@ __global__ __launch_bounds__(BS) void random_sample_merge(uint64_t *result, cons
                                                            float topp, uint32_t topk, float temperature,
                                                            const RandomSamplePart *heads, const unsigned long long *lists,
                                                            uint32_t groups) {
+    AMD_ARGS_NOW(result, probs, voc, random_val, topp, topk, temperature, heads, lists, groups);
     constexpr int CMAX = 4096, PER_LANE = CMAX / BS;
     __shared__ TopkShared sh;
     __shared__ unsigned long long pool[CMAX];

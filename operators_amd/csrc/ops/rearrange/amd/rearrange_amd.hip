@@ -25,7 +25,16 @@ struct OuterDims {
     uint32_t shape[kRearrangeMaxDims];
     int64_t dst_stride[kRearrangeMaxDims];
     int64_t src_stride[kRearrangeMaxDims];
+    FastDiv by_shape[kRearrangeMaxDims];// division by shape[k], for the FAST kernels
 };
+
+// All of an OuterDims argument as operands of AMD_ARGS_NOW: 22 of them, neighbours of 4 bytes taken two at a time.
+#define ARGS_OF_DIMS(d)                                                                                                                          \
+    d.ndim, arg_pair(d.shape[0], d.shape[1]), arg_pair(d.shape[2], d.shape[3]), arg_pair(d.shape[4], d.shape[5]), d.dst_stride[0], d.dst_stride[1],             \
+        d.dst_stride[2], d.dst_stride[3], d.dst_stride[4], d.dst_stride[5], d.src_stride[0], d.src_stride[1], d.src_stride[2], d.src_stride[3], \
+        d.src_stride[4], d.src_stride[5], arg_pair(d.by_shape[0]), arg_pair(d.by_shape[1]), arg_pair(d.by_shape[2]), arg_pair(d.by_shape[3]), arg_pair(d.by_shape[4]),   \
+        arg_pair(d.by_shape[5])
+static_assert(kRearrangeMaxDims == 6, "ARGS_OF_DIMS lists six dimensions");
 
 // The access unit: the widest of 16, 8, 4, 2, 1 bytes that divides the row
 // length, every stride and both base addresses.
@@ -42,21 +51,37 @@ template<> struct Unit<1> { typedef uint8_t type; };
 // since the row number is uniform.
 // BUFST (16-byte units, large outputs): stores are written through L2 as
 // buffer stores relative to the start of the destination row (see StreamOut).
-template<int BYTES, bool BUFST, int LANES>
+template<int BYTES, bool BUFST, int LANES, bool FAST>
 __global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row) {
     typedef typename Unit<BYTES>::type U;
+    // every argument up front (see AMD_ARGS_NOW; the number of rows to step by is not needed before the first load is out)
+    AMD_ARGS_NOW(dst, src, rows, units_per_row, ARGS_OF_DIMS(d));
     const uint32_t col = blockIdx.x * LANES + threadIdx.x;
     if (col >= units_per_row) return;
     for (uint64_t r = blockIdx.y; r < rows; r += gridDim.y) {
         int64_t od = 0, os = 0;
-        uint64_t rest = r;
+        if constexpr (FAST) {// fewer than 2^31 rows: multiplications instead of divisions
+            uint32_t rest = static_cast<uint32_t>(r);
 #pragma unroll
-        for (int k = 0; k < kRearrangeMaxDims; ++k) {
-            if (k < d.ndim) {
-                const uint64_t i = rest % d.shape[k];
-                rest /= d.shape[k];
-                od += static_cast<int64_t>(i) * d.dst_stride[k];
-                os += static_cast<int64_t>(i) * d.src_stride[k];
+            for (int k = 0; k < kRearrangeMaxDims; ++k) {
+                if (k < d.ndim) {
+                    const uint32_t q = fast_quotient(rest, d.by_shape[k]);
+                    const uint32_t i = rest - q * d.shape[k];
+                    rest = q;
+                    od += static_cast<int64_t>(i) * d.dst_stride[k];
+                    os += static_cast<int64_t>(i) * d.src_stride[k];
+                }
+            }
+        } else {
+            uint64_t rest = r;
+#pragma unroll
+            for (int k = 0; k < kRearrangeMaxDims; ++k) {
+                if (k < d.ndim) {
+                    const uint64_t i = rest % d.shape[k];
+                    rest /= d.shape[k];
+                    od += static_cast<int64_t>(i) * d.dst_stride[k];
+                    os += static_cast<int64_t>(i) * d.src_stride[k];
+                }
             }
         }
         const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
@@ -73,25 +98,44 @@ __global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint
 // allows, which makes the divisions cheap.  BUFST (16-byte units only): the
 // whole destination lies within 4 GiB of its base and no stride is negative,
 // so stores go out as buffer stores relative to the base (see StreamOut).
-template<int BYTES, typename Idx, bool BUFST>
-__global__ __launch_bounds__(Lanes<BYTES>::value) void rearrange_flat(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t total_units, Idx units_per_row) {
+template<int BYTES, typename Idx, bool BUFST, bool FAST>
+__global__ __launch_bounds__(Lanes<BYTES>::value) void rearrange_flat(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t total_units, Idx units_per_row,
+                                                                    FastDiv by_row) {
     typedef typename Unit<BYTES>::type U;
+    AMD_ARGS_NOW(dst, src, total_units, units_per_row, arg_pair(by_row), gridDim.x, ARGS_OF_DIMS(d));
     // one pass for anything a single launch can span (2^32 work-items); the loop covers the rest
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * Lanes<BYTES>::value;
     for (uint64_t idx64 = static_cast<uint64_t>(blockIdx.x) * Lanes<BYTES>::value + threadIdx.x; idx64 < total_units; idx64 += step) {
         const Idx idx = static_cast<Idx>(idx64);
-        Idx rest = idx / units_per_row;
-        const Idx col = idx - rest * units_per_row;
+        Idx rest, col;
         int64_t od = 0, os = 0;
+        if constexpr (FAST) {// fewer than 2^31 units in all: multiplications instead of divisions
+            static_assert(sizeof(Idx) == 4, "FAST numbers units with 32 bits");
+            rest = fast_quotient(idx, by_row);
+            col = idx - rest * units_per_row;
 #pragma unroll
-        for (int k = 0; k < kRearrangeMaxDims; ++k) {
-            if (k < d.ndim) {
-                const Idx ext = static_cast<Idx>(d.shape[k]);
-                const Idx q = rest / ext;
-                const Idx i = rest - q * ext;
-                rest = q;
-                od += static_cast<int64_t>(i) * d.dst_stride[k];
-                os += static_cast<int64_t>(i) * d.src_stride[k];
+            for (int k = 0; k < kRearrangeMaxDims; ++k) {
+                if (k < d.ndim) {
+                    const uint32_t q = fast_quotient(rest, d.by_shape[k]);
+                    const uint32_t i = rest - q * d.shape[k];
+                    rest = q;
+                    od += static_cast<int64_t>(i) * d.dst_stride[k];
+                    os += static_cast<int64_t>(i) * d.src_stride[k];
+                }
+            }
+        } else {
+            rest = idx / units_per_row;
+            col = idx - rest * units_per_row;
+#pragma unroll
+            for (int k = 0; k < kRearrangeMaxDims; ++k) {
+                if (k < d.ndim) {
+                    const Idx ext = static_cast<Idx>(d.shape[k]);
+                    const Idx q = rest / ext;
+                    const Idx i = rest - q * ext;
+                    rest = q;
+                    od += static_cast<int64_t>(i) * d.dst_stride[k];
+                    os += static_cast<int64_t>(i) * d.src_stride[k];
+                }
             }
         }
         const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
@@ -130,28 +174,36 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         const int lanes = wave_rows ? kWave : (half ? 128 : 256);
         const dim3 grid(static_cast<unsigned>(ceil_div(upr, lanes)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
         const bool bufst = BYTES == 16 && large && desc.row_bytes < (1ull << 32);
-        if (wave_rows) {
-            if (bufst) rearrange_rows<BYTES, BYTES == 16, kWave><<<grid, kWave, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
-            else rearrange_rows<BYTES, false, kWave><<<grid, kWave, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
-        } else if (half) {
-            if (bufst) rearrange_rows<BYTES, BYTES == 16, 128><<<grid, 128, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
-            else rearrange_rows<BYTES, false, 128><<<grid, 128, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
-        } else {
-            if (bufst) rearrange_rows<BYTES, BYTES == 16, 256><<<grid, 256, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
-            else rearrange_rows<BYTES, false, 256><<<grid, 256, 0, stream>>>(pd, ps, d, desc.rows, static_cast<uint32_t>(upr));
-        }
+        const bool fast = desc.rows < kFastDivLimit;
+        const uint32_t upr32 = static_cast<uint32_t>(upr);
+#define REARRANGE_ROWS(BUFST, LANES, FAST) rearrange_rows<BYTES, BUFST, LANES, FAST><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32)
+#define REARRANGE_ROWS_OF(LANES)                                      \
+    do {                                                              \
+        if (bufst && fast) REARRANGE_ROWS(BYTES == 16, LANES, true);  \
+        else if (bufst) REARRANGE_ROWS(BYTES == 16, LANES, false);    \
+        else if (fast) REARRANGE_ROWS(false, LANES, true);            \
+        else REARRANGE_ROWS(false, LANES, false);                     \
+    } while (0)
+        if (wave_rows) REARRANGE_ROWS_OF(kWave);
+        else if (half) REARRANGE_ROWS_OF(128);
+        else REARRANGE_ROWS_OF(256);
+#undef REARRANGE_ROWS_OF
+#undef REARRANGE_ROWS
     } else {// short rows, or a single row too long for 32-bit column numbers
         const uint64_t total = desc.rows * upr;
         const uint64_t want = ceil_div(total, kBlock);
         const uint64_t blocks = want < max_grid_1d(kBlock) ? want : max_grid_1d(kBlock);
-        if (total < (1ull << 32)) {
-            if (BYTES == 16 && large && forward && dst_span < (1ull << 32)) {
-                rearrange_flat<BYTES, uint32_t, BYTES == 16><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr));
-            } else {
-                rearrange_flat<BYTES, uint32_t, false><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr));
-            }
+        const unsigned grid = static_cast<unsigned>(blocks);
+        const bool bufst = BYTES == 16 && large && forward && dst_span < (1ull << 32);
+        if (total < kFastDivLimit) {
+            const FastDiv by_row = fast_div(static_cast<uint32_t>(upr));
+            if (bufst) rearrange_flat<BYTES, uint32_t, BYTES == 16, true><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row);
+            else rearrange_flat<BYTES, uint32_t, false, true><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row);
+        } else if (total < (1ull << 32)) {
+            if (bufst) rearrange_flat<BYTES, uint32_t, BYTES == 16, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), FastDiv{});
+            else rearrange_flat<BYTES, uint32_t, false, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), FastDiv{});
         } else {
-            rearrange_flat<BYTES, uint64_t, false><<<static_cast<unsigned>(blocks), kBlock, 0, stream>>>(pd, ps, d, total, upr);
+            rearrange_flat<BYTES, uint64_t, false, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, upr, FastDiv{});
         }
     }
 }
@@ -177,6 +229,7 @@ infiniopStatus_t amdRearrange(RearrangeAmdDescriptor_t desc, void *dst, void con
         d.shape[k] = used ? static_cast<uint32_t>(desc->shape[k]) : 1;
         d.dst_stride[k] = used ? desc->dst_stride[k] : 0;
         d.src_stride[k] = used ? desc->src_stride[k] : 0;
+        d.by_shape[k] = fast_div(d.shape[k] < kFastDivLimit ? d.shape[k] : 1);// an extent beyond the limit means more rows than the FAST kernels take
         if (used) align |= static_cast<uint64_t>(desc->dst_stride[k]) | static_cast<uint64_t>(desc->src_stride[k]);
     }
     AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);

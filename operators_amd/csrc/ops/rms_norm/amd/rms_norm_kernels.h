@@ -180,10 +180,18 @@ struct Residual<true> {
 };
 namespace {
 
+// Every argument of a kernel below fetched at its top (see AMD_ARGS_NOW); `more` are the kernel's own beside the common ones.
+#define RMS_ARGS_NOW(...)                                                                                                                 \
+    do {                                                                                                                                  \
+        if constexpr (ADD) AMD_ARGS_NOW(y, x, w, w_kind, n, d, stride_y, stride_x, eps, res.c, res.b, res.stride_c, res.stride_b, ##__VA_ARGS__); \
+        else AMD_ARGS_NOW(y, x, w, w_kind, n, d, stride_y, stride_x, eps, ##__VA_ARGS__);                                                  \
+    } while (0)
+
 template<typename T, int BS, int NV, int WHOME, bool EXACT, bool THROUGH, bool ADD, bool AHEAD = true>
 __global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                      uint64_t first_mul, uint64_t hop, uint64_t span, Residual<ADD> res) {
+    RMS_ARGS_NOW(first_mul, hop, span, blockDim.x);
     // BS = 0: the lane count is the launch's (any multiple of 64 up to 1024)
     constexpr int MAX_WAVES = (BS != 0 ? BS : 1024) / kWave;
     const uint32_t bs = BS != 0 ? BS : blockDim.x;
@@ -351,6 +359,7 @@ template<typename T, int BS, int NV, int R, bool EXACT, bool THROUGH, bool ADD>
 __global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                      Residual<ADD> res) {
+    RMS_ARGS_NOW();
     constexpr int WAVES = BS / kWave;
     __shared__ float red[R * NV * WAVES];
     const uint32_t nvec = d / 8;
@@ -493,6 +502,7 @@ template<typename T, int P, bool THROUGH, bool ADD>
 __global__ __launch_bounds__(kWave) void rms_norm_short(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                         uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                         Residual<ADD> res) {
+    RMS_ARGS_NOW(gridDim.x);
     constexpr uint32_t RPW = kWave / P;// rows per wavefront
     const uint32_t nvec = d / 8;
     const uint32_t sub = threadIdx.x % P, rr = threadIdx.x / P;
@@ -538,6 +548,7 @@ template<typename T, bool ADD>
 __global__ __launch_bounds__(256) void rms_norm_generic(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                          uint64_t n, uint64_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                          Residual<ADD> res) {
+    RMS_ARGS_NOW(gridDim.x);
     constexpr int BS = 256, WAVES = BS / kWave;
     constexpr uint64_t kChunk = 8 * kWave, kMaxChunks = 128;
     __shared__ float red[2 * WAVES];

@@ -110,31 +110,39 @@ __global__ __launch_bounds__(kBlock) void rope_vec(uint16_t *t, const uint64_t *
 
 // One pass, one tile of BS work items per workgroup, in the order the
 // dispatcher hands workgroups out.  UNI: a token's work items are a multiple
-// of BS, so a workgroup lies inside one token and its position and table base
-// are found with scalar arithmetic and scalar loads, which run beside the
-// vector loads of the data.  Otherwise every lane loads its token's position
-// itself, after the data loads: asked for first, the position delays the data
-// behind it (k [8192, 8, 128] bf16 with 4 heads per lane: 10.6 us position
-// first, 8.7 us position last).  The head count is a multiple of HPT (every
-// lane's heads exist): nothing is predicated, so no load can sink into a
-// branch behind the wait for another.
+// of BS, so a workgroup lies inside one token and its position is one load
+// from a uniform address, asked for before the data and waited for alone
+// (vector loads return in order).  Otherwise every lane loads its token's
+// position itself, after the data loads: asked for first, the position delays
+// the data behind it (k [8192, 8, 128] bf16 with 4 heads per lane: 10.6 us
+// position first, 8.7 us position last).  Positions fetched per wavefront
+// through the scalar unit, so that the table loads can follow the data loads
+// at once, measured the same as that (k 8.8 us, [4096, 32, 128] fp16 13.2 us):
+// in a tensor of this size the strided rows bound the time (a strided copy of
+// k's rows takes 9.4 us, a dense one 8.2 us).
+// The head count is a multiple of HPT (every lane's heads exist): nothing is
+// predicated, so no load can sink into a branch behind the wait for another.
 template<typename T, int BS, int HPT, bool BUFST, bool UNI>
 __global__ __launch_bounds__(BS) void rope_once(uint16_t *__restrict__ t, const uint64_t *__restrict__ pos,
                                                 const float *__restrict__ sin_t, const float *__restrict__ cos_t,
                                                 uint32_t total_items, uint32_t items_per_token, uint32_t vecs_per_head, uint32_t groups,
-                                                uint32_t head_dim, int64_t stride_token, int64_t stride_head) {
+                                                uint32_t head_dim, int64_t stride_token, int64_t stride_head, FastDiv by_token,
+                                                FastDiv by_head) {
+    AMD_ARGS_NOW(t, pos, sin_t, cos_t, total_items, items_per_token, vecs_per_head, groups, head_dim, stride_token, stride_head,
+                 arg_pair(by_token), arg_pair(by_head));
+    // fewer than 2^31 work items: the two divisions are multiplications (see FastDiv)
     uint32_t token, rem;
     if constexpr (UNI) {
         const uint32_t item0 = blockIdx.x * BS;
-        token = item0 / items_per_token;
+        token = fast_quotient(item0, by_token);
         rem = item0 - token * items_per_token + threadIdx.x;
     } else {
         const uint32_t item = blockIdx.x * BS + threadIdx.x;
         if (item >= total_items) return;
-        token = item / items_per_token;
+        token = fast_quotient(item, by_token);
         rem = item - token * items_per_token;
     }
-    const uint32_t g = rem / vecs_per_head;
+    const uint32_t g = fast_quotient(rem, by_head);
     const uint32_t cv = rem - g * vecs_per_head;
     uint64_t p;
     if constexpr (UNI) p = pos[token];
@@ -256,7 +264,8 @@ void launch_vec(const RoPEAmdDescriptor &d, uint16_t *t, const uint64_t *pos, co
     rope_once<T, kBlock, HPT, B, U><<<grid, kBlock, 0, stream>>>(t, pos, sn, cs, static_cast<uint32_t>(total),                \
                                                                  static_cast<uint32_t>(ipt), static_cast<uint32_t>(vph),      \
                                                                  static_cast<uint32_t>(groups), static_cast<uint32_t>(d.head_dim), \
-                                                                 d.stride_token, d.stride_head)
+                                                                 d.stride_token, d.stride_head, fast_div(static_cast<uint32_t>(ipt)), \
+                                                                 fast_div(static_cast<uint32_t>(vph)))
 #define ROPE_ONCE_BU(HPT)                                \
     do {                                                 \
         if (b1 && uni) ROPE_ONCE_GO(HPT, true, true);    \

@@ -109,6 +109,7 @@ template<typename T, typename Idx, bool ROWWISE>
 __global__ __launch_bounds__(kWave) void swiglu_vec(uint16_t *c, const uint16_t *a, const uint16_t *b,
                                                      uint64_t nvec, Idx vecs_per_row,
                                                      int64_t stride_c, int64_t stride_a, int64_t stride_b) {
+    AMD_ARGS_NOW(c, a, b, nvec, vecs_per_row, stride_c, stride_a, stride_b, gridDim.x);
     const Where<Idx, ROWWISE> where{vecs_per_row};
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kWave;
     for (uint64_t v = static_cast<uint64_t>(blockIdx.x) * kWave + threadIdx.x; v < nvec; v += step) {
@@ -128,6 +129,7 @@ template<typename T, int LANES>
 __global__ __launch_bounds__(LANES) void swiglu_rows(uint16_t *c, const uint16_t *a, const uint16_t *b,
                                                       uint64_t rows, uint32_t vecs_per_row,
                                                       int64_t stride_c, int64_t stride_a, int64_t stride_b) {
+    AMD_ARGS_NOW(c, a, b, rows, vecs_per_row, stride_c, stride_a, stride_b);
     const uint32_t col = blockIdx.x * LANES + threadIdx.x;
     if (col >= vecs_per_row) return;
     const int64_t e = static_cast<int64_t>(col) * 8;
