@@ -83,7 +83,9 @@ inline FastDiv fast_div(uint32_t d) {
     while ((1ull << shift) < d) ++shift;
     return FastDiv{static_cast<uint32_t>((((1ull << shift) - d) << 32) / d + 1), shift};
 }
-__device__ __forceinline__ uint32_t fast_quotient(uint32_t n, FastDiv d) { return (__umulhi(n, d.mul) + n) >> d.shift; }
+__host__ __device__ __forceinline__ uint32_t fast_quotient(uint32_t n, FastDiv d) {
+    return (static_cast<uint32_t>((static_cast<uint64_t>(n) * d.mul) >> 32) + n) >> d.shift;// the high half of a 32 x 32 bit product: one instruction
+}
 // two 4-byte kernel arguments that lie side by side, as one operand of AMD_ARGS_NOW
 __device__ __forceinline__ uint64_t arg_pair(uint32_t lo, uint32_t hi) { return lo | static_cast<uint64_t>(hi) << 32; }
 __device__ __forceinline__ uint64_t arg_pair(FastDiv f) { return arg_pair(f.mul, f.shift); }
