@@ -731,6 +731,8 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
             else RMS_ONCE_GO(1024, 1, 1, true, false);
             return;
         }
+        // (Wider rows in one pass with two vectors per lane: d = 16384 92.2 us against 93.9 us looping, and
+        // 105-111 us against 92-95 us at 9216-14336, where a third of the lanes has nothing to load.)
     }
 #undef RMS_ONCE
 #undef RMS_ONCE_GO
@@ -751,7 +753,13 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // so rows of up to 12 KiB get two workgroups per unit and longer ones one.
     uint64_t per_cu = d * sizeof(uint16_t) > 12 * 1024 ? 1 : 2;
     int home = kWLds;
-    if (lds_bytes > lds_limit || lds_bytes > 64 * 1024) {
+    // LDS holds up to 160 KiB per workgroup on gfx950 (rows of up to 40 704 elements); above 80 KiB only one
+    // workgroup fits a compute unit.  128 MiB of bf16 rows, weights in LDS against re-read through L2 per row:
+    //   d = 18432  48.0 / 58.8 us     d = 24576  48.0 / 55.1 us     d = 32768  49.5 / 54.3 us
+    // The fused form has no registers for a second row at these widths, and one workgroup per unit working
+    // one row at a time is slower than two that re-read the weights (d = 18432: 108.2 / 102.9 us,
+    // d = 24576: 102.3 / 96.7 us), so it keeps its weights in LDS up to 64 KiB only.
+    if (lds_bytes > lds_limit || (ADD && lds_bytes > 64 * 1024)) {
         home = kWGlobal;
         per_cu = 2;
     }

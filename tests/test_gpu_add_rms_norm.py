@@ -56,7 +56,9 @@ def check_y(got, want, dt, what, max_frac=5e-3):
                                  # short rows, several to a wavefront (per-head norms), with ragged last wavefronts
                                  (5001, 128), (1003, 64), (777, 256), (333, 72), (50, 200),
                                  # widths of common models on the looping kernels
-                                 (600, 5120), (530, 7168), (300, 12288)])
+                                 (600, 5120), (530, 7168), (300, 12288),
+                                 # rows whose fp32 weights take more than 64 KiB of LDS, and the first size beyond what LDS holds
+                                 (300, 18432), (270, 32768), (265, 40704), (262, 40960)])
 def test_against_oracle_and_against_the_two_separate_calls(ctx, dt, wdt, n, d):
     a, b, w = inputs(n, d, dt, wdt, n * 11 + d)
     want_c, want_y = oracle.add_rms_norm(a, b, w, 1e-5, dt, wdt)

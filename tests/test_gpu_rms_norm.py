@@ -53,6 +53,8 @@ def test_golden_odd_sizes(ctx):
                                  (1100, 4608), (300, 9216), (280, 11264), (290, 6656),
                                  # and two of them with an output large enough to be written through L2
                                  (5600, 6144), (4700, 7168),
+                                 # rows whose fp32 weights take more than 64 KiB of LDS (up to 160 KiB per workgroup), and the first size beyond
+                                 (300, 18432), (290, 20480), (280, 24576), (270, 32768), (265, 40704), (262, 40960),
                                  # short rows, several to a wavefront (per-head norms): full and ragged last wavefronts, rows that
                                  # do not fill their lanes, an output large enough to be written through L2
                                  (5001, 128), (4096, 128), (1003, 64), (777, 256), (333, 72), (101, 16), (50, 200), (270000, 128)])
