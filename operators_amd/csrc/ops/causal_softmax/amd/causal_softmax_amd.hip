@@ -268,7 +268,11 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     //   [2, 16384, 16384]  one per row 277-280, 64 per unit 282-284
     // so every row gets a workgroup of its own - the dispatcher then evens out
     // the causal triangle by itself - except rows of 512 elements and fewer,
-    // where a workgroup's start costs as much as its row.
+    // where a workgroup's start costs as much as its row.  Those short rows are bound by
+    // instruction issue, not by memory: about 220 vector instructions per row whatever part of
+    // it the mask keeps, four cycles each on a 16-lane SIMD ([2048, 512, 512] fp16: 374 us =
+    // 875 cycles per row and SIMD; the same bytes as [8192, 256, 256] take 735 us).  Asking
+    // for 2 or 4 rows per wavefront before working on the first moved that by -5 to +2 %.
     const uint64_t cap = nvec <= 64 ? static_cast<uint64_t>(d.cu_count) * 512 : rows;
     const uint64_t limit = amd::max_grid_1d(1024);// the kernel strides over what the grid does not cover
     const unsigned grid = static_cast<unsigned>(std::min({rows, cap, limit}));
