@@ -79,6 +79,7 @@ struct FastDiv {
 };
 constexpr uint64_t kFastDivLimit = 1ull << 31;// operands and divisors must be below this
 inline FastDiv fast_div(uint32_t d) {
+    if (d == 0) return FastDiv{0, 0};// nothing to divide by: the caller has no work to launch
     uint32_t shift = 0;
     while ((1ull << shift) < d) ++shift;
     return FastDiv{static_cast<uint32_t>((((1ull << shift) - d) << 32) / d + 1), shift};
