@@ -227,6 +227,150 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
     }
 }
 
+// Reductions over the P = 8, 16 or 32 lanes that share a short row: the first
+// steps of the wavefront trees (amd::wave_sum, amd::wave_max), stopped at the
+// group's width.  They combine the same values in the same order as the full
+// trees do when the lanes beyond the row hold zeros (or -inf for the maximum),
+// so a short row gets the bits it would get with a wavefront to itself.
+template<int P>
+__device__ __forceinline__ float segment_sum(float v) {
+    static_assert(P == 8 || P == 16 || P == 32, "lanes per row");
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));// quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));// quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));// row_half_mirror
+    if constexpr (P >= 16) {
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));// row_mirror
+    }
+    if constexpr (P == 32) v += __shfl_xor(v, 16);// the neighbouring row of 16 lanes
+    return v;
+}
+template<int P>
+__device__ __forceinline__ float segment_max(float v) {
+    static_assert(P == 8 || P == 16 || P == 32, "lanes per row");
+    int b = __builtin_bit_cast(int, v);
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0xB1, 0xF, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x4E, 0xF, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x141, 0xF, 0xF, false)));
+    if constexpr (P >= 16) {
+        b = __builtin_bit_cast(int, v);
+        v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x140, 0xF, 0xF, false)));
+    }
+    if constexpr (P == 32) v = fmaxf(v, __shfl_xor(v, 16));
+    return v;
+}
+
+// Rows of up to 256 elements: P lanes per row, one vector per lane, 64 / P
+// consecutive rows of one matrix per wavefront (the host takes this form when
+// the matrix has a multiple of 64 / P rows, so a wavefront never straddles two
+// matrices).  A row of the other kernel costs its wavefront about 220 vector
+// instructions however short it is; here that cost is shared by 2, 4 or 8 rows.
+// The arithmetic is causal_softmax_rows' with NV = 1, the kept length being a
+// per-lane value; the sums are the same trees (see segment_sum).
+template<typename T, int P, bool THROUGH>
+__global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint64_t groups, uint32_t seq, uint32_t total,
+                                                              int64_t stride_b, int64_t stride_i, FastDiv by_groups_per_matrix,
+                                                              uint32_t groups_per_matrix) {
+    AMD_ARGS_NOW(y, groups, seq, total, stride_b, stride_i, arg_pair(by_groups_per_matrix), groups_per_matrix, gridDim.x);
+    constexpr uint32_t RPW = kWave / P;// rows per wavefront
+    const uint32_t nvec = total / 8;
+    const uint32_t sub = threadIdx.x % P, rr = threadIdx.x / P;
+    const float neg_inf = -__builtin_inff();
+    for (uint64_t g = blockIdx.x; g < groups; g += gridDim.x) {
+        // group g of RPW rows: matrix b, rows i0 .. i0 + RPW - 1 (fewer than 2^31 groups, see FastDiv)
+        const uint32_t b = fast_quotient(static_cast<uint32_t>(g), by_groups_per_matrix);
+        const uint32_t i0 = (static_cast<uint32_t>(g) - b * groups_per_matrix) * RPW;
+        uint16_t *base = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i0) * stride_i;// the same for every lane
+        const uint32_t row_off = rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
+        const uint32_t keep = total - seq + i0 + rr + 1;
+        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = (keep - 1) / 8;
+        const u32x4 cur = ld16_stream(reinterpret_cast<const uint8_t *>(base) + row_off + (sub < last_vec ? sub : last_vec) * 16);
+        const bool straddles = tail != 0 && sub + 1 == keep_vecs;
+        const bool whole = sub < keep_vecs && !straddles;// every element of this lane's vector is kept
+
+        float mx = neg_inf, mn = __builtin_inff();
+        float f[8];
+        widen8<T>(cur, f);
+        if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+            if (straddles) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (static_cast<uint32_t>(e) < tail) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+                }
+            }
+        }
+        if (whole) {
+            if constexpr (T::kPackedMinMax) {
+                typename T::pair mx2 = T::as_pair(cur.x), mn2 = mx2;
+                const uint32_t w[3] = {cur.y, cur.z, cur.w};
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    mx2 = T::max2(mx2, T::as_pair(w[i]));
+                    mn2 = T::min2(mn2, T::as_pair(w[i]));
+                }
+                mx = fmaxf(T::first(mx2), T::second(mx2));
+                mn = fminf(T::first(mn2), T::second(mn2));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+            }
+        }
+        mx = segment_max<P>(mx);
+
+        const float lowest = mn - mx;// +inf - max for a lane without kept elements: passes the test below
+        const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
+        float part = 0.0f;
+        if (sub < keep_vecs) {
+            if (lean) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[e] = exp_nonpositive(f[e] - mx);
+            } else {
+                float slow[8];// an array of its own for the call: f stays in registers
+#pragma unroll
+                for (int e = 0; e < 8; ++e) slow[e] = f[e];
+                exp_any8(slow, mx);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[e] = slow[e];
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+            if (straddles) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[e] = static_cast<uint32_t>(e) < tail ? f[e] : 0.0f;
+            }
+        }
+        if (sub < keep_vecs) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) part += f[e];
+        }
+        const float sum = segment_sum<P>(part);
+        const float rcp = 1.0f / sum;
+
+        u32x4 packed{0, 0, 0, 0};
+        if (sub < keep_vecs) {
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float q = f[e] * rcp;
+                o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, f[e]), rcp, q);
+            }
+            packed = narrow8_unit_range<T>(o);
+        }
+        if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+            if (straddles) {// its masked tail is zero whatever the row turned into
+                uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (static_cast<uint32_t>(e) >= tail) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                }
+                packed = u32x4{w[0], w[1], w[2], w[3]};
+            }
+        }
+        if (sub < nvec) StreamOut<THROUGH>(base).st16(row_off + sub * 16, packed);
+    }
+}
+
 // Any row length, any alignment: three passes over the row with element
 // accesses; the later passes find the row in cache.
 template<typename T>
@@ -284,6 +428,35 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     }
     const bool through = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
     const FastDiv by_seq = fast_div(static_cast<uint32_t>(d.seq));
+    // Rows of up to 256 elements, several to a wavefront (see causal_softmax_short), when a matrix has a whole
+    // number of such groups of rows and a group lies within reach of a 32-bit byte offset from its first row.
+    // Measured on MI355X, fp16, one row per wavefront -> several:
+    //   [8192, 256, 256]  700 -> 338 us (bf16 633 -> 317)   [32768, 128, 128]  1385 -> 334 us   [131072, 64, 64]  2765 -> 324 us
+    // with 2048 wavefronts per compute unit striding over the groups (128 / 512 / 8192 per unit: 382 / 348 / 351 us at 256).
+    if (nvec <= 32 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
+        const unsigned lanes = nvec <= 8 ? 8 : (nvec <= 16 ? 16 : 32);
+        const unsigned rpw = kWave / lanes;
+        if (d.seq % rpw == 0) {
+            const uint64_t groups = rows / rpw;
+            const uint32_t gpm = static_cast<uint32_t>(d.seq / rpw);
+            const uint64_t capg = static_cast<uint64_t>(d.cu_count) * 2048;
+            const unsigned g = static_cast<unsigned>(std::min(groups, capg));
+#define CS_SHORT(P)                                                                                                            \
+    do {                                                                                                                       \
+        if (through)                                                                                                           \
+            causal_softmax_short<T, P, true><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
+                                                                      d.stride_b, d.stride_i, fast_div(gpm), gpm);             \
+        else                                                                                                                   \
+            causal_softmax_short<T, P, false><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
+                                                                       d.stride_b, d.stride_i, fast_div(gpm), gpm);            \
+    } while (0)
+            if (lanes == 8) CS_SHORT(8);
+            else if (lanes == 16) CS_SHORT(16);
+            else CS_SHORT(32);
+#undef CS_SHORT
+            return;
+        }
+    }
 #define CS_LAUNCH(BS, NV)                                                                                                      \
     do {                                                                                                                       \
         if (through)                                                                                                           \

@@ -51,6 +51,10 @@ CASES = [
     ((7, 13), None), ((5, 5), None), ((1, 8), None), ((3, 16, 16), None),
     ((2, 300, 4096), None), ((2, 64, 8192), None), ((1, 9, 32768), None), ((1, 5, 40000), None),
     ((4, 33, 1000), None), ((2, 128, 136), (128 * 144, 144, 1)), ((3, 10, 64), (1000, 65, 1)),
+    # rows of up to 256 elements, several to a wavefront: 8, 16 and 32 lanes per row, rows that do not fill their lanes, padded rows,
+    # a row count that is no multiple of the rows per wavefront (one row per wavefront again), more groups of rows than wavefronts
+    ((5, 64, 128), None), ((3, 100, 256), None), ((2, 30, 200), None), ((6, 24, 40), None), ((4, 16, 64), (16 * 80 + 8, 80, 1)),
+    ((3, 13, 64), None), ((300000, 16, 16), None), ((9, 256, 256), None),
 ]
 
 
@@ -97,6 +101,30 @@ def test_infinities_and_long_tails(ctx):
     got, _, _ = run(ctx, y, y.shape, None, "f16")
     check(got, want, "f16", "infinities and tails", max_frac=2e-2)
     assert np.isnan(oracle.decode(got, "f16")[0, 5, 0])
+
+
+def test_short_rows_give_the_bits_of_a_wavefront_per_row(ctx):
+    """Rows of up to 256 elements share a wavefront (8, 16 or 32 lanes each) when
+    the rows of a group lie within 2 GiB of each other; rows 256 MiB apart get a
+    wavefront each.  Both forms add in the same order: same data, same bits."""
+    import torch
+
+    for dt, tdt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
+        for total in (64, 128, 256):
+            seq = 8
+            rng = np.random.default_rng(900 + total)
+            vals = rng.standard_normal((1, seq, total)).astype(np.float32) * 3
+            vals[0, 2, 1] = -np.inf
+            vals[0, 5, :3] = 400.0
+            codes = oracle.encode(vals, dt)
+            dense = to_torch(codes, dt).reshape(1, seq, total)
+            far = torch.zeros(seq << 27, dtype=tdt, device="cuda").as_strided((1, seq, total), (seq << 27, 1 << 27, 1))
+            far.copy_(dense)
+            ctx.causal_softmax(dense)
+            ctx.causal_softmax(far)
+            torch.cuda.synchronize()
+            assert torch.equal(dense.view(torch.int16), far.contiguous().view(torch.int16)), (dt, total)
+            del far
 
 
 def test_status_codes_match_reference(ctx):
