@@ -65,6 +65,13 @@ SHAPES = [
     ((5, 6, 7, 8), (5, 6, 7, 8), (1,)),             # scalar-like operand
     ((3, 64, 64), (64,), (3, 64, 1)),               # a broadcast along leading dims, b along inner
     ((2, 3, 4, 5, 6, 8), (2, 1, 4, 1, 6, 8), (3, 1, 5, 1, 8)),  # six merged dims
+    # a whole tensor plus an operand broadcast along outer dimensions only, rows of whole wavefronts of vectors (the tiled form):
+    ((3, 5, 512), (3, 5, 512), (3, 1, 512)),        # a bias per batch entry
+    ((3, 5, 1024), (3, 1, 1024), (3, 5, 1024)),     # the same with the operands swapped, two tiles per row
+    ((2, 3, 4, 512), (2, 3, 4, 512), (2, 1, 4, 512)),  # an attention mask: the inner two dimensions merge
+    ((2, 3, 4, 512), (2, 3, 4, 512), (1, 3, 1, 512)),  # broadcast along two separate outer dimensions
+    ((2, 3, 2, 2, 3, 512), (2, 3, 2, 2, 3, 512), (2, 1, 2, 1, 3, 512)),  # and along alternating ones
+    ((70, 600, 512), (70, 600, 512), (70, 1, 512)), # large enough to be written through L2
 ]
 
 
