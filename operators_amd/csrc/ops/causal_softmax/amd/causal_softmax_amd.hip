@@ -261,17 +261,23 @@ __device__ __forceinline__ float segment_max(float v) {
     return v;
 }
 
-// Rows of up to 256 elements: P lanes per row, one vector per lane, 64 / P
-// consecutive rows of one matrix per wavefront (the host takes this form when
-// the matrix has a multiple of 64 / P rows, so a wavefront never straddles two
-// matrices).  A row of the other kernel costs its wavefront about 220 vector
-// instructions however short it is; here that cost is shared by 2, 4 or 8 rows.
-// The arithmetic is causal_softmax_rows' with NV = 1, the kept length being a
-// per-lane value; the sums are the same trees (see segment_sum).
-template<typename T, int P, bool THROUGH>
+// Rows of up to 512 elements: P lanes per row, NV vectors per lane (vector
+// sub + k * P for lane sub of the row), 64 / P consecutive rows of one matrix
+// per wavefront (the host takes this form when the matrix has a multiple of
+// 64 / P rows, so a wavefront never straddles two matrices).  A row of the
+// other kernel costs its wavefront about 220 vector instructions however short
+// it is and whatever part of it the mask keeps; here the fixed part of that is
+// shared by 2, 4 or 8 rows, and with two vectors per lane (rows of 257-512
+// elements, two to a wavefront) the second vector costs nothing while both
+// rows keep 256 columns or fewer.  The arithmetic is causal_softmax_rows', the
+// kept length being a per-lane value; the sums are the same trees, one per
+// vector index k, added in the order the whole-wavefront tree adds its halves
+// (see segment_sum).
+template<typename T, int P, int NV, bool THROUGH>
 __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint64_t groups, uint32_t seq, uint32_t total,
                                                               int64_t stride_b, int64_t stride_i, FastDiv by_groups_per_matrix,
                                                               uint32_t groups_per_matrix) {
+    static_assert(NV == 1 || NV == 2, "the sums of more vector indices would have to be added pairwise, as the whole-wavefront tree does");
     AMD_ARGS_NOW(y, groups, seq, total, stride_b, stride_i, arg_pair(by_groups_per_matrix), groups_per_matrix, gridDim.x);
     constexpr uint32_t RPW = kWave / P;// rows per wavefront
     const uint32_t nvec = total / 8;
@@ -285,89 +291,114 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
         const uint32_t row_off = rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
         const uint32_t keep = total - seq + i0 + rr + 1;
         const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = (keep - 1) / 8;
-        const u32x4 cur = ld16_stream(reinterpret_cast<const uint8_t *>(base) + row_off + (sub < last_vec ? sub : last_vec) * 16);
-        const bool straddles = tail != 0 && sub + 1 == keep_vecs;
-        const bool whole = sub < keep_vecs && !straddles;// every element of this lane's vector is kept
+        u32x4 cur[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = sub + k * P;
+            cur[k] = ld16_stream(reinterpret_cast<const uint8_t *>(base) + row_off + (v < last_vec ? v : last_vec) * 16);
+        }
 
         float mx = neg_inf, mn = __builtin_inff();
-        float f[8];
-        widen8<T>(cur, f);
-        if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
-            if (straddles) {
+        float f[NV][8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    if (static_cast<uint32_t>(e) < tail) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = sub + k * P;
+            if (k > 0 && __builtin_amdgcn_ballot_w64(v < keep_vecs) == 0) continue;// no row of this wavefront reaches that far
+            const bool straddles = tail != 0 && v + 1 == keep_vecs;
+            widen8<T>(cur[k], f[k]);
+            if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                if (straddles) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (static_cast<uint32_t>(e) < tail) mx = fmaxf(mx, f[k][e]), mn = fminf(mn, f[k][e]);
+                    }
                 }
             }
-        }
-        if (whole) {
-            if constexpr (T::kPackedMinMax) {
-                typename T::pair mx2 = T::as_pair(cur.x), mn2 = mx2;
-                const uint32_t w[3] = {cur.y, cur.z, cur.w};
+            if (v < keep_vecs && !straddles) {// every element of this vector is kept
+                if constexpr (T::kPackedMinMax) {
+                    typename T::pair mx2 = T::as_pair(cur[k].x), mn2 = mx2;
+                    const uint32_t w[3] = {cur[k].y, cur[k].z, cur[k].w};
 #pragma unroll
-                for (int i = 0; i < 3; ++i) {
-                    mx2 = T::max2(mx2, T::as_pair(w[i]));
-                    mn2 = T::min2(mn2, T::as_pair(w[i]));
+                    for (int i = 0; i < 3; ++i) {
+                        mx2 = T::max2(mx2, T::as_pair(w[i]));
+                        mn2 = T::min2(mn2, T::as_pair(w[i]));
+                    }
+                    mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
+                    mn = fminf(mn, fminf(T::first(mn2), T::second(mn2)));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[k][e]), mn = fminf(mn, f[k][e]);
                 }
-                mx = fmaxf(T::first(mx2), T::second(mx2));
-                mn = fminf(T::first(mn2), T::second(mn2));
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
             }
         }
         mx = segment_max<P>(mx);
 
         const float lowest = mn - mx;// +inf - max for a lane without kept elements: passes the test below
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
-        float part = 0.0f;
-        if (sub < keep_vecs) {
-            if (lean) {
+        float sum = 0.0f;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) f[e] = exp_nonpositive(f[e] - mx);
-            } else {
-                float slow[8];// an array of its own for the call: f stays in registers
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = sub + k * P;
+            if (k > 0 && __builtin_amdgcn_ballot_w64(v < keep_vecs) == 0) continue;// its sum would be an exact zero
+            const bool straddles = tail != 0 && v + 1 == keep_vecs;
+            if (v < keep_vecs) {
+                if (lean) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) slow[e] = f[e];
-                exp_any8(slow, mx);
+                    for (int e = 0; e < 8; ++e) f[k][e] = exp_nonpositive(f[k][e] - mx);
+                } else {
+                    float slow[8];// an array of its own for the call: f stays in registers
 #pragma unroll
-                for (int e = 0; e < 8; ++e) f[e] = slow[e];
+                    for (int e = 0; e < 8; ++e) slow[e] = f[k][e];
+                    exp_any8(slow, mx);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) f[k][e] = slow[e];
+                }
             }
-        }
-        if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
-            if (straddles) {
+            if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                if (straddles) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) f[e] = static_cast<uint32_t>(e) < tail ? f[e] : 0.0f;
+                    for (int e = 0; e < 8; ++e) f[k][e] = static_cast<uint32_t>(e) < tail ? f[k][e] : 0.0f;
+                }
             }
-        }
-        if (sub < keep_vecs) {
+            float part = 0.0f;
+            if (v < keep_vecs) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) part += f[e];
+                for (int e = 0; e < 8; ++e) part += f[k][e];
+            }
+            const float tree = segment_sum<P>(part);
+            sum = k == 0 ? tree : tree + sum;// the whole-wavefront tree adds the upper lanes' sum to the lower lanes'
         }
-        const float sum = segment_sum<P>(part);
         const float rcp = 1.0f / sum;
 
-        u32x4 packed{0, 0, 0, 0};
-        if (sub < keep_vecs) {
-            float o[8];
+        const StreamOut<THROUGH> out(base);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float q = f[e] * rcp;
-                o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, f[e]), rcp, q);
-            }
-            packed = narrow8_unit_range<T>(o);
-        }
-        if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
-            if (straddles) {// its masked tail is zero whatever the row turned into
-                uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = sub + k * P;
+            u32x4 packed{0, 0, 0, 0};
+            if (k == 0 || __builtin_amdgcn_ballot_w64(v < keep_vecs) != 0) {
+                const bool straddles = tail != 0 && v + 1 == keep_vecs;
+                if (v < keep_vecs) {
+                    float o[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    if (static_cast<uint32_t>(e) >= tail) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                    for (int e = 0; e < 8; ++e) {
+                        const float q = f[k][e] * rcp;
+                        o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, f[k][e]), rcp, q);
+                    }
+                    packed = narrow8_unit_range<T>(o);
                 }
-                packed = u32x4{w[0], w[1], w[2], w[3]};
+                if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                    if (straddles) {// its masked tail is zero whatever the row turned into
+                        uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            if (static_cast<uint32_t>(e) >= tail) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                        }
+                        packed = u32x4{w[0], w[1], w[2], w[3]};
+                    }
+                }
             }
+            if (v < nvec) out.st16(row_off + v * 16, packed);
         }
-        if (sub < nvec) StreamOut<THROUGH>(base).st16(row_off + sub * 16, packed);
     }
 }
 
@@ -428,31 +459,45 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     }
     const bool through = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
     const FastDiv by_seq = fast_div(static_cast<uint32_t>(d.seq));
-    // Rows of up to 256 elements, several to a wavefront (see causal_softmax_short), when a matrix has a whole
+    // Rows of up to 512 elements, several to a wavefront (see causal_softmax_short), when a matrix has a whole
     // number of such groups of rows and a group lies within reach of a 32-bit byte offset from its first row.
     // Measured on MI355X, fp16, one row per wavefront -> several:
-    //   [8192, 256, 256]  700 -> 338 us (bf16 633 -> 317)   [32768, 128, 128]  1385 -> 334 us   [131072, 64, 64]  2765 -> 324 us
-    // with 2048 wavefronts per compute unit striding over the groups (128 / 512 / 8192 per unit: 382 / 348 / 351 us at 256).
-    if (nvec <= 32 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
-        const unsigned lanes = nvec <= 8 ? 8 : (nvec <= 16 ? 16 : 32);
-        const unsigned rpw = kWave / lanes;
-        if (d.seq % rpw == 0) {
+    //   [2048, 512, 512]  374 -> 267 us (bf16 322 -> 260)   [8192, 256, 256]  700 -> 274 us
+    //   [32768, 128, 128]  1385 -> 291 us                    [131072, 64, 64]  2765 -> 324 us
+    // with 2048 wavefronts per compute unit striding over the groups (128 / 512 / 8192 per unit: 382 / 348 / 351 us
+    // at 256 columns with 32 lanes per row).
+    if (nvec <= 64 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
+        // The fewest lanes per row that hold it with one or two vectors each, among those whose rows per
+        // wavefront divide the matrix's row count: two vectors per lane halve the work of the rows that the
+        // mask cuts to half their length or less ([8192, 256, 256] fp16: 16 lanes x 2 vectors 274 us against
+        // 338 us with 32 x 1; [2048, 512, 512]: 32 x 2 267 us against 374 us with a wavefront per row).
+        unsigned lanes = 0, per_lane = 0;
+        for (const unsigned p : {8u, 16u, 32u}) {
+            for (const unsigned v : {1u, 2u}) {
+                if (lanes == 0 && p * v >= nvec && d.seq % (kWave / p) == 0) lanes = p, per_lane = v;
+            }
+        }
+        if (lanes != 0) {
+            const unsigned rpw = kWave / lanes;
             const uint64_t groups = rows / rpw;
             const uint32_t gpm = static_cast<uint32_t>(d.seq / rpw);
             const uint64_t capg = static_cast<uint64_t>(d.cu_count) * 2048;
             const unsigned g = static_cast<unsigned>(std::min(groups, capg));
-#define CS_SHORT(P)                                                                                                            \
+#define CS_SHORT(P, NV)                                                                                                        \
     do {                                                                                                                       \
         if (through)                                                                                                           \
-            causal_softmax_short<T, P, true><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
-                                                                      d.stride_b, d.stride_i, fast_div(gpm), gpm);             \
+            causal_softmax_short<T, P, NV, true><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
+                                                                          d.stride_b, d.stride_i, fast_div(gpm), gpm);         \
         else                                                                                                                   \
-            causal_softmax_short<T, P, false><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
-                                                                       d.stride_b, d.stride_i, fast_div(gpm), gpm);            \
+            causal_softmax_short<T, P, NV, false><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
+                                                                           d.stride_b, d.stride_i, fast_div(gpm), gpm);        \
     } while (0)
-            if (lanes == 8) CS_SHORT(8);
-            else if (lanes == 16) CS_SHORT(16);
-            else CS_SHORT(32);
+            if (lanes == 8 && per_lane == 1) CS_SHORT(8, 1);
+            else if (lanes == 8) CS_SHORT(8, 2);
+            else if (lanes == 16 && per_lane == 1) CS_SHORT(16, 1);
+            else if (lanes == 16) CS_SHORT(16, 2);
+            else if (per_lane == 1) CS_SHORT(32, 1);
+            else CS_SHORT(32, 2);
 #undef CS_SHORT
             return;
         }

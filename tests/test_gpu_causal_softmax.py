@@ -55,6 +55,8 @@ CASES = [
     # a row count that is no multiple of the rows per wavefront (one row per wavefront again), more groups of rows than wavefronts
     ((5, 64, 128), None), ((3, 100, 256), None), ((2, 30, 200), None), ((6, 24, 40), None), ((4, 16, 64), (16 * 80 + 8, 80, 1)),
     ((3, 13, 64), None), ((300000, 16, 16), None), ((9, 256, 256), None),
+    # rows of 257-512 elements, two to a wavefront with two vectors per lane: square, wide, ragged, padded, an odd number of rows
+    ((5, 512, 512), None), ((3, 40, 400), None), ((2, 300, 512), None), ((3, 64, 264), None), ((2, 16, 504), (16 * 520, 520, 1)), ((2, 33, 512), None),
 ]
 
 
@@ -104,13 +106,13 @@ def test_infinities_and_long_tails(ctx):
 
 
 def test_short_rows_give_the_bits_of_a_wavefront_per_row(ctx):
-    """Rows of up to 256 elements share a wavefront (8, 16 or 32 lanes each) when
+    """Rows of up to 512 elements share a wavefront (8, 16 or 32 lanes each) when
     the rows of a group lie within 2 GiB of each other; rows 256 MiB apart get a
     wavefront each.  Both forms add in the same order: same data, same bits."""
     import torch
 
     for dt, tdt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
-        for total in (64, 128, 256):
+        for total in (64, 72, 128, 136, 200, 256, 264, 384, 512):
             seq = 8
             rng = np.random.default_rng(900 + total)
             vals = rng.standard_normal((1, seq, total)).astype(np.float32) * 3
