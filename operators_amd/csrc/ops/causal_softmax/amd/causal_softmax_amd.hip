@@ -277,7 +277,7 @@ template<typename T, int P, int NV, bool THROUGH>
 __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint64_t groups, uint32_t seq, uint32_t total,
                                                               int64_t stride_b, int64_t stride_i, FastDiv by_groups_per_matrix,
                                                               uint32_t groups_per_matrix) {
-    static_assert(NV == 1 || NV == 2, "the sums of more vector indices would have to be added pairwise, as the whole-wavefront tree does");
+    static_assert(NV >= 1 && NV <= 3 && P * NV <= kWave, "up to three vector indices, added as the whole-wavefront tree adds them");
     AMD_ARGS_NOW(y, groups, seq, total, stride_b, stride_i, arg_pair(by_groups_per_matrix), groups_per_matrix, gridDim.x);
     constexpr uint32_t RPW = kWave / P;// rows per wavefront
     const uint32_t nvec = total / 8;
@@ -335,10 +335,11 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
 
         const float lowest = mn - mx;// +inf - max for a lane without kept elements: passes the test below
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
-        float sum = 0.0f;
+        float tree[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = sub + k * P;
+            tree[k] = 0.0f;
             if (k > 0 && __builtin_amdgcn_ballot_w64(v < keep_vecs) == 0) continue;// its sum would be an exact zero
             const bool straddles = tail != 0 && v + 1 == keep_vecs;
             if (v < keep_vecs) {
@@ -365,9 +366,12 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
 #pragma unroll
                 for (int e = 0; e < 8; ++e) part += f[k][e];
             }
-            const float tree = segment_sum<P>(part);
-            sum = k == 0 ? tree : tree + sum;// the whole-wavefront tree adds the upper lanes' sum to the lower lanes'
+            tree[k] = segment_sum<P>(part);
         }
+        // the order in which the whole-wavefront tree adds these groups of lanes: upper to lower, pairwise
+        float sum = tree[0];
+        if constexpr (NV == 2) sum = tree[1] + tree[0];
+        if constexpr (NV == 3) sum = tree[2] + (tree[1] + tree[0]);
         const float rcp = 1.0f / sum;
 
         const StreamOut<THROUGH> out(base);
@@ -467,14 +471,18 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     // with 2048 wavefronts per compute unit striding over the groups (128 / 512 / 8192 per unit: 382 / 348 / 351 us
     // at 256 columns with 32 lanes per row).
     if (nvec <= 64 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
-        // The fewest lanes per row that hold it with one or two vectors each, among those whose rows per
-        // wavefront divide the matrix's row count: two vectors per lane halve the work of the rows that the
-        // mask cuts to half their length or less ([8192, 256, 256] fp16: 16 lanes x 2 vectors 274 us against
-        // 338 us with 32 x 1; [2048, 512, 512]: 32 x 2 267 us against 374 us with a wavefront per row).
+        // Lanes per row x vectors per lane: the pair that wastes the fewest lanes, the fewer lanes per row (more
+        // rows per wavefront) when two waste the same, among those whose rows per wavefront divide the matrix's
+        // row count.  More than one vector per lane spares the rows that the mask cuts short the work of the
+        // vectors they do not reach.  Measured, fp16 (us):
+        //   [2048, 512, 512]   32 x 2  265   16 x 4  274          [8192, 256, 256]   16 x 2  274   32 x 1  344   8 x 4  286
+        //   [4096, 384, 384]   16 x 3  318   32 x 2  341          [32768, 128, 128]   8 x 2  296   16 x 1  344
+        //   [16384, 192, 192]  16 x 2  338    8 x 3  339   32 x 1  516
         unsigned lanes = 0, per_lane = 0;
         for (const unsigned p : {8u, 16u, 32u}) {
-            for (const unsigned v : {1u, 2u}) {
-                if (lanes == 0 && p * v >= nvec && d.seq % (kWave / p) == 0) lanes = p, per_lane = v;
+            for (const unsigned v : {1u, 2u, 3u}) {
+                const bool fits = p * v >= nvec && p * v <= kWave && d.seq % (kWave / p) == 0;
+                if (fits && (lanes == 0 || p * v < lanes * per_lane)) lanes = p, per_lane = v;
             }
         }
         if (lanes != 0) {
@@ -492,12 +500,16 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
             causal_softmax_short<T, P, NV, false><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
                                                                            d.stride_b, d.stride_i, fast_div(gpm), gpm);        \
     } while (0)
-            if (lanes == 8 && per_lane == 1) CS_SHORT(8, 1);
-            else if (lanes == 8) CS_SHORT(8, 2);
-            else if (lanes == 16 && per_lane == 1) CS_SHORT(16, 1);
-            else if (lanes == 16) CS_SHORT(16, 2);
-            else if (per_lane == 1) CS_SHORT(32, 1);
-            else CS_SHORT(32, 2);
+            switch (lanes * 10 + per_lane) {
+                case 81: CS_SHORT(8, 1); break;
+                case 82: CS_SHORT(8, 2); break;
+                case 83: CS_SHORT(8, 3); break;
+                case 161: CS_SHORT(16, 1); break;
+                case 162: CS_SHORT(16, 2); break;
+                case 163: CS_SHORT(16, 3); break;
+                case 321: CS_SHORT(32, 1); break;
+                default: CS_SHORT(32, 2); break;
+            }
 #undef CS_SHORT
             return;
         }

@@ -112,7 +112,7 @@ def test_short_rows_give_the_bits_of_a_wavefront_per_row(ctx):
     import torch
 
     for dt, tdt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
-        for total in (64, 72, 128, 136, 200, 256, 264, 384, 512):
+        for total in (64, 72, 128, 136, 192, 200, 256, 264, 320, 384, 512):
             seq = 8
             rng = np.random.default_rng(900 + total)
             vals = rng.standard_normal((1, seq, total)).astype(np.float32) * 3
