@@ -439,6 +439,7 @@ def ops_table(ctx, args, gen):
         "Q1 rms_norm bf16 [524288,128] w f32 (a per-head norm: 8192 tokens x 64 heads)": lambda: [make_rms_norm(ctx, 524288, 128, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * 524288 * 128, nset))],
         "N1 causal_softmax f16 [32,4096,4096]": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, f16, gen, "causal_softmax") for _ in range(2)],
         "N1b causal_softmax bf16 [32,4096,4096] (the Attention row's softmax on its own)": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, bf16, gen, "causal_softmax") for _ in range(2)],
+        "N1c causal_softmax f16 [2048,512,512] (short rows: two to a wavefront)": lambda: [make_causal_softmax(ctx, 2048, 512, 512, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
         # Not an operator of the library: a plain device-to-device copy of known
