@@ -319,6 +319,41 @@ __device__ __forceinline__ float wave_max(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// Reductions over groups of P = 8, 16 or 32 neighbouring lanes (short rows that
+// share a wavefront): the first steps of wave_sum and wave_max, stopped at the
+// group's width; every lane of a group ends up with the group's result.  They
+// combine the same values in the same order as the full trees do when the
+// lanes beyond the row hold zeros (or -inf for the maximum), so a short row
+// gets the bits it would get with a wavefront to itself.
+template<int P>
+__device__ __forceinline__ float segment_sum(float v) {
+    static_assert(P == 8 || P == 16 || P == 32, "lanes per row");
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));// quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));// quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));// row_half_mirror
+    if constexpr (P >= 16) {
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));// row_mirror
+    }
+    if constexpr (P == 32) v += __shfl_xor(v, 16);// the neighbouring row of 16 lanes
+    return v;
+}
+template<int P>
+__device__ __forceinline__ float segment_max(float v) {
+    static_assert(P == 8 || P == 16 || P == 32, "lanes per row");
+    int b = __builtin_bit_cast(int, v);
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0xB1, 0xF, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x4E, 0xF, 0xF, false)));
+    b = __builtin_bit_cast(int, v);
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x141, 0xF, 0xF, false)));
+    if constexpr (P >= 16) {
+        b = __builtin_bit_cast(int, v);
+        v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, 0x140, 0xF, 0xF, false)));
+    }
+    if constexpr (P == 32) v = fmaxf(v, __shfl_xor(v, 16));
+    return v;
+}
+
 // Maximum over a workgroup; same slot discipline as block_sum below.
 template<int WAVES>
 __device__ __forceinline__ float block_max(float v, float *slots, int phase) {

@@ -482,22 +482,9 @@ __global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t 
 // would leave most of a wavefront idle at one row each.  Here P = 8, 16 or 32
 // lanes serve a row, one vector per lane, and a wavefront takes 64 / P
 // consecutive rows; the sum of squares is the first steps of the wavefront
-// tree (amd::wave_sum), stopped at the group's width, which adds the same
-// values in the same order as the full tree would with zeros in the absent
-// lanes - so these rows, too, give the bits every other form gives.
-template<int P>
-__device__ __forceinline__ float segment_sum(float v) {
-    static_assert(P == 8 || P == 16 || P == 32, "lanes per row");
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));// quad_perm [1,0,3,2]
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));// quad_perm [2,3,0,1]
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));// row_half_mirror
-    if constexpr (P >= 16) {
-        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));// row_mirror
-    }
-    if constexpr (P == 32) v += __shfl_xor(v, 16);// the neighbouring row of 16 lanes
-    return v;
-}
-
+// tree (amd::segment_sum), which adds the same values in the same order as
+// the full tree would with zeros in the absent lanes - so these rows, too,
+// give the bits every other form gives.
 template<typename T, int P, bool THROUGH, bool ADD>
 __global__ __launch_bounds__(kWave) void rms_norm_short(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                         uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
