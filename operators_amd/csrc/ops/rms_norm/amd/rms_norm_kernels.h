@@ -738,7 +738,11 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     //   d =  7168:  45.6 / 47.0 / 46.3 / 47.4 us      d = 16384:  46.7 / 46.7 us
     //   d =  8192:  44.6 / 44.8 / 45.2 / 45.5 us
     // so rows of up to 12 KiB get two workgroups per unit and longer ones one.
+    // The two widths that split into 512-lane workgroups of whole vectors are the exception: two of those per
+    // unit measure the same or better than one (d = 8192: 43.7-44.6 against 44.3-44.7 us on two machines;
+    // d = 16384: 45.0-45.9 against 46.0-46.6 us).
     uint64_t per_cu = d * sizeof(uint16_t) > 12 * 1024 ? 1 : 2;
+    if (!ADD && (d == 8192 || d == 16384)) per_cu = 2;
     int home = kWLds;
     // LDS holds up to 160 KiB per workgroup on gfx950 (rows of up to 40 704 elements); above 80 KiB only one
     // workgroup fits a compute unit.  128 MiB of bf16 rows, weights in LDS against re-read through L2 per row:
