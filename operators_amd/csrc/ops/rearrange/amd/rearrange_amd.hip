@@ -161,7 +161,15 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         forward = forward && d.dst_stride[k] >= 0;
         dst_span += (d.shape[k] - 1) * static_cast<uint64_t>(d.dst_stride[k] >= 0 ? d.dst_stride[k] : 0);
     }
-    if (upr >= kWave && upr < (1ull << 31)) {
+    // Rows of fewer than 1024 units: single-wavefront tiles over the flat (row, unit) space, split by
+    // multiplication, measure the same or better than a 2-D grid of 128- or 256-lane row workgroups once the
+    // copy is large (bf16 rows out of a wider buffer, us: 64 units per row 21.4 against 29.6, 96 units 31.1
+    // against 34.0, 192 units 31.2 against 32.1, 384 units 31.6 against 32.6, 512 units 22.2 against 22.7,
+    // 352 units 16.2 both); a small copy of few rows is the exception (8192 rows of 128 units, 16 MiB: 9.5
+    // against 8.8), so rows of at least two wavefronts keep the row workgroups below 32 MiB.
+    const uint64_t units = desc.rows * upr;
+    const bool tiles = BYTES == 16 && units < kFastDivLimit && (upr < 2 * kWave || (upr < 16 * kWave && units * BYTES >= (32ull << 20)));
+    if (upr >= kWave && upr < (1ull << 31) && !tiles) {
         // A 2-D grid of single-wavefront workgroups needs at least 16 of them per
         // row.  Measured on MI355X with 128 MiB of fp16 rows: 16 KiB rows 41.3 us
         // with 64 lanes and 42.1 us with 256; 8 KiB rows (8 wavefronts each) 57.5

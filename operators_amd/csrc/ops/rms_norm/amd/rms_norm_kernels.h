@@ -743,8 +743,6 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // d = 16384: 45.0-45.9 against 46.0-46.6 us).
     uint64_t per_cu = d * sizeof(uint16_t) > 12 * 1024 ? 1 : 2;
     if (!ADD && (d == 8192 || d == 16384)) per_cu = 2;
-    if (getenv("RMS_PER_CU")) per_cu = atoi(getenv("RMS_PER_CU"));
-    const uint64_t lds_pad = getenv("RMS_LDS_PAD") ? atoi(getenv("RMS_LDS_PAD")) : 0;
     int home = kWLds;
     // LDS holds up to 160 KiB per workgroup on gfx950 (rows of up to 40 704 elements); above 80 KiB only one
     // workgroup fits a compute unit.  128 MiB of bf16 rows, weights in LDS against re-read through L2 per row:
@@ -808,10 +806,10 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
 #define RMS_EXACT(BS, NV, LANES)                                                                                       \
     do {                                                                                                               \
         if (through)                                                                                                   \
-            rms_norm_rows<T, BS, NV, kWLds, true, true, ADD><<<static_cast<unsigned>(grid), LANES, std::max(lds_bytes, lds_pad), stream>>>( \
+            rms_norm_rows<T, BS, NV, kWLds, true, true, ADD><<<static_cast<unsigned>(grid), LANES, lds_bytes, stream>>>( \
                 py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res); \
         else                                                                                                           \
-            rms_norm_rows<T, BS, NV, kWLds, true, false, ADD><<<static_cast<unsigned>(grid), LANES, std::max(lds_bytes, lds_pad), stream>>>( \
+            rms_norm_rows<T, BS, NV, kWLds, true, false, ADD><<<static_cast<unsigned>(grid), LANES, lds_bytes, stream>>>( \
                 py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, first_mul, hop, span, res); \
         return;                                                                                                        \
     } while (0)

@@ -88,9 +88,11 @@ __device__ __forceinline__ u32x4 swiglu8(u32x4 va, u32x4 vb) {
 template<typename Idx, bool ROWWISE>
 struct Where {
     Idx vecs_per_row;
+    FastDiv by_row;// division by vecs_per_row for 32-bit positions below kFastDivLimit
     __device__ __forceinline__ void split(uint64_t v, Idx &row, Idx &col) const {
         if constexpr (ROWWISE) {
-            row = static_cast<Idx>(v) / vecs_per_row;
+            if constexpr (sizeof(Idx) == 4) row = fast_quotient(static_cast<uint32_t>(v), by_row);
+            else row = static_cast<Idx>(v) / vecs_per_row;
             col = static_cast<Idx>(v) - row * vecs_per_row;
         } else {
             row = 0;
@@ -108,9 +110,9 @@ struct Where {
 template<typename T, typename Idx, bool ROWWISE>
 __global__ __launch_bounds__(kWave) void swiglu_vec(uint16_t *c, const uint16_t *a, const uint16_t *b,
                                                      uint64_t nvec, Idx vecs_per_row,
-                                                     int64_t stride_c, int64_t stride_a, int64_t stride_b) {
-    AMD_ARGS_NOW(c, a, b, nvec, vecs_per_row, stride_c, stride_a, stride_b, gridDim.x);
-    const Where<Idx, ROWWISE> where{vecs_per_row};
+                                                     int64_t stride_c, int64_t stride_a, int64_t stride_b, FastDiv by_row) {
+    AMD_ARGS_NOW(c, a, b, nvec, vecs_per_row, stride_c, stride_a, stride_b, arg_pair(by_row), gridDim.x);
+    const Where<Idx, ROWWISE> where{vecs_per_row, by_row};
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kWave;
     for (uint64_t v = static_cast<uint64_t>(blockIdx.x) * kWave + threadIdx.x; v < nvec; v += step) {
         Idx row, col;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(kWave) void swiglu_vec(uint16_t *c, const uint16_t 
     }
 }
 
-// Row-strided tensors whose rows hold at least a wavefront of vectors:
+// Row-strided tensors whose rows hold at least 16 wavefronts of vectors:
 // blockIdx.y walks the rows and blockIdx.x the row's vectors, so no lane
 // divides anything and no workgroup straddles two rows.
 template<typename T, int LANES>
@@ -180,35 +182,26 @@ void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const v
     // One row, or every row stride equal to the width: the tensors are dense.
     const bool dense = d.rows == 1 || (d.stride_a == di && d.stride_b == di && d.stride_c == di);
     const bool small = nvec < (1ull << 31);
-    // Measured at [8192, 28672] bf16 from a fused [8192, 57344] buffer: the row
-    // form is 4 % faster than the flat index split by division.
-    if (!dense && vpr >= kWave && vpr < (1ull << 31)) {
+    // Row-strided tensors (the halves of a fused gate/up buffer).  Rows of at least 1024 vectors: a 2-D grid of
+    // single-wavefront workgroups, no lane divides anything.  Shorter rows: the same tiles over the flat (row,
+    // vector) space, split by a multiplication (see FastDiv) - a 2-D grid of single wavefronts needs at least 16
+    // of them per row, and the 128- or 256-lane row workgroups it would take instead measure the same or worse
+    // (bf16 from a fused buffer, us: [131072, 512] 60.3 against 69.4, [16384, 4096] 60.9 against 62.5,
+    // [65536, 1024] 60.2 against 61.6, [23831, 2816] 60.7 against 60.2; at [8192, 28672] the two forms are
+    // level, 204.8 and 204.4, where the split by a run-time division cost the flat form 4 %).
+    if (!dense && vpr >= 16 * kWave && vpr < (1ull << 31)) {
         const unsigned gy = static_cast<unsigned>(d.rows < 65535 ? d.rows : 65535);
-        // A 2-D grid of single-wavefront workgroups needs at least 16 of them per
-        // row; with fewer (rows under 8192 elements) it is up to 40 % slower than
-        // 256-lane workgroups (measured with a strided copy of the same shape).
-        if (vpr >= 16 * kWave) {
-            swiglu_rows<T, kWave><<<dim3(static_cast<unsigned>(ceil_div(vpr, kWave)), gy), kWave, 0, stream>>>(
-                pc, pa, pb, d.rows, static_cast<uint32_t>(vpr), d.stride_c, d.stride_a, d.stride_b);
-        } else if (ceil_div(vpr, 128) * 128 < ceil_div(vpr, kBlock) * kBlock) {
-            // the row fills 128-lane workgroups better than 256-lane ones: [23831, 2816] bf16 from a fused
-            // buffer (352 vectors per row) 60.7 us against 70.0 us, 6912 wide 61.1 against 64.5, 7168 wide
-            // 61.8 against 64.3; where both fit equally there is nothing between them
-            swiglu_rows<T, 128><<<dim3(static_cast<unsigned>(ceil_div(vpr, 128)), gy), 128, 0, stream>>>(
-                pc, pa, pb, d.rows, static_cast<uint32_t>(vpr), d.stride_c, d.stride_a, d.stride_b);
-        } else {
-            swiglu_rows<T, kBlock><<<dim3(static_cast<unsigned>(ceil_div(vpr, kBlock)), gy), kBlock, 0, stream>>>(
-                pc, pa, pb, d.rows, static_cast<uint32_t>(vpr), d.stride_c, d.stride_a, d.stride_b);
-        }
+        swiglu_rows<T, kWave><<<dim3(static_cast<unsigned>(ceil_div(vpr, kWave)), gy), kWave, 0, stream>>>(
+            pc, pa, pb, d.rows, static_cast<uint32_t>(vpr), d.stride_c, d.stride_a, d.stride_b);
         return;
     }
     if (dense) {
-        swiglu_vec<T, uint64_t, false><<<grid, kWave, 0, stream>>>(pc, pa, pb, nvec, vpr, d.stride_c, d.stride_a, d.stride_b);
+        swiglu_vec<T, uint64_t, false><<<grid, kWave, 0, stream>>>(pc, pa, pb, nvec, vpr, d.stride_c, d.stride_a, d.stride_b, FastDiv{});
     } else if (small) {
         swiglu_vec<T, uint32_t, true><<<grid, kWave, 0, stream>>>(pc, pa, pb, nvec, static_cast<uint32_t>(vpr),
-                                                                   d.stride_c, d.stride_a, d.stride_b);
+                                                                   d.stride_c, d.stride_a, d.stride_b, fast_div(static_cast<uint32_t>(vpr)));
     } else {
-        swiglu_vec<T, uint64_t, true><<<grid, kWave, 0, stream>>>(pc, pa, pb, nvec, vpr, d.stride_c, d.stride_a, d.stride_b);
+        swiglu_vec<T, uint64_t, true><<<grid, kWave, 0, stream>>>(pc, pa, pb, nvec, vpr, d.stride_c, d.stride_a, d.stride_b, FastDiv{});
     }
 }
 
