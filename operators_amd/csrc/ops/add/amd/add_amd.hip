@@ -100,31 +100,37 @@ struct BcastDims {
     uint64_t shape[kAddMaxDims];
     int64_t a_stride[kAddMaxDims];
     int64_t b_stride[kAddMaxDims];
+    FastDiv by_shape[kAddMaxDims];// division by shape[k], k >= 1, for the kernels that number positions with 32 bits
 };
 
-// All of a BcastDims argument as operands of AMD_ARGS_NOW (25 of the 30 an asm statement takes).
-#define ARGS_OF_BCAST(d)                                                                                                                       \
-    d.ndim, d.shape[0], d.shape[1], d.shape[2], d.shape[3], d.shape[4], d.shape[5], d.shape[6], d.shape[7], d.a_stride[0], d.a_stride[1],     \
-        d.a_stride[2], d.a_stride[3], d.a_stride[4], d.a_stride[5], d.a_stride[6], d.a_stride[7], d.b_stride[0], d.b_stride[1], d.b_stride[2], \
-        d.b_stride[3], d.b_stride[4], d.b_stride[5], d.b_stride[6], d.b_stride[7]
-static_assert(kAddMaxDims == 8, "ARGS_OF_BCAST lists eight dimensions");
+// The innermost four dimensions of a BcastDims argument as operands of AMD_ARGS_NOW (what nearly every
+// broadcast has after merging; the rest are fetched when a fifth dimension is met).
+#define ARGS_OF_BCAST(d)                                                                                                               \
+    d.ndim, d.shape[0], d.shape[1], d.shape[2], d.shape[3], d.a_stride[0], d.a_stride[1], d.a_stride[2], d.a_stride[3], d.b_stride[0], \
+        d.b_stride[1], d.b_stride[2], d.b_stride[3], arg_pair(d.by_shape[1]), arg_pair(d.by_shape[2]), arg_pair(d.by_shape[3])
 
 // Split a flat position (in units of `first_extent` along the innermost
-// dimension) into operand offsets.  Idx is 32-bit when every quantity fits,
-// which keeps the divisions cheap.
+// dimension) into operand offsets.  Idx is 32-bit when every quantity is
+// below 2^31, and the divisions are then multiplications (see FastDiv).
 template<typename Idx>
-__device__ __forceinline__ void bcast_offsets(const BcastDims &d, Idx pos, Idx inner_extent, int64_t inner_scale,
+__device__ __forceinline__ void bcast_offsets(const BcastDims &d, Idx pos, Idx inner_extent, FastDiv by_inner, int64_t inner_scale,
                                               int64_t &off_a, int64_t &off_b) {
-    const Idx in = pos % inner_extent;
-    Idx rest = pos / inner_extent;
+    constexpr bool FAST = sizeof(Idx) == 4;
+    Idx rest;
+    if constexpr (FAST) rest = fast_quotient(static_cast<uint32_t>(pos), by_inner);
+    else rest = pos / inner_extent;
+    const Idx in = pos - rest * inner_extent;
     off_a = static_cast<int64_t>(in) * inner_scale * d.a_stride[0];
     off_b = static_cast<int64_t>(in) * inner_scale * d.b_stride[0];
 #pragma unroll
     for (int k = 1; k < kAddMaxDims; ++k) {
         if (k < d.ndim) {
             const Idx ext = static_cast<Idx>(d.shape[k]);
-            const Idx i = rest % ext;
-            rest /= ext;
+            Idx q;
+            if constexpr (FAST) q = fast_quotient(static_cast<uint32_t>(rest), d.by_shape[k]);
+            else q = rest / ext;
+            const Idx i = rest - q * ext;
+            rest = q;
             off_a += static_cast<int64_t>(i) * d.a_stride[k];
             off_b += static_cast<int64_t>(i) * d.b_stride[k];
         }
@@ -152,13 +158,13 @@ __device__ __forceinline__ u32x4 fetch_operand(const typename Op::scalar *p, uin
 // stands still (one element, replicated).
 template<typename Op, typename Idx, int A_MODE, int B_MODE>
 __global__ __launch_bounds__(kBlock) void add_bcast_vec(u32x4 *c, const typename Op::scalar *a,
-                                                        const typename Op::scalar *b, BcastDims d, uint64_t nvec) {
-    AMD_ARGS_NOW(c, a, b, nvec, gridDim.x, ARGS_OF_BCAST(d));
+                                                        const typename Op::scalar *b, BcastDims d, uint64_t nvec, FastDiv by_inner) {
+    AMD_ARGS_NOW(c, a, b, nvec, gridDim.x, arg_pair(by_inner), ARGS_OF_BCAST(d));
     const Idx inner_vecs = static_cast<Idx>(d.shape[0] / Op::kPerVec);
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
     for (uint64_t v = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; v < nvec; v += step) {
         int64_t oa = 0, ob = 0;
-        bcast_offsets<Idx>(d, static_cast<Idx>(v), inner_vecs, Op::kPerVec, oa, ob);
+        bcast_offsets<Idx>(d, static_cast<Idx>(v), inner_vecs, by_inner, Op::kPerVec, oa, ob);
         const u32x4 va = fetch_operand<Op, A_MODE>(a, v, oa);
         const u32x4 vb = fetch_operand<Op, B_MODE>(b, v, ob);
         st16_stream(c + v, Op::vec(va, vb));
@@ -262,13 +268,13 @@ __global__ __launch_bounds__(kWave) void add_bcast_tiles(u32x4 *c, const u32x4 *
 // Element form: any strides.
 template<typename Op, typename Idx>
 __global__ __launch_bounds__(kBlock) void add_bcast_scalar(typename Op::scalar *c, const typename Op::scalar *a,
-                                                           const typename Op::scalar *b, BcastDims d, uint64_t n) {
-    AMD_ARGS_NOW(c, a, b, n, gridDim.x, ARGS_OF_BCAST(d));
+                                                           const typename Op::scalar *b, BcastDims d, uint64_t n, FastDiv by_inner) {
+    AMD_ARGS_NOW(c, a, b, n, gridDim.x, arg_pair(by_inner), ARGS_OF_BCAST(d));
     const Idx inner = static_cast<Idx>(d.shape[0]);
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
     for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += step) {
         int64_t oa, ob;
-        bcast_offsets<Idx>(d, static_cast<Idx>(i), inner, 1, oa, ob);
+        bcast_offsets<Idx>(d, static_cast<Idx>(i), inner, by_inner, 1, oa, ob);
         c[i] = Op::one(a[oa], b[ob]);
     }
 }
@@ -314,6 +320,7 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         d.shape[k] = k < desc.ndim ? desc.shape[k] : 1;
         d.a_stride[k] = k < desc.ndim ? desc.a_stride[k] : 0;
         d.b_stride[k] = k < desc.ndim ? desc.b_stride[k] : 0;
+        d.by_shape[k] = fast_div(small ? static_cast<uint32_t>(d.shape[k]) : 1);
     }
 
     // 128-bit access needs: inner extent a multiple of the vector width, inner
@@ -340,8 +347,9 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
             return static_cast<int>(kFull);
         };
         const int ma = mode_of(desc.a_stride), mb = mode_of(desc.b_stride);
-        auto go = [&](auto kernel) {
-            kernel<<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const S *>(a), static_cast<const S *>(b), d, nvec);
+        auto go = [&](auto kernel) {// (single-wavefront tiles measure 1-3 % slower here: the operand that stands still is a 2-byte load per lane)
+            kernel<<<grid, kBlock, 0, stream>>>(static_cast<u32x4 *>(c), static_cast<const S *>(a), static_cast<const S *>(b), d, nvec,
+                                                fast_div(small ? static_cast<uint32_t>(desc.shape[0] / w) : 1));
         };
         // rows form: two merged dimensions with at least a wavefront of vectors in the inner one
         const uint64_t inner_vecs = desc.shape[0] / w;
@@ -423,10 +431,10 @@ infiniopStatus_t launch_add(const AddAmdDescriptor &desc, void *c, const void *a
         const unsigned grid = grid_for(n, kBlock, cus, 64);
         if (small) {
             add_bcast_scalar<Op, uint32_t><<<grid, kBlock, 0, stream>>>(static_cast<S *>(c), static_cast<const S *>(a),
-                                                                        static_cast<const S *>(b), d, n);
+                                                                        static_cast<const S *>(b), d, n, fast_div(static_cast<uint32_t>(desc.shape[0])));
         } else {
             add_bcast_scalar<Op, uint64_t><<<grid, kBlock, 0, stream>>>(static_cast<S *>(c), static_cast<const S *>(a),
-                                                                        static_cast<const S *>(b), d, n);
+                                                                        static_cast<const S *>(b), d, n, FastDiv{});
         }
     }
     return STATUS_SUCCESS;
