@@ -46,12 +46,12 @@ template<> struct Unit<2> { typedef uint16_t type; };
 template<> struct Unit<1> { typedef uint8_t type; };
 
 // blockIdx.y walks the rows, blockIdx.x the units of a row: rows of at least a
-// wavefront of units.  The row's offsets are found by dividing the row number
+// wavefront of units.  The row's offsets are found by splitting the row number
 // by the merged outer extents - once per workgroup row, on the scalar unit,
-// since the row number is uniform.
+// since the row number is uniform, and by multiplication (see FastDiv).
 // BUFST (16-byte units, large outputs): stores are written through L2 as
 // buffer stores relative to the start of the destination row (see StreamOut).
-template<int BYTES, bool BUFST, int LANES, bool FAST>
+template<int BYTES, bool BUFST, int LANES>
 __global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row) {
     typedef typename Unit<BYTES>::type U;
     // every argument up front (see AMD_ARGS_NOW; the number of rows to step by is not needed before the first load is out)
@@ -60,28 +60,15 @@ __global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint
     if (col >= units_per_row) return;
     for (uint64_t r = blockIdx.y; r < rows; r += gridDim.y) {
         int64_t od = 0, os = 0;
-        if constexpr (FAST) {// fewer than 2^31 rows: multiplications instead of divisions
-            uint32_t rest = static_cast<uint32_t>(r);
+        uint32_t rest = static_cast<uint32_t>(r);// fewer than 2^31 rows (the host sends more to rearrange_flat): see FastDiv
 #pragma unroll
-            for (int k = 0; k < kRearrangeMaxDims; ++k) {
-                if (k < d.ndim) {
-                    const uint32_t q = fast_quotient(rest, d.by_shape[k]);
-                    const uint32_t i = rest - q * d.shape[k];
-                    rest = q;
-                    od += static_cast<int64_t>(i) * d.dst_stride[k];
-                    os += static_cast<int64_t>(i) * d.src_stride[k];
-                }
-            }
-        } else {
-            uint64_t rest = r;
-#pragma unroll
-            for (int k = 0; k < kRearrangeMaxDims; ++k) {
-                if (k < d.ndim) {
-                    const uint64_t i = rest % d.shape[k];
-                    rest /= d.shape[k];
-                    od += static_cast<int64_t>(i) * d.dst_stride[k];
-                    os += static_cast<int64_t>(i) * d.src_stride[k];
-                }
+        for (int k = 0; k < kRearrangeMaxDims; ++k) {
+            if (k < d.ndim) {
+                const uint32_t q = fast_quotient(rest, d.by_shape[k]);
+                const uint32_t i = rest - q * d.shape[k];
+                rest = q;
+                od += static_cast<int64_t>(i) * d.dst_stride[k];
+                os += static_cast<int64_t>(i) * d.src_stride[k];
             }
         }
         const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
@@ -169,7 +156,7 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
     // against 8.8), so rows of at least two wavefronts keep the row workgroups below 32 MiB.
     const uint64_t units = desc.rows * upr;
     const bool tiles = BYTES == 16 && units < kFastDivLimit && (upr < 2 * kWave || (upr < 16 * kWave && units * BYTES >= (32ull << 20)));
-    if (upr >= kWave && upr < (1ull << 31) && !tiles) {
+    if (upr >= kWave && upr < (1ull << 31) && !tiles && desc.rows < kFastDivLimit) {
         // A 2-D grid of single-wavefront workgroups needs at least 16 of them per
         // row.  Measured on MI355X with 128 MiB of fp16 rows: 16 KiB rows 41.3 us
         // with 64 lanes and 42.1 us with 256; 8 KiB rows (8 wavefronts each) 57.5
@@ -182,22 +169,22 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         const int lanes = wave_rows ? kWave : (half ? 128 : 256);
         const dim3 grid(static_cast<unsigned>(ceil_div(upr, lanes)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
         const bool bufst = BYTES == 16 && large && desc.row_bytes < (1ull << 32);
-        const bool fast = desc.rows < kFastDivLimit;
         const uint32_t upr32 = static_cast<uint32_t>(upr);
-#define REARRANGE_ROWS(BUFST, LANES, FAST) rearrange_rows<BYTES, BUFST, LANES, FAST><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32)
-#define REARRANGE_ROWS_OF(LANES)                                      \
-    do {                                                              \
-        if (bufst && fast) REARRANGE_ROWS(BYTES == 16, LANES, true);  \
-        else if (bufst) REARRANGE_ROWS(BYTES == 16, LANES, false);    \
-        else if (fast) REARRANGE_ROWS(false, LANES, true);            \
-        else REARRANGE_ROWS(false, LANES, false);                     \
+#define REARRANGE_ROWS_OF(LANES)                                                                                           \
+    do {                                                                                                                   \
+        if (bufst) rearrange_rows<BYTES, BYTES == 16, LANES><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32);     \
+        else rearrange_rows<BYTES, false, LANES><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32);                 \
     } while (0)
-        if (wave_rows) REARRANGE_ROWS_OF(kWave);
-        else if (half) REARRANGE_ROWS_OF(128);
+        if constexpr (BYTES == 16) {
+            if (wave_rows) {
+                REARRANGE_ROWS_OF(kWave);
+                return;
+            }
+        }
+        if (half) REARRANGE_ROWS_OF(128);
         else REARRANGE_ROWS_OF(256);
 #undef REARRANGE_ROWS_OF
-#undef REARRANGE_ROWS
-    } else {// short rows, or a single row too long for 32-bit column numbers
+    } else {// short rows; or more rows, or a longer row, than 32 bits number (divisions, 64-bit)
         const uint64_t total = desc.rows * upr;
         const uint64_t want = ceil_div(total, kBlock);
         const uint64_t blocks = want < max_grid_1d(kBlock) ? want : max_grid_1d(kBlock);
@@ -207,9 +194,6 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
             const FastDiv by_row = fast_div(static_cast<uint32_t>(upr));
             if (bufst) rearrange_flat<BYTES, uint32_t, BYTES == 16, true><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row);
             else rearrange_flat<BYTES, uint32_t, false, true><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row);
-        } else if (total < (1ull << 32)) {
-            if (bufst) rearrange_flat<BYTES, uint32_t, BYTES == 16, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), FastDiv{});
-            else rearrange_flat<BYTES, uint32_t, false, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), FastDiv{});
         } else {
             rearrange_flat<BYTES, uint64_t, false, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, upr, FastDiv{});
         }

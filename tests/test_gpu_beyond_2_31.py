@@ -109,6 +109,22 @@ def test_rearrange_tokens_to_heads(ctx):
     assert not wide[:, heads:].any()
 
 
+def test_rearrange_more_than_2_to_31_units(ctx):
+    """Rows of 33 bytes out of rows of 40: one-byte units, and more than 2^31 of
+    them, so positions are split with 64-bit divisions."""
+    import torch
+
+    rows, width, pitch = (1 << 26) + 5, 33, 40
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    src = torch.randint(-128, 128, (rows, pitch), generator=g, device="cuda", dtype=torch.int8)
+    dst = torch.zeros((rows, width), dtype=torch.int8, device="cuda")
+    ctx.rearrange(dst, src[:, :width])
+    torch.cuda.synchronize()
+    for r0 in range(0, rows, 1 << 23):  # in slabs to bound memory
+        assert torch.equal(dst[r0:r0 + (1 << 23)], src[r0:r0 + (1 << 23), :width]), r0
+
+
 @pytest.mark.parametrize("heads", [128, 8])
 def test_rope_in_place(ctx, heads):
     import torch
