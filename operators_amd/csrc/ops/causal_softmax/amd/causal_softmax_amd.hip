@@ -372,6 +372,135 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
     }
 }
 
+// Rows longer than a workgroup can hold in registers (more than 32 768
+// elements), 16-byte aligned: three passes over the row with 16-byte accesses
+// - the maximum (and the minimum, for the choice of exponential), the sum of
+// the exponentials, the quotients - UNROLL vectors per lane in flight at a
+// time.  The first pass brings the row in from memory; the other two find it
+// in L2 or in the Infinity Cache, so the exponentials are formed twice but
+// memory is read once.  Masked vectors are written as zeros without being
+// read.  One workgroup per row at a time.
+template<typename T, int BS, bool THROUGH>
+__global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
+                                                          int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
+    AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
+    constexpr int WAVES = BS / kWave, UNROLL = 4;
+    __shared__ float red[4 * WAVES];
+    const uint32_t nvec = total / 8;
+    int phase = 0;
+    for (uint64_t r = blockIdx.x; r < rows; r += gridDim.x, phase ^= 1) {
+        const uint32_t b = fast_quotient(static_cast<uint32_t>(r), by_seq), i = static_cast<uint32_t>(r) - b * seq;// fewer than 2^31 rows (see FastDiv)
+        uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
+        const uint32_t keep = total - seq + i + 1;
+        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u;
+        const uint32_t whole_vecs = keep / 8;// vectors all of whose elements are kept
+
+        // pass 1: maximum and minimum of the kept elements
+        float mx = -__builtin_inff(), mn = __builtin_inff();
+        for (uint32_t v0 = threadIdx.x; v0 < keep_vecs; v0 += BS * UNROLL) {
+            u32x4 x[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t v = v0 + u * BS;
+                x[u] = ld16(row + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);// re-reading the last kept vector changes no maximum
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t v = v0 + u * BS;
+                float f[8];
+                widen8<T>(x[u], f);
+                const uint32_t got = v < keep_vecs ? v : keep_vecs - 1;// the vector that was read
+                const uint32_t lim = got < whole_vecs ? 8u : tail;     // its kept elements (beyond the whole vectors there is only the straddling one)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (static_cast<uint32_t>(e) < lim) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+                }
+            }
+        }
+        mx = block_max<WAVES>(mx, red, phase);
+        const float lowest = mn - mx;
+        const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
+
+        // exp(x - max) of one vector, zero where the mask cuts it
+        auto exps = [&](u32x4 x, uint32_t v, float(&e8)[8]) {
+            widen8<T>(x, e8);
+            if (lean) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) e8[e] = exp_nonpositive(e8[e] - mx);
+            } else {
+                float slow[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) slow[e] = e8[e];
+                exp_any8(slow, mx);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) e8[e] = slow[e];
+            }
+            if (v >= whole_vecs) {// the straddling vector
+#pragma unroll
+                for (int e = 0; e < 8; ++e) e8[e] = static_cast<uint32_t>(e) < tail ? e8[e] : 0.0f;
+            }
+        };
+
+        // pass 2: the sum, each lane over its vectors in ascending order, then the workgroup tree
+        float part = 0.0f;
+        for (uint32_t v0 = threadIdx.x; v0 < keep_vecs; v0 += BS * UNROLL) {
+            u32x4 x[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t v = v0 + u * BS;
+                x[u] = ld16(row + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t v = v0 + u * BS;
+                if (v < keep_vecs) {
+                    float e8[8];
+                    exps(x[u], v, e8);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) part += e8[e];
+                }
+            }
+        }
+        const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
+        const float rcp = 1.0f / sum;
+
+        // pass 3: the quotients, and zeros behind them
+        const StreamOut<THROUGH> out(row);
+        for (uint32_t v0 = threadIdx.x; v0 < nvec; v0 += BS * UNROLL) {
+            u32x4 x[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t v = v0 + u * BS;
+                x[u] = ld16(row + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t v = v0 + u * BS;
+                u32x4 packed{0, 0, 0, 0};
+                if (v < keep_vecs) {
+                    float e8[8], o[8];
+                    exps(x[u], v, e8);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float q = e8[e] * rcp;
+                        o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, e8[e]), rcp, q);
+                    }
+                    packed = narrow8_unit_range<T>(o);
+                    if (v >= whole_vecs) {// its masked tail is zero whatever the row turned into
+                        uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            if (static_cast<uint32_t>(e) >= tail) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                        }
+                        packed = u32x4{w[0], w[1], w[2], w[3]};
+                    }
+                }
+                if (v < nvec) out.st16(v * 16, packed);
+            }
+        }
+    }
+}
+
 // Any row length, any alignment: three passes over the row with element
 // accesses; the later passes find the row in cache.
 template<typename T>
@@ -423,6 +552,22 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const unsigned grid = static_cast<unsigned>(std::min({rows, cap, limit}));
 
     const bool vec_ok = d.total % 8 == 0 && nvec <= 4096 && d.seq < (1ull << 31) && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);
+    const bool long_ok = d.total % 8 == 0 && nvec > 4096 && d.total < (1ull << 31) && rows < kFastDivLimit && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 &&
+                         aligned16(data) && d.total * 2 < (1ull << 32);
+    if (long_ok) {
+        const bool thr = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
+        const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
+        // 1024 lanes take 4096 vectors a turn: rows of fewer than two turns are better served by 512 ([64, 512, 40000] fp16
+        // 1293 against 1584 us; [64, 512, 65536] 2320 against 2171 us; 256 lanes: 1451 and 2394 us)
+        const int lanes = nvec < 8192 ? 512 : 1024;
+        const unsigned g = static_cast<unsigned>(std::min<uint64_t>(rows, amd::max_grid_1d(1024)));
+#define CS_LONG(BS) do { if (thr) causal_softmax_long<T, BS, true><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by); \
+                         else causal_softmax_long<T, BS, false><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by); } while (0)
+        if (lanes == 512) CS_LONG(512);
+        else CS_LONG(1024);
+#undef CS_LONG
+        return;
+    }
     if (!vec_ok) {
         causal_softmax_generic<T><<<grid, 256, 0, stream>>>(py, rows, d.seq, d.total, d.stride_b, d.stride_i);
         return;
@@ -489,6 +634,9 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
             causal_softmax_rows<T, BS, NV, false><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),             \
                                                                            static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by_seq); \
     } while (0)
+    // (A lane count taken from the launch, so that a row of 10240 elements gets 320 lanes x 4 vectors instead of
+    // 512 x 4, measured worse, not better: [64, 512, 10240] fp16 364 against 237 us, [64, 512, 20480] 763
+    // against 647 us - workgroups of 5, 10 or 12 wavefronts sit unevenly on a compute unit's four SIMDs.)
     if (nvec <= 64) CS_LAUNCH(64, 1);
     else if (nvec <= 128) CS_LAUNCH(64, 2);
     else if (nvec <= 256) CS_LAUNCH(64, 4);

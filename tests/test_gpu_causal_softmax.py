@@ -56,6 +56,8 @@ CASES = [
     ((5, 64, 128), None), ((3, 100, 256), None), ((2, 30, 200), None), ((6, 24, 40), None), ((4, 16, 64), (16 * 80 + 8, 80, 1)),
     ((3, 13, 64), None), ((300000, 16, 16), None), ((9, 256, 256), None),
     # rows of 257-512 elements, two to a wavefront with two vectors per lane: square, wide, ragged, padded, an odd number of rows
+    # rows beyond what a workgroup holds in registers: three passes with 16-byte accesses (512 and 1024 lanes), padded rows
+    ((2, 6, 65536), None), ((1, 4, 100000), None), ((2, 3, 40000), (3 * 40008, 40008, 1)), ((1, 7, 32776), None),
     ((5, 512, 512), None), ((3, 40, 400), None), ((2, 300, 512), None), ((3, 64, 264), None), ((2, 16, 504), (16 * 520, 520, 1)), ((2, 33, 512), None),
 ]
 
@@ -103,6 +105,22 @@ def test_infinities_and_long_tails(ctx):
     got, _, _ = run(ctx, y, y.shape, None, "f16")
     check(got, want, "f16", "infinities and tails", max_frac=2e-2)
     assert np.isnan(oracle.decode(got, "f16")[0, 5, 0])
+
+
+def test_infinities_and_long_tails_in_long_rows(ctx):
+    """The same special values in rows of 50 000 elements (the three-pass form)."""
+    rng = np.random.default_rng(79)
+    vals = rng.standard_normal((2, 6, 50000)).astype(np.float32) * 2
+    vals[0, :, 3] = -np.inf
+    vals[0, 4, :] = -np.inf
+    vals[1, :, 49990] = -300.0
+    vals[1, 3, 0] = 200.0
+    vals[1, 5, :30000] = -60000.0
+    y = oracle.encode(vals, "f16")
+    want = oracle.causal_softmax(y.copy(), "f16")
+    got, _, _ = run(ctx, y, y.shape, None, "f16")
+    check(got, want, "f16", "infinities and tails, long rows", max_frac=2e-2)
+    assert np.isnan(oracle.decode(got, "f16")[0, 4, 0])
 
 
 def test_short_rows_give_the_bits_of_a_wavefront_per_row(ctx):
