@@ -58,18 +58,44 @@ __device__ __attribute__((noinline)) void exp_any8(float *v, float mx) {
 // Loads are unconditional: a lane whose vector lies in the masked part
 // re-reads the row's last kept vector, which the memory pipeline merges into
 // one request.
-template<typename T, int BS, int NV, bool THROUGH>
+// RAGGED: rows that do not all start on 128-byte boundaries - the scores of an
+// attention over a number of keys that is no multiple of 64 - of at least 16
+// elements.  Two things change.
+// (1) The vectors are the whole 16-byte aligned ones inside the row (its
+// body), as many as the workgroup has room for.  The up to 7 elements in front
+// of the first of them and the up to 56 behind the last are taken one each by
+// the lanes of the first wavefront, with 2-byte loads and stores, and enter
+// the maximum, the sum and the quotients beside those lanes' vectors: about 25
+// more vector instructions per row and nothing else.  So a row of 4100
+// elements is still one wavefront's: 512 vectors and 4 elements.  (Taking the two 16-byte vectors that
+// overlap the row's ends instead, and masking what is not the row's, cost
+// 25-40 % at 1000-4000 elements; 16-byte accesses at 2-byte alignment, which
+// gfx950 also serves, were 3-4 times slower still.)
+// (2) Lanes take the vectors rotated by the body's distance from a 128-byte
+// boundary (slot s holds vector s - shift, the first `shift` slots the last
+// vectors the workgroup has room for), so that the 1 KiB a wavefront loads or
+// stores with one instruction is made of whole 128-byte lines.  Without that,
+// measured on MI355X: [32, 4088, 4088] fp16 360 us against 260 us for
+// [32, 4032, 4032], [128, 1000, 1000] 83 us against 65 us for [128, 960, 960].
+template<typename T, int BS, int NV, bool THROUGH, bool RAGGED>
 __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
                                                           int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
     AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
     constexpr int WAVES = BS / kWave;
     __shared__ float red[4 * WAVES];// two slot sets for the maxima, two for the sums
-    const uint32_t nvec = total / 8;
     const float neg_inf = -__builtin_inff();
 
     struct Row {
-        uint16_t *ptr;
-        uint32_t keep;// columns kept, 1..total
+        uint16_t *ptr;  // the row's first element
+        uint32_t keep;  // columns kept, 1..total
+        uint32_t head;  // elements in front of the body, 0..7; 0 unless RAGGED
+        uint32_t nvec;  // vectors of the body
+        uint32_t shift; // 16-byte vectors between the 128-byte boundary in front of the body and the body; 0 unless RAGGED
+    };
+    // the vector of the body that this lane holds in its slot k
+    auto vector_at = [&](const Row &row, int k) {
+        const uint32_t s = k * BS + threadIdx.x - row.shift;
+        return RAGGED && static_cast<int32_t>(s) < 0 ? s + NV * BS : s;
     };
     // Global row r = b*seq + i.  All workgroups work on neighbouring rows at
     // any one time (measured: faster than giving each matrix of the batch its
@@ -78,7 +104,17 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
     const uint32_t hop_b = fast_quotient(hop, by_seq), hop_i = hop - hop_b * seq;// the grid is far below 2^31 rows (see FastDiv)
     uint64_t b = fast_quotient(blockIdx.x, by_seq);
     uint32_t i = blockIdx.x - static_cast<uint32_t>(b) * seq;
-    auto here = [&]() { return Row{y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i, total - seq + i + 1}; };
+    auto here = [&]() {
+        uint16_t *ptr = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
+        if constexpr (RAGGED) {
+            const uint32_t head = (8u - static_cast<uint32_t>(reinterpret_cast<uintptr_t>(ptr) & 15u) / 2) & 7u;
+            const uint32_t shift = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(ptr + head) & 127u) / 16;
+            const uint32_t whole = (total - head) / 8;
+            return Row{ptr, total - seq + i + 1, head, whole < NV * BS ? whole : NV * BS, shift};
+        } else {
+            return Row{ptr, total - seq + i + 1, 0u, total / 8, 0u};
+        }
+    };
     auto advance = [&]() {
         b += hop_b;
         i += hop_i;
@@ -87,12 +123,20 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
             ++b;
         }
     };
+    // kept columns of the body: all of them when !RAGGED, possibly none otherwise
+    auto kept_in_body = [&](const Row &row) {
+        if constexpr (!RAGGED) return row.keep;
+        const uint32_t past_head = row.keep > row.head ? row.keep - row.head : 0u;
+        return past_head < row.nvec * 8 ? past_head : row.nvec * 8;
+    };
     auto load_row = [&](const Row &row, u32x4(&dst)[NV]) {
-        const uint32_t last_vec = (row.keep - 1) / 8;
+        const uint32_t keep = kept_in_body(row);
+        const uint32_t last_vec = RAGGED && keep == 0 ? 0u : (keep - 1) / 8;
+        const uint16_t *body = row.ptr + row.head;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
-            dst[k] = ld16_stream(row.ptr + static_cast<uint64_t>(v < last_vec ? v : last_vec) * 8);
+            const uint32_t v = vector_at(row, k);
+            dst[k] = ld16_stream(body + static_cast<uint64_t>(v < last_vec ? v : last_vec) * 8);
         }
     };
     // The one vector of a row that straddles the mask (when the kept length is
@@ -104,15 +148,26 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
     // row that turned to NaN would otherwise leak into them).  Everything else
     // runs without a per-element test.
     auto finish_row = [&](const Row &row, const u32x4(&cur)[NV], int phase) {
-        const uint32_t keep = row.keep;
+        const uint32_t keep = kept_in_body(row), nvec = row.nvec;
         const uint32_t keep_vecs = (keep + 7) / 8;
         const uint32_t tail = keep & 7u;// kept elements of the straddling vector, 0 when there is none
+        // RAGGED: lanes 0-7 of the workgroup hold the elements in front of the body, lanes 8-63 those behind it
+        [[maybe_unused]] uint32_t end_col = 0;// this lane's column of the row, if end_mine
+        [[maybe_unused]] bool end_mine = false, end_kept = false;
+        [[maybe_unused]] float end_x = 0.0f;
+        if constexpr (RAGGED) {
+            const uint32_t t = threadIdx.x;
+            end_col = t < 8 ? t : row.head + nvec * 8 + (t - 8);
+            end_mine = t < 8 ? t < row.head : (t < kWave && end_col < total);
+            end_kept = end_mine && end_col < row.keep;
+            if (end_kept) end_x = T::one(row.ptr[end_col]);
+        }
         float mx = neg_inf, mn = __builtin_inff();
         [[maybe_unused]] typename T::pair mx2, mn2;
         if constexpr (T::kPackedMinMax) mx2 = T::splat(neg_inf), mn2 = T::splat(__builtin_inff());
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
+            const uint32_t v = vector_at(row, k);
             const bool straddles = tail != 0 && v + 1 == keep_vecs;
             if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
                 if (straddles) {
@@ -143,6 +198,9 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
             mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
             mn = fminf(mn, fminf(T::first(mn2), T::second(mn2)));
         }
+        if constexpr (RAGGED) {
+            if (end_kept) mx = fmaxf(mx, end_x), mn = fminf(mn, end_x);
+        }
         mx = block_max<WAVES>(mx, red, phase);
 
         // d = x - max <= 0.  Anything below the lean exponential's range (-inf
@@ -155,7 +213,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
         float part = 0.0f;
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
+            const uint32_t v = vector_at(row, k);
             if (v >= keep_vecs) continue;
             widen8<T>(cur[k], f[k]);
             if (lean) {
@@ -179,21 +237,38 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
 #pragma unroll
             for (int e = 0; e < 8; ++e) part += f[k][e];
         }
+        [[maybe_unused]] float end_f = 0.0f;
+        if constexpr (RAGGED) {
+            if (threadIdx.x < kWave) {
+                if (lean) {
+                    end_f = exp_nonpositive(end_x - mx);
+                } else {
+                    float slow[8] = {end_x, mx, mx, mx, mx, mx, mx, mx};
+                    exp_any8(slow, mx);
+                    end_f = slow[0];
+                }
+                end_f = end_kept ? end_f : 0.0f;
+                part += end_f;
+            }
+        }
         const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
         const float rcp = 1.0f / sum;
-        const StreamOut<THROUGH> out(row.ptr);// the row is the same for every lane of the workgroup
+        const StreamOut<THROUGH> out(row.ptr + row.head);// the row is the same for every lane of the workgroup
+        // e / sum: one residual step makes the quotient correctly rounded in all but rare cases
+        auto quotient = [&](float e) {
+            const float q = e * rcp;
+            return __builtin_fmaf(__builtin_fmaf(-sum, q, e), rcp, q);
+        };
 
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            const uint32_t v = k * BS + threadIdx.x;
+            const uint32_t v = vector_at(row, k);
+            u32x4 packed{0, 0, 0, 0};
             if (v < keep_vecs) {
                 float o[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float q = f[k][e] * rcp;// e / sum: one residual step makes the quotient correctly rounded in all but rare cases
-                    o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, f[k][e]), rcp, q);
-                }
-                u32x4 packed = narrow8_unit_range<T>(o);
+                for (int e = 0; e < 8; ++e) o[e] = quotient(f[k][e]);
+                packed = narrow8_unit_range<T>(o);
                 const bool straddles = tail != 0 && v + 1 == keep_vecs;
                 if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
                     if (straddles) {// its masked tail is zero whatever the row turned into
@@ -205,10 +280,11 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
                         packed = u32x4{w[0], w[1], w[2], w[3]};
                     }
                 }
-                out.st16(v * 16, packed);
-            } else if (v < nvec) {
-                out.st16(v * 16, u32x4{0, 0, 0, 0});
             }
+            if (v < nvec) out.st16(v * 16, packed);
+        }
+        if constexpr (RAGGED) {
+            if (end_mine) row.ptr[end_col] = end_kept ? static_cast<uint16_t>(T::narrow2_fast(quotient(end_f), 0.0f) & 0xFFFFu) : uint16_t{0};
         }
     };
 
@@ -372,28 +448,41 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
     }
 }
 
-// Rows longer than a workgroup can hold in registers (more than 32 768
-// elements), 16-byte aligned: three passes over the row with 16-byte accesses
-// - the maximum (and the minimum, for the choice of exponential), the sum of
-// the exponentials, the quotients - UNROLL vectors per lane in flight at a
-// time.  The first pass brings the row in from memory; the other two find it
-// in L2 or in the Infinity Cache, so the exponentials are formed twice but
-// memory is read once.  Masked vectors are written as zeros without being
-// read.  One workgroup per row at a time.
-template<typename T, int BS, bool THROUGH>
+// Rows that the register kernels above do not take: longer than a workgroup
+// can hold (more than 32 768 elements), or RAGGED - rows that do not start on
+// 16-byte boundaries or whose length is no multiple of 8, which is what the
+// scores of an attention over an arbitrary number of keys look like.  Three
+// passes over the row with 16-byte accesses - the maximum (and the minimum,
+// for the choice of exponential), the sum of the exponentials, the quotients -
+// UNROLL vectors per lane in flight at a time.  The first pass brings the row
+// in from memory; the other two find it in L2 or in the Infinity Cache, so the
+// exponentials are formed twice but memory is read once.  Masked vectors are
+// written as zeros without being read.  One workgroup per row at a time.
+// RAGGED: the vectors are the 16-byte aligned ones that cover the row, so the
+// first holds up to 7 elements of whatever lies in front of the row and the
+// last up to 7 of what lies behind it (both inside the same 16 bytes as an
+// element of the row, so reading them is safe).  Those foreign elements take
+// no part in the reductions, and the two edge vectors are written element by
+// element by the lane that owns them - the neighbouring bytes belong to other
+// rows, which other workgroups are working on.  (16-byte accesses at 2-byte
+// alignment, which gfx950 also serves, measured 3-4 times slower than this.)
+template<typename T, int BS, bool THROUGH, bool RAGGED>
 __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
                                                           int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
     AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
     constexpr int WAVES = BS / kWave, UNROLL = 4;
     __shared__ float red[4 * WAVES];
-    const uint32_t nvec = total / 8;
     int phase = 0;
     for (uint64_t r = blockIdx.x; r < rows; r += gridDim.x, phase ^= 1) {
         const uint32_t b = fast_quotient(static_cast<uint32_t>(r), by_seq), i = static_cast<uint32_t>(r) - b * seq;// fewer than 2^31 rows (see FastDiv)
         uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
-        const uint32_t keep = total - seq + i + 1;
-        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u;
-        const uint32_t whole_vecs = keep / 8;// vectors all of whose elements are kept
+        // positions count from the 16-byte boundary at or in front of the row: the row is [lo, end), its kept part [lo, hi)
+        const uint32_t lo = RAGGED ? static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u) / 2 : 0u;
+        const uint16_t *base = row - lo;
+        const uint32_t hi = lo + (total - seq + i + 1), end = lo + total;
+        const uint32_t keep_vecs = (hi + 7) / 8, nvec = (end + 7) / 8;// vectors that hold kept elements; vectors that hold elements of the row
+        const uint32_t kept_from = (lo + 7) / 8, kept_to = hi / 8;      // vectors [kept_from, kept_to) are kept entirely
+        const uint32_t own_to = end / 8;                                // vectors [kept_from, own_to) belong to the row entirely
 
         // pass 1: maximum and minimum of the kept elements
         float mx = -__builtin_inff(), mn = __builtin_inff();
@@ -402,18 +491,27 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const uint32_t v = v0 + u * BS;
-                x[u] = ld16(row + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);// re-reading the last kept vector changes no maximum
+                x[u] = ld16(base + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);// re-reading the last kept vector changes no maximum
             }
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const uint32_t v = v0 + u * BS;
+                const uint32_t got = v < keep_vecs ? v : keep_vecs - 1;// the vector that was read
                 float f[8];
                 widen8<T>(x[u], f);
-                const uint32_t got = v < keep_vecs ? v : keep_vecs - 1;// the vector that was read
-                const uint32_t lim = got < whole_vecs ? 8u : tail;     // its kept elements (beyond the whole vectors there is only the straddling one)
+                const bool edge = got < kept_from || got >= kept_to;
+                if (__builtin_amdgcn_ballot_w64(edge) != 0) {
+                    if (edge) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    if (static_cast<uint32_t>(e) < lim) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+                        for (int e = 0; e < 8; ++e) {
+                            const uint32_t p = got * 8 + e;
+                            if (p >= lo && p < hi) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+                        }
+                    }
+                }
+                if (!edge) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
                 }
             }
         }
@@ -421,7 +519,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
         const float lowest = mn - mx;
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
 
-        // exp(x - max) of one vector, zero where the mask cuts it
+        // exp(x - max) of the elements of vector v, zero for those that are not kept
         auto exps = [&](u32x4 x, uint32_t v, float(&e8)[8]) {
             widen8<T>(x, e8);
             if (lean) {
@@ -435,9 +533,15 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
 #pragma unroll
                 for (int e = 0; e < 8; ++e) e8[e] = slow[e];
             }
-            if (v >= whole_vecs) {// the straddling vector
+            const bool edge = v < kept_from || v >= kept_to;
+            if (__builtin_amdgcn_ballot_w64(edge) != 0) {
+                if (edge) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) e8[e] = static_cast<uint32_t>(e) < tail ? e8[e] : 0.0f;
+                    for (int e = 0; e < 8; ++e) {
+                        const uint32_t p = v * 8 + e;
+                        e8[e] = p >= lo && p < hi ? e8[e] : 0.0f;
+                    }
+                }
             }
         };
 
@@ -448,7 +552,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const uint32_t v = v0 + u * BS;
-                x[u] = ld16(row + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
+                x[u] = ld16(base + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
             }
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
@@ -465,13 +569,13 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
         const float rcp = 1.0f / sum;
 
         // pass 3: the quotients, and zeros behind them
-        const StreamOut<THROUGH> out(row);
+        const StreamOut<THROUGH> out(const_cast<uint16_t *>(base));
         for (uint32_t v0 = threadIdx.x; v0 < nvec; v0 += BS * UNROLL) {
             u32x4 x[UNROLL];
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const uint32_t v = v0 + u * BS;
-                x[u] = ld16(row + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
+                x[u] = ld16(base + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
             }
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
@@ -486,16 +590,34 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
                         o[e] = __builtin_fmaf(__builtin_fmaf(-sum, q, e8[e]), rcp, q);
                     }
                     packed = narrow8_unit_range<T>(o);
-                    if (v >= whole_vecs) {// its masked tail is zero whatever the row turned into
-                        uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+                    const bool edge = v < kept_from || v >= kept_to;
+                    if (__builtin_amdgcn_ballot_w64(edge) != 0) {
+                        if (edge) {// what is not kept is zero whatever the row turned into
+                            uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            if (static_cast<uint32_t>(e) >= tail) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                            for (int e = 0; e < 8; ++e) {
+                                const uint32_t p = v * 8 + e;
+                                if (!(p >= lo && p < hi)) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                            }
+                            packed = u32x4{w[0], w[1], w[2], w[3]};
                         }
-                        packed = u32x4{w[0], w[1], w[2], w[3]};
                     }
                 }
-                if (v < nvec) out.st16(v * 16, packed);
+                const bool mine = v >= kept_from && v < own_to;// all sixteen bytes are the row's
+                if (mine) out.st16(v * 16, packed);
+                if constexpr (RAGGED) {
+                    const bool shared = !mine && v < nvec;
+                    if (__builtin_amdgcn_ballot_w64(shared) != 0) {
+                        if (shared) {
+                            const uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const uint32_t p = v * 8 + e;
+                                if (p >= lo && p < end) row[static_cast<int64_t>(p) - lo] = static_cast<uint16_t>(w[e / 2] >> (16 * (e & 1)));
+                            }
+                        }
+                    }
+                }
             }
         }
     }
@@ -547,25 +669,43 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     // it the mask keeps, four cycles each on a 16-lane SIMD ([2048, 512, 512] fp16: 374 us =
     // 875 cycles per row and SIMD; the same bytes as [8192, 256, 256] take 735 us).  Asking
     // for 2 or 4 rows per wavefront before working on the first moved that by -5 to +2 %.
-    const uint64_t cap = nvec <= 64 ? static_cast<uint64_t>(d.cu_count) * 512 : rows;
+    const bool aligned = d.total % 8 == 0 && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);
+    const bool in_lines = aligned && d.stride_i % 64 == 0 && d.stride_b % 64 == 0 && (reinterpret_cast<uintptr_t>(data) & 127u) == 0;// rows start on 128-byte boundaries
+    // Vectors per row that the kernel must have room for.  The ragged form takes up to 56 elements behind them one by one
+    // (see causal_softmax_rows), which rows in whole lines also use when that spares them the next larger form.
+    const auto form_of = [](uint64_t vectors) { return vectors <= 64 ? 0 : 64 - __builtin_clzll(vectors - 1) - 6; };// 64, 128, 256, ... vectors
+    const uint64_t spared = d.total <= 56 ? 1 : ceil_div(d.total - 56, 8);
+    const bool ragged = !in_lines || form_of(spared) < form_of(nvec);
+    const uint64_t cover = ragged ? spared : nvec;
+    const uint64_t cap = cover <= 64 ? static_cast<uint64_t>(d.cu_count) * 512 : rows;
     const uint64_t limit = amd::max_grid_1d(1024);// the kernel strides over what the grid does not cover
     const unsigned grid = static_cast<unsigned>(std::min({rows, cap, limit}));
 
-    const bool vec_ok = d.total % 8 == 0 && nvec <= 4096 && d.seq < (1ull << 31) && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 && aligned16(data);
-    const bool long_ok = d.total % 8 == 0 && nvec > 4096 && d.total < (1ull << 31) && rows < kFastDivLimit && d.stride_i % 8 == 0 && d.stride_b % 8 == 0 &&
-                         aligned16(data) && d.total * 2 < (1ull << 32);
+    const bool even = (reinterpret_cast<uintptr_t>(data) & 1u) == 0;// elements lie on 2-byte boundaries
+    const bool vec_ok = even && cover <= 4096 && d.seq < (1ull << 31) && (!ragged || d.total >= 16);
+    // Rows of more than 32 768 elements (see causal_softmax_long).  Measured on MI355X, fp16, against the element kernel:
+    //   [64, 512, 65536]  2171 us (49 %) against 7230 us     [64, 512, 40000]  1293 against 4194 us
+    const uint64_t vecs = cover;
+    const bool long_ok = even && cover > 4096 && d.total + 8 < (1ull << 31) && rows < kFastDivLimit;
     if (long_ok) {
         const bool thr = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
         const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
-        // 1024 lanes take 4096 vectors a turn: rows of fewer than two turns are better served by 512 ([64, 512, 40000] fp16
-        // 1293 against 1584 us; [64, 512, 65536] 2320 against 2171 us; 256 lanes: 1451 and 2394 us)
-        const int lanes = nvec < 8192 ? 512 : 1024;
+        // a turn of the workgroup takes 4 vectors per lane: the lane count that covers the row in the fewest turns with the fewest idle lanes
+        // ([64, 512, 40000] fp16: 512 lanes 1293 us, 1024 lanes 1584 us, 256 lanes 1451 us; [64, 512, 65536]: 2320, 2171, 2394 us)
+        const int lanes = vecs < 8192 ? 512 : 1024;
         const unsigned g = static_cast<unsigned>(std::min<uint64_t>(rows, amd::max_grid_1d(1024)));
-#define CS_LONG(BS) do { if (thr) causal_softmax_long<T, BS, true><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by); \
-                         else causal_softmax_long<T, BS, false><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by); } while (0)
+#define CS_LONG_GO(BS, TH, RG) causal_softmax_long<T, BS, TH, RG><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)
+#define CS_LONG(BS)                                        \
+    do {                                                   \
+        if (!aligned && thr) CS_LONG_GO(BS, true, true);   \
+        else if (!aligned) CS_LONG_GO(BS, false, true);    \
+        else if (thr) CS_LONG_GO(BS, true, false);         \
+        else CS_LONG_GO(BS, false, false);                 \
+    } while (0)
         if (lanes == 512) CS_LONG(512);
         else CS_LONG(1024);
 #undef CS_LONG
+#undef CS_LONG_GO
         return;
     }
     if (!vec_ok) {
@@ -581,7 +721,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     //   [32768, 128, 128]  1385 -> 291 us                    [131072, 64, 64]  2765 -> 324 us
     // with 2048 wavefronts per compute unit striding over the groups (128 / 512 / 8192 per unit: 382 / 348 / 351 us
     // at 256 columns with 32 lanes per row).
-    if (nvec <= 64 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
+    if (aligned && nvec <= 64 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
         // Lanes per row x vectors per lane: the pair that wastes the fewest lanes, the fewer lanes per row (more
         // rows per wavefront) when two waste the same, among those whose rows per wavefront divide the matrix's
         // row count.  More than one vector per lane spares the rows that the mask cuts short the work of the
@@ -625,26 +765,32 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
             return;
         }
     }
-#define CS_LAUNCH(BS, NV)                                                                                                      \
-    do {                                                                                                                       \
-        if (through)                                                                                                           \
-            causal_softmax_rows<T, BS, NV, true><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),              \
-                                                                          static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by_seq); \
-        else                                                                                                                   \
-            causal_softmax_rows<T, BS, NV, false><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq),             \
-                                                                           static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by_seq); \
+#define CS_GO(BS, NV, TH, RG) \
+    causal_softmax_rows<T, BS, NV, TH, RG><<<grid, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by_seq)
+#define CS_LAUNCH(BS, NV)                               \
+    do {                                                \
+        if (through && !ragged) CS_GO(BS, NV, true, false); \
+        else if (through) CS_GO(BS, NV, true, true);    \
+        else if (!ragged) CS_GO(BS, NV, false, false);  \
+        else CS_GO(BS, NV, false, true);                \
     } while (0)
     // (A lane count taken from the launch, so that a row of 10240 elements gets 320 lanes x 4 vectors instead of
     // 512 x 4, measured worse, not better: [64, 512, 10240] fp16 364 against 237 us, [64, 512, 20480] 763
     // against 647 us - workgroups of 5, 10 or 12 wavefronts sit unevenly on a compute unit's four SIMDs.)
-    if (nvec <= 64) CS_LAUNCH(64, 1);
-    else if (nvec <= 128) CS_LAUNCH(64, 2);
-    else if (nvec <= 256) CS_LAUNCH(64, 4);
-    else if (nvec <= 512) CS_LAUNCH(64, 8);
-    else if (nvec <= 1024) CS_LAUNCH(256, 4);
-    else if (nvec <= 2048) CS_LAUNCH(512, 4);
+    // Rows that do not start on 128-byte boundaries, or are no multiple of 8 elements long, take the ragged form of the
+    // same kernels.  Measured on MI355X, fp16, us (in brackets the element kernel, which used to take the unaligned ones,
+    // and the plain form, which used to take those on 16-byte boundaries):
+    //   [32, 4095, 4095]  285 (1033)   [32, 1024, 4099]  85 (392)   [64, 512, 1027]  24 (78)   [256, 128, 333]  18 (45)
+    //   [32, 4088, 4088]  278 (360)    [32, 4100, 4104]  281 (450)  [32, 2048, 2056]  74 (100)  [128, 1000, 1000]  72 (83)
+    if (cover <= 64) CS_LAUNCH(64, 1);
+    else if (cover <= 128) CS_LAUNCH(64, 2);
+    else if (cover <= 256) CS_LAUNCH(64, 4);
+    else if (cover <= 512) CS_LAUNCH(64, 8);
+    else if (cover <= 1024) CS_LAUNCH(256, 4);
+    else if (cover <= 2048) CS_LAUNCH(512, 4);
     else CS_LAUNCH(1024, 4);
 #undef CS_LAUNCH
+#undef CS_GO
 }
 
 }// namespace

@@ -56,6 +56,11 @@ CASES = [
     ((5, 64, 128), None), ((3, 100, 256), None), ((2, 30, 200), None), ((6, 24, 40), None), ((4, 16, 64), (16 * 80 + 8, 80, 1)),
     ((3, 13, 64), None), ((300000, 16, 16), None), ((9, 256, 256), None),
     # rows of 257-512 elements, two to a wavefront with two vectors per lane: square, wide, ragged, padded, an odd number of rows
+    # lengths that are no multiple of 8 and rows that do not start on 16-byte boundaries (what attention over an arbitrary number
+    # of keys produces): the aligned vectors that cover a row, its two edge vectors written element by element; every workgroup size
+    ((32, 20, 333), None), ((3, 100, 1027), None), ((2, 50, 4099), None), ((2, 9, 33001), None), ((5, 60, 63), None), ((4, 7, 7), None),
+    ((2, 130, 2050), None), ((3, 40, 2048), (40 * 2051, 2051, 1)), ((2, 5, 70003), None), ((6, 300, 301), None),
+    ((2, 40, 4100), None), ((2, 33, 2104), None), ((2, 33, 2105), None), ((3, 50, 1080), None), ((2, 1000, 1000), None), ((1, 600, 4088), None),
     # rows beyond what a workgroup holds in registers: three passes with 16-byte accesses (512 and 1024 lanes), padded rows
     ((2, 6, 65536), None), ((1, 4, 100000), None), ((2, 3, 40000), (3 * 40008, 40008, 1)), ((1, 7, 32776), None),
     ((5, 512, 512), None), ((3, 40, 400), None), ((2, 300, 512), None), ((3, 64, 264), None), ((2, 16, 504), (16 * 520, 520, 1)), ((2, 33, 512), None),
@@ -74,6 +79,40 @@ def test_against_oracle(ctx, dt, case):
     keep = np.arange(total)[None, :] <= total - seq + np.arange(seq)[:, None]
     assert not got[..., ~keep].any(), "masked columns must be exact zeros"
     check(got, want, dt, f"{shape} {strides} {dt}", max_frac=2e-2 if total > 4096 else 5e-3)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("start,shape,pitch", [(3, (4, 50, 333), 341), (1, (2, 30, 1000), 1001), (5, (3, 17, 2047), 2047), (7, (2, 9, 4101), 4110),
+                                               (2, (2, 4, 33333), 33339), (0, (3, 21, 77), 77), (6, (40, 3, 5), 5), (4, (2, 6, 520), 523),
+                                               # up to 56 elements behind a workgroup's vectors are taken one by one, also for rows in whole lines
+                                               (0, (2, 10, 4152), 4160), (0, (3, 12, 2104), 2112), (3, (2, 12, 2105), 2111), (0, (2, 7, 32800), 32832),
+                                               (5, (2, 9, 32830), 32831), (1, (3, 10, 16), 16), (0, (3, 10, 15), 15), (3, (2, 16, 17), 19), (0, (2, 70, 568), 576)])
+def test_ragged_rows_leave_their_neighbours_alone(ctx, dt, start, shape, pitch):
+    """Rows that start anywhere and end anywhere, inside a buffer of other data:
+    `start` elements in front of the first row, `pitch - total` between rows.
+    The kernels read the 16-byte vectors that cover a row and must write the
+    row's own elements only."""
+    import torch
+
+    batch, seq, total = shape
+    rng = np.random.default_rng(900 + start + total)
+    y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 2, dt)
+    want = oracle.causal_softmax(y.copy(), dt)
+    span = start + batch * seq * pitch + 11
+    before = rng.integers(0, 0x3C00, span, dtype=np.uint16)
+    buf = to_torch(before, dt)
+    view = torch.as_strided(buf, shape, (seq * pitch, pitch, 1), storage_offset=start)
+    view.copy_(to_torch(y, dt).reshape(shape))
+    ctx.causal_softmax(view)
+    torch.cuda.synchronize()
+    got, after = to_codes(view), to_codes(buf)
+    check(got, want, dt, f"{start} {shape} {pitch} {dt}", max_frac=2e-2 if total > 4096 else 5e-3)
+    keep = np.arange(total)[None, :] <= total - seq + np.arange(seq)[:, None]
+    assert not got[..., ~keep].any()
+    own = np.zeros(span, bool)
+    rows = start + (np.arange(batch * seq) * pitch)[:, None] + np.arange(total)[None, :]
+    own[rows.ravel()] = True
+    assert np.array_equal(before[~own], after[~own]), "elements outside the rows were written"
 
 
 def test_attention_scores_shape(ctx):
