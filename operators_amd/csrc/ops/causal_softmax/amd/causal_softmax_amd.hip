@@ -78,10 +78,13 @@ __device__ __attribute__((noinline)) void exp_any8(float *v, float mx) {
 // measured on MI355X: [32, 4088, 4088] fp16 360 us against 260 us for
 // [32, 4032, 4032], [128, 1000, 1000] 83 us against 65 us for [128, 960, 960].
 template<typename T, int BS, int NV, bool THROUGH, bool RAGGED>
-__global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
+__global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(BS == 512 && NV == 8 ? 4 : 1)))// 512 x 8: two workgroups per compute unit
+void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total,
                                                           int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
     AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
     constexpr int WAVES = BS / kWave;
+    // the form held to 128 registers has none to spare for the packed comparisons' second pair of accumulators
+    constexpr bool kPacked = T::kPackedMinMax && !(RAGGED && BS == 512 && NV == 8);
     __shared__ float red[4 * WAVES];// two slot sets for the maxima, two for the sums
     const float neg_inf = -__builtin_inff();
 
@@ -94,8 +97,8 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
     };
     // the vector of the body that this lane holds in its slot k
     auto vector_at = [&](const Row &row, int k) {
-        const uint32_t s = k * BS + threadIdx.x - row.shift;
-        return RAGGED && static_cast<int32_t>(s) < 0 ? s + NV * BS : s;
+        const uint32_t s = k * BS + threadIdx.x - row.shift;// shift < 8: only slot 0 can fall in front of the body
+        return RAGGED && k == 0 && static_cast<int32_t>(s) < 0 ? s + NV * BS : s;
     };
     // Global row r = b*seq + i.  All workgroups work on neighbouring rows at
     // any one time (measured: faster than giving each matrix of the batch its
@@ -164,7 +167,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
         }
         float mx = neg_inf, mn = __builtin_inff();
         [[maybe_unused]] typename T::pair mx2, mn2;
-        if constexpr (T::kPackedMinMax) mx2 = T::splat(neg_inf), mn2 = T::splat(__builtin_inff());
+        if constexpr (kPacked) mx2 = T::splat(neg_inf), mn2 = T::splat(__builtin_inff());
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = vector_at(row, k);
@@ -180,7 +183,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
                 }
             }
             if (v >= keep_vecs || straddles) continue;// wholly masked: nothing to reduce, zeros are stored below
-            if constexpr (T::kPackedMinMax) {
+            if constexpr (kPacked) {
                 const uint32_t w[4] = {cur[k].x, cur[k].y, cur[k].z, cur[k].w};
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
                 for (int e = 0; e < 8; ++e) mx = fmaxf(mx, b[e]), mn = fminf(mn, b[e]);
             }
         }
-        if constexpr (T::kPackedMinMax) {
+        if constexpr (kPacked) {
             mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
             mn = fminf(mn, fminf(T::first(mn2), T::second(mn2)));
         }
@@ -211,6 +214,20 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
         float f[NV][8];
         float part = 0.0f;
+        [[maybe_unused]] float end_f = 0.0f;
+        if constexpr (RAGGED) {
+            if (threadIdx.x < kWave) {
+                if (lean) {
+                    end_f = exp_nonpositive(end_x - mx);
+                } else {
+                    float slow[8] = {end_x, mx, mx, mx, mx, mx, mx, mx};
+                    exp_any8(slow, mx);
+                    end_f = slow[0];
+                }
+                end_f = end_kept ? end_f : 0.0f;
+                part = end_f;
+            }
+        }
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = vector_at(row, k);
@@ -237,20 +254,6 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
 #pragma unroll
             for (int e = 0; e < 8; ++e) part += f[k][e];
         }
-        [[maybe_unused]] float end_f = 0.0f;
-        if constexpr (RAGGED) {
-            if (threadIdx.x < kWave) {
-                if (lean) {
-                    end_f = exp_nonpositive(end_x - mx);
-                } else {
-                    float slow[8] = {end_x, mx, mx, mx, mx, mx, mx, mx};
-                    exp_any8(slow, mx);
-                    end_f = slow[0];
-                }
-                end_f = end_kept ? end_f : 0.0f;
-                part += end_f;
-            }
-        }
         const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
         const float rcp = 1.0f / sum;
         const StreamOut<THROUGH> out(row.ptr + row.head);// the row is the same for every lane of the workgroup
@@ -259,6 +262,9 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
             const float q = e * rcp;
             return __builtin_fmaf(__builtin_fmaf(-sum, q, e), rcp, q);
         };
+        if constexpr (RAGGED) {
+            if (end_mine) row.ptr[end_col] = end_kept ? static_cast<uint16_t>(T::narrow2_fast(quotient(end_f), 0.0f) & 0xFFFFu) : uint16_t{0};
+        }
 
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -282,9 +288,6 @@ __global__ __launch_bounds__(BS) void causal_softmax_rows(uint16_t *y, uint64_t 
                 }
             }
             if (v < nvec) out.st16(v * 16, packed);
-        }
-        if constexpr (RAGGED) {
-            if (end_mine) row.ptr[end_col] = end_kept ? static_cast<uint16_t>(T::narrow2_fast(quotient(end_f), 0.0f) & 0xFFFFu) : uint16_t{0};
         }
     };
 
@@ -653,7 +656,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
     // Rows of up to 4096 elements are taken by single wavefronts (no barrier, no
-    // LDS), longer ones by 256-1024 lanes.  Measured on MI355X, fp16 / bf16:
+    // LDS), longer ones by 256 or 512 lanes.  Measured on MI355X, fp16 / bf16:
     //   [32, 4096, 4096]   one workgroup per row 264 / 261-266 us (76 %), 256 workgroups per
     //                      compute unit 267 / 267-274, 64 per unit 293 / 292-299; 128 or 256
     //                      lanes per row 264-288 / 261-270
@@ -774,6 +777,10 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         else if (!ragged) CS_GO(BS, NV, false, false);  \
         else CS_GO(BS, NV, false, true);                \
     } while (0)
+    // Rows of 16 385-32 768 elements: 512 lanes x 8 vectors, held to 128 registers so that a compute unit has two rows in
+    // hand and one row's arithmetic overlaps the other's loads and stores.  1024 lanes x 4 vectors (one row per unit, its
+    // phases strictly one after the other) measured, fp16: [64, 512, 20480] 644 -> 430 us (52 -> 77 %), [64, 512, 32768]
+    // 945 -> 768 us, [2, 20480, 20480] 682 -> 454 us, [1, 32768, 32768] 723 -> 583 us.
     // (A lane count taken from the launch, so that a row of 10240 elements gets 320 lanes x 4 vectors instead of
     // 512 x 4, measured worse, not better: [64, 512, 10240] fp16 364 against 237 us, [64, 512, 20480] 763
     // against 647 us - workgroups of 5, 10 or 12 wavefronts sit unevenly on a compute unit's four SIMDs.)
@@ -788,7 +795,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     else if (cover <= 512) CS_LAUNCH(64, 8);
     else if (cover <= 1024) CS_LAUNCH(256, 4);
     else if (cover <= 2048) CS_LAUNCH(512, 4);
-    else CS_LAUNCH(1024, 4);
+    else CS_LAUNCH(512, 8);
 #undef CS_LAUNCH
 #undef CS_GO
 }

@@ -63,6 +63,8 @@ CASES = [
     ((2, 40, 4100), None), ((2, 33, 2104), None), ((2, 33, 2105), None), ((3, 50, 1080), None), ((2, 1000, 1000), None), ((1, 600, 4088), None),
     # rows beyond what a workgroup holds in registers: three passes with 16-byte accesses (512 and 1024 lanes), padded rows
     ((2, 6, 65536), None), ((1, 4, 100000), None), ((2, 3, 40000), (3 * 40008, 40008, 1)), ((1, 7, 32776), None),
+    # 16 385-32 768 elements: 512 lanes x 8 vectors, whole lines and ragged
+    ((2, 5, 20480), None), ((1, 6, 32768), None), ((2, 4, 20001), None), ((1, 3, 32760), (3 * 32776, 32776, 1)),
     ((5, 512, 512), None), ((3, 40, 400), None), ((2, 300, 512), None), ((3, 64, 264), None), ((2, 16, 504), (16 * 520, 520, 1)), ((2, 33, 512), None),
 ]
 
