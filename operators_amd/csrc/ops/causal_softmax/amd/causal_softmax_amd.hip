@@ -459,13 +459,16 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
 // Rows that the register kernels above do not take: longer than a workgroup
 // can hold (more than 32 768 elements), or RAGGED - rows that do not start on
 // 16-byte boundaries or whose length is no multiple of 8, which is what the
-// scores of an attention over an arbitrary number of keys look like.  Three
-// passes over the row with 16-byte accesses - the maximum (and the minimum,
-// for the choice of exponential), the sum of the exponentials, the quotients -
-// UNROLL vectors per lane in flight at a time.  The first pass brings the row
-// in from memory; the other two find it in L2 or in the Infinity Cache, so the
-// exponentials are formed twice but memory is read once.  Masked vectors are
-// written as zeros without being read.  One workgroup per row at a time.
+// scores of an attention over an arbitrary number of keys look like.  Two
+// passes over the row with 16-byte accesses, UNROLL vectors per lane in flight
+// at a time: the maximum (and the minimum, for the choice of exponential)
+// together with the sum of the exponentials, then the quotients.  The first
+// pass brings the row in from memory; the second finds it in L2 or in the
+// Infinity Cache, so the exponentials are formed twice but memory is read
+// once.  (With the sum in a pass of its own, after the maximum: [64, 512,
+// 65536] fp16 2163 us against 1691 us, [64, 512, 40000] 1288 against 1001 us.)
+// Masked vectors are written as zeros without being read.  One workgroup per
+// row at a time.
 // RAGGED: the vectors are the 16-byte aligned ones that cover the row, so the
 // first holds up to 7 elements of whatever lies in front of the row and the
 // last up to 7 of what lies behind it (both inside the same 16 bytes as an
@@ -494,34 +497,56 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
 
         // pass 1: maximum and minimum of the kept elements
         float mx = -__builtin_inff(), mn = __builtin_inff();
-        for (uint32_t v0 = threadIdx.x; v0 < keep_vecs; v0 += BS * UNROLL) {
-            u32x4 x[UNROLL];
+        // ... and the sum of the exponentials in the same sweep: each lane keeps the maximum of what it has seen so far
+        // (own_max) and the sum of exp(x - own_max) (own_sum), rescaled when the maximum grows.  The sum only feeds the
+        // denominator, so its exponentials are the plain v_exp_f32 of a rounded product (relative error below 2e-6
+        // wherever a term matters, no range limits: -inf and underflow give 0).
+        float own_max = -__builtin_inff(), own_sum = 0.0f;
+        {
+            constexpr float kL2e = 1.44269502162933349609375f;
+            auto exp_rough = [&](float d) { return __builtin_amdgcn_exp2f(d * kL2e); };
+            for (uint32_t v0 = threadIdx.x; v0 < keep_vecs; v0 += BS * UNROLL) {
+                u32x4 x[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint32_t v = v0 + u * BS;
-                x[u] = ld16(base + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);// re-reading the last kept vector changes no maximum
-            }
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint32_t v = v0 + u * BS;
+                    x[u] = ld16(base + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
+                }
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint32_t v = v0 + u * BS;
-                const uint32_t got = v < keep_vecs ? v : keep_vecs - 1;// the vector that was read
-                float f[8];
-                widen8<T>(x[u], f);
-                const bool edge = got < kept_from || got >= kept_to;
-                if (__builtin_amdgcn_ballot_w64(edge) != 0) {
-                    if (edge) {
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint32_t v = v0 + u * BS;
+                    if (v >= keep_vecs) continue;
+                    float f[8], low[8];
+                    widen8<T>(x[u], f);
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            const uint32_t p = got * 8 + e;
-                            if (p >= lo && p < hi) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+                    for (int e = 0; e < 8; ++e) low[e] = f[e];
+                    const bool edge = v < kept_from || v >= kept_to;
+                    if (__builtin_amdgcn_ballot_w64(edge) != 0) {
+                        if (edge) {// what is not kept: -inf for the maximum and the sum, +inf for the minimum
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const uint32_t p = v * 8 + e;
+                                const bool kept = p >= lo && p < hi;
+                                f[e] = kept ? f[e] : -__builtin_inff();
+                                low[e] = kept ? low[e] : __builtin_inff();
+                            }
                         }
                     }
-                }
-                if (!edge) {
+                    float top = f[0];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[e]), mn = fminf(mn, f[e]);
+                    for (int e = 1; e < 8; ++e) top = fmaxf(top, f[e]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) mn = fminf(mn, low[e]);
+                    const float grown = fmaxf(own_max, top);
+                    const float from = grown == -__builtin_inff() ? 0.0f : grown;// nothing finite yet: every term is exp(-inf) = 0
+                    float add = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) add += exp_rough(f[e] - from);
+                    own_sum = own_sum * (own_max == grown ? 1.0f : exp_rough(own_max - grown)) + add;
+                    own_max = grown;
                 }
             }
+            mx = own_max;
         }
         mx = block_max<WAVES>(mx, red, phase);
         const float lowest = mn - mx;
@@ -553,30 +578,12 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
             }
         };
 
-        // pass 2: the sum, each lane over its vectors in ascending order, then the workgroup tree
-        float part = 0.0f;
-        for (uint32_t v0 = threadIdx.x; v0 < keep_vecs; v0 += BS * UNROLL) {
-            u32x4 x[UNROLL];
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint32_t v = v0 + u * BS;
-                x[u] = ld16(base + static_cast<uint64_t>(v < keep_vecs ? v : keep_vecs - 1) * 8);
-            }
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint32_t v = v0 + u * BS;
-                if (v < keep_vecs) {
-                    float e8[8];
-                    exps(x[u], v, e8);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) part += e8[e];
-                }
-            }
-        }
+        // this lane's sum, brought from its own maximum to the row's (a lane that saw nothing finite holds 0), then the workgroup tree
+        const float part = own_max == mx ? own_sum : own_sum * __builtin_amdgcn_exp2f((own_max - mx) * 1.44269502162933349609375f);
         const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
         const float rcp = 1.0f / sum;
 
-        // pass 3: the quotients, and zeros behind them
+        // pass 2: the quotients, and zeros behind them
         const StreamOut<THROUGH> out(const_cast<uint16_t *>(base));
         for (uint32_t v0 = threadIdx.x; v0 < nvec; v0 += BS * UNROLL) {
             u32x4 x[UNROLL];
@@ -692,14 +699,14 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const bool even = (reinterpret_cast<uintptr_t>(data) & 1u) == 0;// elements lie on 2-byte boundaries
     const bool vec_ok = even && cover <= 4096 && d.seq < (1ull << 31) && (!ragged || d.total >= 16);
     // Rows of more than 32 768 elements (see causal_softmax_long).  Measured on MI355X, fp16, against the element kernel:
-    //   [64, 512, 65536]  2171 us (49 %) against 7230 us     [64, 512, 40000]  1293 against 4194 us
+    //   [64, 512, 65536]  1691 us (63 %) against 7230 us     [64, 512, 40000]  1001 against 4194 us
     const uint64_t vecs = cover;
     const bool long_ok = even && cover > 4096 && d.total + 8 < (1ull << 31) && rows < kFastDivLimit;
     if (long_ok) {
         const bool thr = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
         const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
         // a turn of the workgroup takes 4 vectors per lane: the lane count that covers the row in the fewest turns with the fewest idle lanes
-        // ([64, 512, 40000] fp16: 512 lanes 1293 us, 1024 lanes 1584 us, 256 lanes 1451 us; [64, 512, 65536]: 2320, 2171, 2394 us)
+        // ([64, 512, 40000] fp16: 512 lanes 996 us, 1024 lanes 1138 us; [64, 512, 65536]: 1752, 1684 us; [32, 512, 100000]: 1577, 1388 us)
         const int lanes = vecs < 8192 ? 512 : 1024;
         const unsigned g = static_cast<unsigned>(std::min<uint64_t>(rows, amd::max_grid_1d(1024)));
 #define CS_LONG_GO(BS, TH, RG) causal_softmax_long<T, BS, TH, RG><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)

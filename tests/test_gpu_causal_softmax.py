@@ -61,7 +61,7 @@ CASES = [
     ((32, 20, 333), None), ((3, 100, 1027), None), ((2, 50, 4099), None), ((2, 9, 33001), None), ((5, 60, 63), None), ((4, 7, 7), None),
     ((2, 130, 2050), None), ((3, 40, 2048), (40 * 2051, 2051, 1)), ((2, 5, 70003), None), ((6, 300, 301), None),
     ((2, 40, 4100), None), ((2, 33, 2104), None), ((2, 33, 2105), None), ((3, 50, 1080), None), ((2, 1000, 1000), None), ((1, 600, 4088), None),
-    # rows beyond what a workgroup holds in registers: three passes with 16-byte accesses (512 and 1024 lanes), padded rows
+    # rows beyond what a workgroup holds in registers: two passes with 16-byte accesses (512 and 1024 lanes), padded rows
     ((2, 6, 65536), None), ((1, 4, 100000), None), ((2, 3, 40000), (3 * 40008, 40008, 1)), ((1, 7, 32776), None),
     # 16 385-32 768 elements: 512 lanes x 8 vectors, whole lines and ragged
     ((2, 5, 20480), None), ((1, 6, 32768), None), ((2, 4, 20001), None), ((1, 3, 32760), (3 * 32776, 32776, 1)),
@@ -149,7 +149,7 @@ def test_infinities_and_long_tails(ctx):
 
 
 def test_infinities_and_long_tails_in_long_rows(ctx):
-    """The same special values in rows of 50 000 elements (the three-pass form)."""
+    """The same special values in rows of 50 000 elements (the two-pass form)."""
     rng = np.random.default_rng(79)
     vals = rng.standard_normal((2, 6, 50000)).astype(np.float32) * 2
     vals[0, :, 3] = -np.inf
