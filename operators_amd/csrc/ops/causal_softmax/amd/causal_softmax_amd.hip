@@ -469,10 +469,11 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
 // 65536] fp16 2163 us against 1691 us, [64, 512, 40000] 1288 against 1001 us.)
 // Masked vectors are written as zeros without being read.  One workgroup per
 // row at a time.
-// RAGGED: the vectors are the 16-byte aligned ones that cover the row, so the
-// first holds up to 7 elements of whatever lies in front of the row and the
-// last up to 7 of what lies behind it (both inside the same 16 bytes as an
-// element of the row, so reading them is safe).  Those foreign elements take
+// RAGGED: the vectors are the 16-byte aligned ones from the 128-byte boundary
+// in front of the row (so that a wavefront's 1 KiB per instruction is whole
+// lines) to the end of the row, so the first few hold elements of whatever
+// lies in front of the row and the last up to 7 of what lies behind it (all
+// inside the same 128 bytes as an element of the row, so reading them is safe).  Those foreign elements take
 // no part in the reductions, and the two edge vectors are written element by
 // element by the lane that owns them - the neighbouring bytes belong to other
 // rows, which other workgroups are working on.  (16-byte accesses at 2-byte
@@ -487,8 +488,8 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
     for (uint64_t r = blockIdx.x; r < rows; r += gridDim.x, phase ^= 1) {
         const uint32_t b = fast_quotient(static_cast<uint32_t>(r), by_seq), i = static_cast<uint32_t>(r) - b * seq;// fewer than 2^31 rows (see FastDiv)
         uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
-        // positions count from the 16-byte boundary at or in front of the row: the row is [lo, end), its kept part [lo, hi)
-        const uint32_t lo = RAGGED ? static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u) / 2 : 0u;
+        // positions count from the 128-byte boundary at or in front of the row: the row is [lo, end), its kept part [lo, hi)
+        const uint32_t lo = RAGGED ? static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 127u) / 2 : 0u;
         const uint16_t *base = row - lo;
         const uint32_t hi = lo + (total - seq + i + 1), end = lo + total;
         const uint32_t keep_vecs = (hi + 7) / 8, nvec = (end + 7) / 8;// vectors that hold kept elements; vectors that hold elements of the row
@@ -701,7 +702,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     // Rows of more than 32 768 elements (see causal_softmax_long).  Measured on MI355X, fp16, against the element kernel:
     //   [64, 512, 65536]  1691 us (63 %) against 7230 us     [64, 512, 40000]  1001 against 4194 us
     const uint64_t vecs = cover;
-    const bool long_ok = even && cover > 4096 && d.total + 8 < (1ull << 31) && rows < kFastDivLimit;
+    const bool long_ok = even && cover > 4096 && d.total + 64 < (1ull << 31) && rows < kFastDivLimit;
     if (long_ok) {
         const bool thr = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
         const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
@@ -712,8 +713,8 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
 #define CS_LONG_GO(BS, TH, RG) causal_softmax_long<T, BS, TH, RG><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)
 #define CS_LONG(BS)                                        \
     do {                                                   \
-        if (!aligned && thr) CS_LONG_GO(BS, true, true);   \
-        else if (!aligned) CS_LONG_GO(BS, false, true);    \
+        if (!in_lines && thr) CS_LONG_GO(BS, true, true);  \
+        else if (!in_lines) CS_LONG_GO(BS, false, true);   \
         else if (thr) CS_LONG_GO(BS, true, false);         \
         else CS_LONG_GO(BS, false, false);                 \
     } while (0)
