@@ -163,3 +163,26 @@ def test_causal_softmax_in_place(ctx):
         ctx.causal_softmax(part.view(1, seq, seq))
         torch.cuda.synchronize()
         assert same_bits(y[b], part), b
+
+
+def test_causal_softmax_ragged_rows_in_place(ctx):
+    """Rows of 21 001 elements: no row starts where another does within its
+    128-byte line, and element 2^31 lies in the last matrix.  The copy of a
+    matrix is placed at the same distance from a 128-byte boundary, so that the
+    lanes take the same vectors and the sums add in the same order."""
+    import torch
+
+    batch, seq, total = 6, 20001, 21001
+    y = randn16((batch, seq, total), 12, torch.float16)
+    parts = {}
+    for b in (0, 3, batch - 1):
+        start = (b * seq * total) % 64
+        buf = torch.zeros(start + seq * total, dtype=torch.float16, device="cuda")
+        parts[b] = buf[start:].view(1, seq, total)
+        parts[b].copy_(y[b])
+    ctx.causal_softmax(y)
+    torch.cuda.synchronize()
+    for b, part in parts.items():
+        ctx.causal_softmax(part)
+        torch.cuda.synchronize()
+        assert same_bits(y[b], part[0]), b
