@@ -117,6 +117,47 @@ def test_ragged_rows_leave_their_neighbours_alone(ctx, dt, start, shape, pitch):
     assert np.array_equal(before[~own], after[~own]), "elements outside the rows were written"
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_random_ragged_views(ctx, seed):
+    """Any row length, any pitch, any distance of the first row from a 128-byte
+    boundary, drawn at random: against the oracle, masked columns exact zeros,
+    every element outside the rows untouched."""
+    import torch
+
+    rng = np.random.default_rng(7100 + seed)
+    dt = str(rng.choice(["f16", "bf16"]))
+    total = int(np.exp(rng.uniform(np.log(1), np.log(70000))))
+    seq = int(min(total, rng.choice([1, 2, 3, 9, 40, 130, total])))
+    batch = int(rng.choice([1, 2, 3]))
+    while batch * seq * total > (1 << 21):
+        if seq > 4:
+            seq //= 2
+        else:
+            batch = 1
+            break
+    pitch = total + int(rng.choice([0, 0, 1, 3, 8, 11, 64]))
+    start = int(rng.integers(0, 64))
+    shape = (batch, seq, total)
+    y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 3, dt)
+    want = oracle.causal_softmax(y.copy(), dt)
+    span = start + batch * seq * pitch + 9
+    before = rng.integers(0, 0x3C00, span, dtype=np.uint16)
+    buf = to_torch(before, dt)
+    view = torch.as_strided(buf, shape, (seq * pitch, pitch, 1), storage_offset=start)
+    view.copy_(to_torch(y, dt).reshape(shape))
+    ctx.causal_softmax(view)
+    torch.cuda.synchronize()
+    got, after = to_codes(view), to_codes(buf)
+    what = f"seed {seed}: {shape} pitch {pitch} start {start} {dt}"
+    check(got, want, dt, what, max_frac=2e-2 if total > 4096 else 5e-3)
+    keep = np.arange(total)[None, :] <= total - seq + np.arange(seq)[:, None]
+    assert not got[..., ~keep].any(), what
+    own = np.zeros(span, bool)
+    rows = start + (np.arange(batch * seq) * pitch)[:, None] + np.arange(total)[None, :]
+    own[rows.ravel()] = True
+    assert np.array_equal(before[~own], after[~own]), what + ": elements outside the rows were written"
+
+
 def test_attention_scores_shape(ctx):
     """[heads, seq, total] = [8, 2048, 2048] fp16 with a scale typical of q.k/sqrt(d)."""
     rng = np.random.default_rng(77)
