@@ -458,6 +458,7 @@ def ops_table(ctx, args, gen):
         "N1c causal_softmax f16 [2048,512,512] (short rows: two to a wavefront)": lambda: [make_causal_softmax(ctx, 2048, 512, 512, f16, gen, "causal_softmax") for _ in range(2)],
         "N1d causal_softmax f16 [32,4095,4095] (ragged rows: every row starts at another 2-byte offset in its 128-byte line)": lambda: [make_causal_softmax(ctx, 32, 4095, 4095, f16, gen, "causal_softmax") for _ in range(2)],
         "N1e causal_softmax f16 [64,512,20480] (a chunk of 512 queries against 20480 keys: 512 lanes x 8 vectors)": lambda: [make_causal_softmax(ctx, 64, 512, 20480, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1f causal_softmax f16 [64,512,65536] (rows beyond a workgroup's registers: two passes over the row)": lambda: [make_causal_softmax(ctx, 64, 512, 65536, f16, gen, "causal_softmax") for _ in range(2)],
     }
     if args.only and "calibration" in args.only:
         # Not an operator of the library: a plain device-to-device copy of known
