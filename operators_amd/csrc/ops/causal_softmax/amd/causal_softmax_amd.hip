@@ -669,8 +669,8 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     auto *py = static_cast<uint16_t *>(data);
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
-    // Rows of up to 4096 elements are taken by single wavefronts (no barrier, no
-    // LDS), longer ones by 256 or 512 lanes.  Measured on MI355X, fp16 / bf16:
+    // Rows of up to 3072 elements are taken by single wavefronts (no barrier, no
+    // LDS), longer ones by 128, 256 or 512 lanes.  Measured on MI355X, fp16 / bf16 (rows of 4096 with one wavefront):
     //   [32, 4096, 4096]   one workgroup per row 264 / 261-266 us (76 %), 256 workgroups per
     //                      compute unit 267 / 267-274, 64 per unit 293 / 292-299; 128 or 256
     //                      lanes per row 264-288 / 261-270
@@ -808,7 +808,8 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     if (cover <= 64) CS_LAUNCH(64, 1);
     else if (cover <= 128) CS_LAUNCH(64, 2);
     else if (cover <= 256) CS_LAUNCH(64, 4);
-    else if (cover <= 512) CS_LAUNCH(64, 8);
+    else if (cover <= 384) CS_LAUNCH(64, 8);
+    else if (cover <= 512) CS_LAUNCH(128, 4);// two wavefronts: [32, 4096, 4096] bf16 261 against 269 us with 64 x 8 (fp16 261 / 265), [64, 512, 4096] bf16 84 / 88; at 384 vectors 64 x 8 is 1-2 % ahead
     else if (cover <= 1024) CS_LAUNCH(256, 4);
     else if (cover <= 2048) CS_LAUNCH(512, 4);
     else CS_LAUNCH(512, 8);
