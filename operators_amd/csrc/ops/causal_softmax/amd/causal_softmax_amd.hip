@@ -807,6 +807,8 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     //   [32, 4088, 4088]  278 (360)    [32, 4100, 4104]  281 (450)  [32, 2048, 2056]  74 (100)  [128, 1000, 1000]  72 (83)
     if (cover <= 64) CS_LAUNCH(64, 1);
     else if (cover <= 128) CS_LAUNCH(64, 2);
+    else if (cover <= 256 && cover > 192 && !ragged && !T::kPackedMinMax) CS_LAUNCH(128, 2);// bf16 rows of 2048 in whole lines: 257 against 269 us
+                                                                                              // (fp16 264 / 269 at seq 2048, 158 / 155 at seq 512; 1536 columns 173 / 150; ragged 2047: 299 / 281)
     else if (cover <= 256) CS_LAUNCH(64, 4);
     else if (cover <= 384) CS_LAUNCH(64, 8);
     else if (cover <= 512) CS_LAUNCH(128, 4);// two wavefronts: [32, 4096, 4096] bf16 261 against 269 us with 64 x 8 (fp16 261 / 265), [64, 512, 4096] bf16 84 / 88; at 384 vectors 64 x 8 is 1-2 % ahead
