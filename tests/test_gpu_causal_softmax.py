@@ -217,6 +217,41 @@ def test_infinities_and_long_tails(ctx):
     assert np.isnan(oracle.decode(got, "f16")[0, 5, 0])
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("start,shape", [(3, (2, 24, 77)), (5, (2, 12, 333)), (1, (2, 6, 4095)), (0, (2, 6, 4100)), (7, (2, 4, 20001)), (2, (2, 3, 33000)), (0, (2, 5, 2048))])
+def test_infinities_and_long_tails_in_ragged_rows(ctx, dt, start, shape):
+    """The special values at the places a ragged row treats apart: its first
+    and last elements (taken one per lane), the vector that straddles the mask,
+    and the body; rows that lie `start` elements behind a 128-byte boundary."""
+    import torch
+
+    batch, seq, total = shape
+    rng = np.random.default_rng(80 + total)
+    vals = rng.standard_normal(shape).astype(np.float32) * 2
+    vals[0, :, 0] = -np.inf                      # a first element
+    vals[0, :, total - 1] = -np.inf              # a last element (kept only in the last row)
+    vals[0, seq - 1, total - 3:] = -300.0        # a long tail at the end of the last row
+    vals[0, 0, :] = -np.inf                      # a row that is -inf throughout: NaN, as on the CPU
+    vals[1, :, 1] = -300.0                       # more than 126 below the maximum: the library exponential
+    vals[1, :, total // 2] = 200.0
+    vals[1, seq - 1, : total // 3] = -60000.0 if dt == "f16" else -3e38
+    if batch > 1 and seq > 2:
+        vals[1, 1, 2] = np.inf                   # +inf in the kept part: that row is NaN, the others are not
+    y = oracle.encode(vals, dt)
+    want = oracle.causal_softmax(y.copy(), dt).reshape(shape)
+    buf = torch.zeros(start + batch * seq * total + 8, dtype=torch.float16 if dt == "f16" else torch.bfloat16, device="cuda")
+    view = buf[start:start + batch * seq * total].view(shape)
+    view.copy_(to_torch(y, dt).reshape(shape))
+    ctx.causal_softmax(view)
+    torch.cuda.synchronize()
+    got = to_codes(view).reshape(shape)
+    nan_want, nan_got = np.isnan(oracle.decode(want.ravel(), dt)).reshape(shape), np.isnan(oracle.decode(got.ravel(), dt)).reshape(shape)
+    assert np.array_equal(nan_want, nan_got), "NaN in other places than on the CPU"
+    assert nan_got[0, 0, 0]
+    check(np.where(nan_got, 0, got).astype(np.uint16), np.where(nan_want, 0, want).astype(np.uint16), dt, f"specials {start} {shape} {dt}", max_frac=2e-2)
+    assert not buf[:start].any() and not buf[start + batch * seq * total:].any()
+
+
 def test_infinities_and_long_tails_in_long_rows(ctx):
     """The same special values in rows of 50 000 elements (the two-pass form)."""
     rng = np.random.default_rng(79)
