@@ -811,7 +811,8 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
                                                                                               // (fp16 264 / 269 at seq 2048, 158 / 155 at seq 512; 1536 columns 173 / 150; ragged 2047: 299 / 281)
     else if (cover <= 256) CS_LAUNCH(64, 4);
     else if (cover <= 384) CS_LAUNCH(64, 8);
-    else if (cover <= 512) CS_LAUNCH(128, 4);// two wavefronts: [32, 4096, 4096] bf16 261 against 269 us with 64 x 8 (fp16 261 / 265), [64, 512, 4096] bf16 84 / 88; at 384 vectors 64 x 8 is 1-2 % ahead
+    else if (cover <= 512) CS_LAUNCH(256, 2);// four wavefronts x 2 vectors.  [32, 4096, 4096] fp16 / bf16: 261 / 256 us; two x 4: 261 / 260; one x 8: 265 / 269.
+                                            // [64, 512, 4096]: 80 / 80, 82 / 83, 83 / 88.  At 384 vectors one wavefront x 8 is 1-2 % ahead; 512 lanes x 1 vector: 348 / 339 us.
     else if (cover <= 1024) CS_LAUNCH(256, 4);
     else if (cover <= 2048) CS_LAUNCH(512, 4);
     else CS_LAUNCH(512, 8);
