@@ -324,29 +324,71 @@ void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
 // kept length being a per-lane value; the sums are the same trees, one per
 // vector index k, added in the order the whole-wavefront tree adds its halves
 // (see segment_sum).
-template<typename T, int P, int NV, bool THROUGH>
+template<typename T, int P, int NV, bool THROUGH, bool RAGGED>
 __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint64_t groups, uint32_t seq, uint32_t total,
                                                               int64_t stride_b, int64_t stride_i, FastDiv by_groups_per_matrix,
                                                               uint32_t groups_per_matrix) {
     static_assert(NV >= 1 && NV <= 3 && P * NV <= kWave, "up to three vector indices, added as the whole-wavefront tree adds them");
     AMD_ARGS_NOW(y, groups, seq, total, stride_b, stride_i, arg_pair(by_groups_per_matrix), groups_per_matrix, gridDim.x);
     constexpr uint32_t RPW = kWave / P;// rows per wavefront
-    const uint32_t nvec = total / 8;
     const uint32_t sub = threadIdx.x % P, rr = threadIdx.x / P;
     const float neg_inf = -__builtin_inff();
     for (uint64_t g = blockIdx.x; g < groups; g += gridDim.x) {
         // group g of RPW rows: matrix b, rows i0 .. i0 + RPW - 1 (fewer than 2^31 groups, see FastDiv)
         const uint32_t b = fast_quotient(static_cast<uint32_t>(g), by_groups_per_matrix);
         const uint32_t i0 = (static_cast<uint32_t>(g) - b * groups_per_matrix) * RPW;
-        uint16_t *base = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i0) * stride_i;// the same for every lane
-        const uint32_t row_off = rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
-        const uint32_t keep = total - seq + i0 + rr + 1;
-        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = (keep - 1) / 8;
+        uint16_t *base = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i0) * stride_i;// the same for every lane unless RAGGED
+        // RAGGED (see causal_softmax_rows): the vectors are the whole 16-byte aligned ones inside the row, the up to 7
+        // elements in front of them and the up to 7 behind are taken one each by the row's first lanes.  All per lane
+        // here, and so is the row itself: a wavefront takes RPW consecutive rows of the whole tensor, whichever matrices
+        // they lie in (the host passes the divisor of seq and the number of rows in place of the groups' figures), the
+        // lanes behind the last row repeat it without storing.
+        const uint32_t row_off = RAGGED ? 0u : rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
+        struct Mine {
+            uint16_t *row, *body;// the row's first element and its first whole vector
+            uint32_t row_keep;   // columns kept of the row
+            uint32_t head, nvec; // elements in front of the vectors, vectors
+            uint32_t keep;       // columns kept of the vectors
+            bool valid;
+        };
+        const Mine mine = [&]() {
+            if constexpr (RAGGED) {
+                const uint64_t r = g * RPW + rr;
+                const bool valid = r < groups_per_matrix;
+                const uint32_t rc = valid ? static_cast<uint32_t>(r) : groups_per_matrix - 1;
+                const uint32_t rb = fast_quotient(rc, by_groups_per_matrix), ri = rc - rb * seq;
+                uint16_t *row = y + static_cast<int64_t>(rb) * stride_b + static_cast<int64_t>(ri) * stride_i;
+                const uint32_t row_keep = total - seq + ri + 1;
+                const uint32_t head = (8u - static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u) / 2) & 7u;
+                const uint32_t nvec = (total - head) / 8;
+                const uint32_t past = row_keep > head ? row_keep - head : 0u;
+                return Mine{row, row + head, row_keep, head, nvec, past < nvec * 8 ? past : nvec * 8, valid};
+            } else {
+                const uint32_t row_keep = total - seq + i0 + rr + 1;
+                return Mine{base, base, row_keep, 0u, total / 8, row_keep, true};
+            }
+        }();
+        const uint32_t row_keep = mine.row_keep, head = mine.head, nvec = mine.nvec, keep = mine.keep;
+        [[maybe_unused]] uint16_t *const row = mine.row;
+        [[maybe_unused]] const bool valid = mine.valid;
+        if constexpr (RAGGED) base = mine.body;
+        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = RAGGED && keep == 0 ? 0u : (keep - 1) / 8;
         u32x4 cur[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = sub + k * P;
             cur[k] = ld16_stream(reinterpret_cast<const uint8_t *>(base) + row_off + (v < last_vec ? v : last_vec) * 16);
+        }
+        // the row's elements in front of its vectors (lane sub takes column sub) and behind them
+        [[maybe_unused]] uint32_t col_t = 0;
+        [[maybe_unused]] bool mine_h = false, mine_t = false, kept_h = false, kept_t = false;
+        [[maybe_unused]] float x_h = 0.0f, x_t = 0.0f;
+        if constexpr (RAGGED) {
+            col_t = head + nvec * 8 + sub;
+            mine_h = sub < head, mine_t = col_t < total;// P >= 8 lanes, at most 7 elements at either end
+            kept_h = mine_h && sub < row_keep, kept_t = mine_t && col_t < row_keep;
+            if (kept_h) x_h = T::one(row[sub]);
+            if (kept_t) x_t = T::one(row[col_t]);
         }
 
         float mx = neg_inf, mn = __builtin_inff();
@@ -382,10 +424,25 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
                 }
             }
         }
+        if constexpr (RAGGED) {
+            if (kept_h) mx = fmaxf(mx, x_h), mn = fminf(mn, x_h);
+            if (kept_t) mx = fmaxf(mx, x_t), mn = fminf(mn, x_t);
+        }
         mx = segment_max<P>(mx);
 
         const float lowest = mn - mx;// +inf - max for a lane without kept elements: passes the test below
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
+        [[maybe_unused]] float e_h = 0.0f, e_t = 0.0f;
+        if constexpr (RAGGED) {
+            if (lean) {
+                e_h = exp_nonpositive(x_h - mx), e_t = exp_nonpositive(x_t - mx);
+            } else {
+                float slow[8] = {x_h, x_t, mx, mx, mx, mx, mx, mx};
+                exp_any8(slow, mx);
+                e_h = slow[0], e_t = slow[1];
+            }
+            e_h = kept_h ? e_h : 0.0f, e_t = kept_t ? e_t : 0.0f;
+        }
         float tree[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -417,6 +474,9 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
 #pragma unroll
                 for (int e = 0; e < 8; ++e) part += f[k][e];
             }
+            if constexpr (RAGGED) {
+                if (k == 0) part += e_h + e_t;
+            }
             tree[k] = segment_sum<P>(part);
         }
         // the order in which the whole-wavefront tree adds these groups of lanes: upper to lower, pairwise
@@ -425,7 +485,7 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
         if constexpr (NV == 3) sum = tree[2] + (tree[1] + tree[0]);
         const float rcp = 1.0f / sum;
 
-        const StreamOut<THROUGH> out(base);
+        const StreamOut<THROUGH> out(RAGGED ? y : base);// RAGGED: not used, every lane has a base of its own
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = sub + k * P;
@@ -452,7 +512,19 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
                     }
                 }
             }
-            if (v < nvec) out.st16(row_off + v * 16, packed);
+            if constexpr (RAGGED) {
+                if (valid && v < nvec) st16_stream(base + v * 8, packed);
+            } else {
+                if (v < nvec) out.st16(row_off + v * 16, packed);
+            }
+        }
+        if constexpr (RAGGED) {
+            auto one = [&](float e) {
+                const float q = e * rcp;
+                return static_cast<uint16_t>(T::narrow2_fast(__builtin_fmaf(__builtin_fmaf(-sum, q, e), rcp, q), 0.0f) & 0xFFFFu);
+            };
+            if (valid && mine_h) row[sub] = kept_h ? one(e_h) : uint16_t{0};
+            if (valid && mine_t) row[col_t] = kept_t ? one(e_t) : uint16_t{0};
         }
     }
 }
@@ -738,7 +810,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     //   [32768, 128, 128]  1385 -> 291 us                    [131072, 64, 64]  2765 -> 324 us
     // with 2048 wavefronts per compute unit striding over the groups (128 / 512 / 8192 per unit: 382 / 348 / 351 us
     // at 256 columns with 32 lanes per row).
-    if (aligned && nvec <= 64 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
+    if ((aligned || d.total >= 16) && nvec <= 64 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
         // Lanes per row x vectors per lane: the pair that wastes the fewest lanes, the fewer lanes per row (more
         // rows per wavefront) when two waste the same, among those whose rows per wavefront divide the matrix's
         // row count.  More than one vector per lane spares the rows that the mask cuts short the work of the
@@ -746,27 +818,31 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         //   [2048, 512, 512]   32 x 2  265   16 x 4  274          [8192, 256, 256]   16 x 2  274   32 x 1  344   8 x 4  286
         //   [4096, 384, 384]   16 x 3  318   32 x 2  341          [32768, 128, 128]   8 x 2  296   16 x 1  344
         //   [16384, 192, 192]  16 x 2  338    8 x 3  339   32 x 1  516
+        const bool together = in_lines;// rows in whole lines: RPW rows of one matrix per wavefront; others: the ragged form, which measures
+                                       // better for them also where they lie on 16-byte boundaries ([2048, 504, 504] fp16 345 against 411 us,
+                                       // [8192, 120, 120] 89 against 164 us; in whole lines it is the other way round: [2048, 512, 512] 335 against 277 us)
         unsigned lanes = 0, per_lane = 0;
         for (const unsigned p : {8u, 16u, 32u}) {
             for (const unsigned v : {1u, 2u, 3u}) {
-                const bool fits = p * v >= nvec && p * v <= kWave && d.seq % (kWave / p) == 0;
+                const bool fits = p * v >= nvec && p * v <= kWave && (!together || d.seq % (kWave / p) == 0);// ragged rows: any consecutive rows
                 if (fits && (lanes == 0 || p * v < lanes * per_lane)) lanes = p, per_lane = v;
             }
         }
         if (lanes != 0) {
             const unsigned rpw = kWave / lanes;
-            const uint64_t groups = rows / rpw;
+            const uint64_t groups = ceil_div(rows, rpw);
             const uint32_t gpm = static_cast<uint32_t>(d.seq / rpw);
             const uint64_t capg = static_cast<uint64_t>(d.cu_count) * 2048;
             const unsigned g = static_cast<unsigned>(std::min(groups, capg));
+#define CS_SHORT_GO(P, NV, TH, RG)                                                                                             \
+    causal_softmax_short<T, P, NV, TH, RG><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
+                                                                    d.stride_b, d.stride_i, RG ? by_seq : fast_div(gpm), RG ? static_cast<uint32_t>(rows) : gpm)
 #define CS_SHORT(P, NV)                                                                                                        \
     do {                                                                                                                       \
-        if (through)                                                                                                           \
-            causal_softmax_short<T, P, NV, true><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
-                                                                          d.stride_b, d.stride_i, fast_div(gpm), gpm);         \
-        else                                                                                                                   \
-            causal_softmax_short<T, P, NV, false><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
-                                                                           d.stride_b, d.stride_i, fast_div(gpm), gpm);        \
+        if (through && together) CS_SHORT_GO(P, NV, true, false);                                                              \
+        else if (through) CS_SHORT_GO(P, NV, true, true);                                                                      \
+        else if (together) CS_SHORT_GO(P, NV, false, false);                                                                   \
+        else CS_SHORT_GO(P, NV, false, true);                                                                                  \
     } while (0)
             switch (lanes * 10 + per_lane) {
                 case 81: CS_SHORT(8, 1); break;
@@ -779,6 +855,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
                 default: CS_SHORT(32, 2); break;
             }
 #undef CS_SHORT
+#undef CS_SHORT_GO
             return;
         }
     }
