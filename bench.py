@@ -70,7 +70,7 @@ def parse():
     ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ops-table", action="store_true", help="skip the per-operator table (C1-C4 and per-op C5)")
-    ap.add_argument("--only", default=None, help="time a single named entry of the per-operator table and exit (for profiling)")
+    ap.add_argument("--only", default=None, help="run a single named entry of the per-operator table and exit (for profiling: exactly --warmup + --steps calls, no settling, so its time includes the clock ramp after idle and reads 4-12 %% above the table's steady figure)")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens of the chain (default: the full configuration)")
     return ap.parse_args()
 
