@@ -818,15 +818,22 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         //   [2048, 512, 512]   32 x 2  265   16 x 4  274          [8192, 256, 256]   16 x 2  274   32 x 1  344   8 x 4  286
         //   [4096, 384, 384]   16 x 3  318   32 x 2  341          [32768, 128, 128]   8 x 2  296   16 x 1  344
         //   [16384, 192, 192]  16 x 2  338    8 x 3  339   32 x 1  516
-        const bool together = in_lines;// rows in whole lines: RPW rows of one matrix per wavefront; others: the ragged form, which measures
+        bool together = in_lines;// rows in whole lines: RPW rows of one matrix per wavefront; others: the ragged form, which measures
                                        // better for them also where they lie on 16-byte boundaries ([2048, 504, 504] fp16 345 against 411 us,
                                        // [8192, 120, 120] 89 against 164 us; in whole lines it is the other way round: [2048, 512, 512] 335 against 277 us)
         unsigned lanes = 0, per_lane = 0;
-        for (const unsigned p : {8u, 16u, 32u}) {
-            for (const unsigned v : {1u, 2u, 3u}) {
-                const bool fits = p * v >= nvec && p * v <= kWave && (!together || d.seq % (kWave / p) == 0);// ragged rows: any consecutive rows
-                if (fits && (lanes == 0 || p * v < lanes * per_lane)) lanes = p, per_lane = v;
+        const auto pick = [&]() {
+            for (const unsigned p : {8u, 16u, 32u}) {
+                for (const unsigned v : {1u, 2u, 3u}) {
+                    const bool fits = p * v >= nvec && p * v <= kWave && (!together || d.seq % (kWave / p) == 0);// ragged rows: any consecutive rows
+                    if (fits && (lanes == 0 || p * v < lanes * per_lane)) lanes = p, per_lane = v;
+                }
             }
+        };
+        pick();
+        if (lanes == 0 && together && d.total >= 16) {// a matrix's rows do not fill wavefronts (seq = 1: decoding): any consecutive rows then
+            together = false;
+            pick();
         }
         if (lanes != 0) {
             const unsigned rpw = kWave / lanes;

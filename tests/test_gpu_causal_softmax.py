@@ -60,6 +60,8 @@ CASES = [
     # of keys produces): the aligned vectors that cover a row, its two edge vectors written element by element; every workgroup size
     ((32, 20, 333), None), ((3, 100, 1027), None), ((2, 50, 4099), None), ((2, 9, 33001), None), ((5, 60, 63), None), ((4, 7, 7), None),
     ((2, 130, 2050), None), ((3, 40, 2048), (40 * 2051, 2051, 1)), ((2, 5, 70003), None), ((6, 300, 301), None),
+    # short rows in whole lines whose matrices do not fill wavefronts (decoding: one row per matrix), any consecutive rows per wavefront
+    ((37, 1, 320), None), ((9, 3, 128), None), ((50, 7, 512), None), ((5, 1, 64), (64 * 3, 64, 1)), ((33, 1, 300), None), ((3, 127, 128), None),
     ((2, 40, 4100), None), ((2, 33, 2104), None), ((2, 33, 2105), None), ((3, 50, 1080), None), ((2, 1000, 1000), None), ((1, 600, 4088), None),
     # rows beyond what a workgroup holds in registers: two passes with 16-byte accesses (512 and 1024 lanes), padded rows
     ((2, 6, 65536), None), ((1, 4, 100000), None), ((2, 3, 40000), (3 * 40008, 40008, 1)), ((1, 7, 32776), None),
