@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_HANDLE_H
 #define INFINIOP_AMD_FWD_HANDLE_H
 #include "infiniop.h"
+#include "export.h"
 #endif

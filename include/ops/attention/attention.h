@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_OPS_ATTENTION_ATTENTION_H
 #define INFINIOP_AMD_FWD_OPS_ATTENTION_ATTENTION_H
 #include "../../infiniop.h"
+#include "../../export.h"
 #endif

@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_OPS_CAUSAL_SOFTMAX_CAUSAL_SOFTMAX_H
 #define INFINIOP_AMD_FWD_OPS_CAUSAL_SOFTMAX_CAUSAL_SOFTMAX_H
 #include "../../infiniop.h"
+#include "../../export.h"
 #endif

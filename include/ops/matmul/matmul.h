@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_OPS_MATMUL_MATMUL_H
 #define INFINIOP_AMD_FWD_OPS_MATMUL_MATMUL_H
 #include "../../infiniop.h"
+#include "../../export.h"
 #endif

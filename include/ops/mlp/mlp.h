@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_OPS_MLP_MLP_H
 #define INFINIOP_AMD_FWD_OPS_MLP_MLP_H
 #include "../../infiniop.h"
+#include "../../export.h"
 #endif

@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_OPS_RANDOM_SAMPLE_RANDOM_SAMPLE_H
 #define INFINIOP_AMD_FWD_OPS_RANDOM_SAMPLE_RANDOM_SAMPLE_H
 #include "../../infiniop.h"
+#include "../../export.h"
 #endif

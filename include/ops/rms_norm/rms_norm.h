@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_OPS_RMS_NORM_RMS_NORM_H
 #define INFINIOP_AMD_FWD_OPS_RMS_NORM_RMS_NORM_H
 #include "../../infiniop.h"
+#include "../../export.h"
 #endif

@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_OPS_ROTARY_EMBEDDING_ROTARY_EMBEDDING_H
 #define INFINIOP_AMD_FWD_OPS_ROTARY_EMBEDDING_ROTARY_EMBEDDING_H
 #include "../../infiniop.h"
+#include "../../export.h"
 #endif

@@ -4,4 +4,5 @@
 #ifndef INFINIOP_AMD_FWD_TENSOR_TENSOR_DESCRIPTOR_H
 #define INFINIOP_AMD_FWD_TENSOR_TENSOR_DESCRIPTOR_H
 #include "../infiniop.h"
+#include "../export.h"
 #endif

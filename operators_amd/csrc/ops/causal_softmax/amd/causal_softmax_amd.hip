@@ -88,8 +88,11 @@ void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
     AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
     constexpr int WAVES = BS / kWave;
     // the form held to 128 registers has none to spare for the packed comparisons' second pair of accumulators
-    constexpr bool kPacked = T::kPackedMinMax && !(RAGGED && BS == 512 && NV == 8);
+    constexpr bool kPacked = T::kPackedMinMax && !(BS == 512 && NV == 8);
     __shared__ float red[4 * WAVES];// two slot sets for the maxima, two for the sums
+    // the same form, RAGGED: the first wavefront's end elements wait in LDS while the exponentials of the vectors are formed
+    constexpr bool kStashEnds = RAGGED && BS == 512 && NV == 8;
+    __shared__ float ends[kStashEnds ? kWave : 1];
     const float neg_inf = -__builtin_inff();
 
     struct Row {
@@ -207,6 +210,9 @@ void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
         }
         if constexpr (RAGGED) {
             if (end_kept) mx = fmaxf(mx, end_x), mn = fminf(mn, end_x);
+            if constexpr (kStashEnds) {
+                if (threadIdx.x < kWave) ends[threadIdx.x] = end_x;// read back by the same lane, behind the barrier below
+            }
         }
         mx = block_max<WAVES>(mx, red, phase);
 
@@ -249,6 +255,7 @@ void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
         [[maybe_unused]] float end_f = 0.0f;
         if constexpr (RAGGED) {
             if (threadIdx.x < kWave) {
+                if constexpr (kStashEnds) end_x = ends[threadIdx.x];
                 if (lean) {
                     end_f = exp_nonpositive(end_x - mx);
                 } else {
@@ -712,6 +719,151 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
     }
 }
 
+// Rows of 32 769 to 131 072 elements on 16-byte boundaries: the row is read
+// once and held in registers as raw 16-bit words - 12, 16 or 20 vectors per
+// lane of a 512-lane workgroup up to 81 920 elements (two workgroups fit a
+// compute unit, so one row's arithmetic runs under the other's loads and
+// stores), 12, 14 or 16 vectors per lane of a 1024-lane workgroup beyond - and
+// the three sweeps (the maximum, the sum, the quotients) widen it anew each
+// time.  Holding the exponentials instead, as causal_softmax_rows does, would
+// take twice the registers; forming them twice costs arithmetic, and at this
+// length arithmetic is what the kernel is short of (at 100 % of the memory
+// rate a compute unit has about 31 vector-instruction slots per element; the
+// full-precision exponential takes 12 and would be needed twice).  So both
+// sweeps use the hardware exp2 of one fused multiply-add,
+// x * log2(e) - max * log2(e): relative error below 3e-6 where a term is not
+// negligible, the same in the sum and in the quotient - well inside what the
+// reference's own left-to-right fp32 sum of tens of thousands of terms leaves
+// open (about 1e-5), and far below half a unit of either 16-bit format.  No
+// range limits: -inf and underflow give 0, NaN stays NaN.
+// Measured on MI355X, fp16, against the two-pass kernel above (which read 30 %
+// of such rows a second time from memory), us:
+//   [64, 512, 40000]   872 /  998     [64, 512, 65536]  1641 / 1677
+//   [64, 256, 120000] 1561 / 1605     [64, 256, 131072] 1651 / 1723
+// A row stride of 64 KiB or more that is a power of two costs every form here
+// about a tenth: the rows that are in flight together then lie in the same
+// memory channels and banks.  [64, 512, 65536] with each row 1 KiB further
+// from the one before it: 1453 us (74 %) against 1641 us (65 %); [64, 512,
+// 32768]: 764 against 815 us.  (Turning the order in which a workgroup's lanes
+// take the row's vectors, by 1 KiB per row, changes nothing: 1647 us - the
+// whole row is in flight at once either way.)
+template<typename T, int BS, int NV, bool THROUGH>
+__global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(4)))
+void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total, int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
+    AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
+    constexpr int WAVES = BS / kWave;
+    constexpr float kL2e = 1.44269502162933349609375f;
+    __shared__ float red[4 * WAVES];
+    const float neg_inf = -__builtin_inff();
+    const uint32_t nvec = total / 8;
+    int phase = 0;
+    for (uint64_t r = blockIdx.x; r < rows; r += gridDim.x, phase ^= 1) {
+        const uint32_t b = fast_quotient(static_cast<uint32_t>(r), by_seq), i = static_cast<uint32_t>(r) - b * seq;// fewer than 2^31 rows (see FastDiv)
+        uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
+        const uint32_t keep = total - seq + i + 1;
+        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = (keep - 1) / 8;
+        auto vector_at = [&](int k) { return static_cast<uint32_t>(k * BS + threadIdx.x); };
+        u32x4 cur[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = vector_at(k);
+            cur[k] = ld16_stream(row + static_cast<uint64_t>(v < last_vec ? v : last_vec) * 8);// masked vectors re-read the last kept one
+        }
+        // the maximum; the one vector that straddles the mask enters element by element
+        float mx = neg_inf;
+        [[maybe_unused]] typename T::pair mx2;
+        if constexpr (T::kPackedMinMax) mx2 = T::splat(neg_inf);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = vector_at(k);
+            const bool straddles = tail != 0 && v + 1 == keep_vecs;
+            if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                if (straddles) {
+                    float f[8];
+                    widen8<T>(cur[k], f);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (static_cast<uint32_t>(e) < tail) mx = fmaxf(mx, f[e]);
+                    }
+                }
+            }
+            if (v >= keep_vecs || straddles) continue;
+            if constexpr (T::kPackedMinMax) {
+                const uint32_t w[4] = {cur[k].x, cur[k].y, cur[k].z, cur[k].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) mx2 = T::max2(mx2, T::as_pair(w[j]));
+            } else {
+                float f[8];
+                widen8<T>(cur[k], f);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) mx = fmaxf(mx, f[e]);
+            }
+        }
+        if constexpr (T::kPackedMinMax) mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
+        mx = block_max<WAVES>(mx, red, phase);
+        // exp(x - max) as exp2(x * log2(e) - max * log2(e)); a row whose maximum is +-inf goes the plain way (inf - inf must give NaN)
+        const bool finite_max = __builtin_fabsf(mx) < __builtin_inff();
+        const float m2 = mx * kL2e;
+        auto exps = [&](u32x4 raw, float(&e8)[8]) {
+            widen8<T>(raw, e8);
+            if (finite_max) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) e8[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(e8[e], kL2e, -m2));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) e8[e] = __builtin_amdgcn_exp2f((e8[e] - mx) * kL2e);
+            }
+        };
+#pragma unroll
+        for (int k = 0; k < NV; ++k) asm volatile("" : "+v"(cur[k]));// the sweeps widen the raw words anew: no widened copy is kept
+        float part = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = vector_at(k);
+            if (v >= keep_vecs) continue;
+            float e8[8];
+            exps(cur[k], e8);
+            const bool straddles = tail != 0 && v + 1 == keep_vecs;
+            if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                if (straddles) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) e8[e] = static_cast<uint32_t>(e) < tail ? e8[e] : 0.0f;
+                }
+            }
+            part += ((e8[0] + e8[1]) + (e8[2] + e8[3])) + ((e8[4] + e8[5]) + (e8[6] + e8[7]));
+        }
+        const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
+        const float rcp = 1.0f / sum;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) asm volatile("" : "+v"(cur[k]));
+        const StreamOut<THROUGH> out(row);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const uint32_t v = vector_at(k);
+            u32x4 packed{0, 0, 0, 0};
+            if (v < keep_vecs) {
+                float e8[8];
+                exps(cur[k], e8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) e8[e] *= rcp;
+                packed = narrow8_unit_range<T>(e8);
+                const bool straddles = tail != 0 && v + 1 == keep_vecs;
+                if (__builtin_amdgcn_ballot_w64(straddles) != 0) {
+                    if (straddles) {// its masked tail is zero whatever the row turned into
+                        uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            if (static_cast<uint32_t>(e) >= tail) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                        }
+                        packed = u32x4{w[0], w[1], w[2], w[3]};
+                    }
+                }
+            }
+            if (v < nvec) out.st16(v * 16, packed);
+        }
+    }
+}
+
 // Any row length, any alignment: three passes over the row with element
 // accesses; the later passes find the row in cache.
 template<typename T>
@@ -779,6 +931,25 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     if (long_ok) {
         const bool thr = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
         const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
+        if (aligned && nvec <= 16 * 1024) {// up to 131 072 elements: held in registers, read once (see causal_softmax_held)
+            const unsigned lanes = nvec <= 20 * 512 ? 512 : 1024;
+            const unsigned g = static_cast<unsigned>(std::min<uint64_t>(rows, amd::max_grid_1d(lanes)));
+#define CS_HELD_GO(BS, NV, TH) causal_softmax_held<T, BS, NV, TH><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)
+#define CS_HELD(BS, NV)               \
+    do {                              \
+        if (thr) CS_HELD_GO(BS, NV, true); \
+        else CS_HELD_GO(BS, NV, false);    \
+    } while (0)
+            if (nvec <= 12 * 512) CS_HELD(512, 12);
+            else if (nvec <= 16 * 512) CS_HELD(512, 16);
+            else if (nvec <= 20 * 512) CS_HELD(512, 20);
+            else if (nvec <= 12 * 1024) CS_HELD(1024, 12);
+            else if (nvec <= 14 * 1024) CS_HELD(1024, 14);
+            else CS_HELD(1024, 16);
+#undef CS_HELD
+#undef CS_HELD_GO
+            return;
+        }
         // a turn of the workgroup takes 4 vectors per lane: the lane count that covers the row in the fewest turns with the fewest idle lanes
         // ([64, 512, 40000] fp16: 512 lanes 996 us, 1024 lanes 1138 us; [64, 512, 65536]: 1752, 1684 us; [32, 512, 100000]: 1577, 1388 us)
         const int lanes = vecs < 8192 ? 512 : 1024;

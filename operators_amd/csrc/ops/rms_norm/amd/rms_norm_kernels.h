@@ -32,6 +32,19 @@ using namespace amd;
 // ---- weight row access ----------------------------------------------------------
 struct WF32 {
     typedef float scalar;
+    struct raw {
+        f32x4 a, b;
+    };
+    // eight weights through a buffer descriptor of the weight row: a per-lane byte offset plus a wavefront-uniform one
+    __device__ static __forceinline__ raw fetch(__amdgpu_buffer_rsrc_t row, uint32_t lane, uint32_t ahead) {
+        const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(row, static_cast<int>(lane), static_cast<int>(ahead), 0);
+        const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(row, static_cast<int>(lane + 16), static_cast<int>(ahead), 0);
+        return raw{__builtin_bit_cast(f32x4, a), __builtin_bit_cast(f32x4, b)};
+    }
+    __device__ static __forceinline__ void spread(const raw &r, float (&g)[8]) {
+        g[0] = r.a.x, g[1] = r.a.y, g[2] = r.a.z, g[3] = r.a.w;
+        g[4] = r.b.x, g[5] = r.b.y, g[6] = r.b.z, g[7] = r.b.w;
+    }
     __device__ static __forceinline__ void load8(const void *w, uint32_t vec, float (&g)[8]) {
         const float *p = static_cast<const float *>(w) + static_cast<uint64_t>(vec) * 8;
         const f32x4 a = ld16f(p), b = ld16f(p + 4);
@@ -43,6 +56,11 @@ struct WF32 {
 template<typename T>
 struct W16 {
     typedef uint16_t scalar;
+    typedef u32x4 raw;
+    __device__ static __forceinline__ raw fetch(__amdgpu_buffer_rsrc_t row, uint32_t lane, uint32_t ahead) {
+        return __builtin_amdgcn_raw_buffer_load_b128(row, static_cast<int>(lane), static_cast<int>(ahead), 0);
+    }
+    __device__ static __forceinline__ void spread(const raw &r, float (&g)[8]) { widen8<T>(r, g); }
     __device__ static __forceinline__ void load8(const void *w, uint32_t vec, float (&g)[8]) {
         widen8<T>(ld16(static_cast<const uint16_t *>(w) + static_cast<uint64_t>(vec) * 8), g);
     }
@@ -345,6 +363,163 @@ __global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y
         load_row(row + hop, xn, bn);
         finish_row(row, xv, bv, 0);
         row += hop;
+    }
+}
+
+// ---- wide rows ----------------------------------------------------------------
+// Rows of more than 32 768 elements, and the fused form from 10 240: one
+// workgroup per compute unit, as many lanes as the row has vectors for (up to
+// 1024), NV raw vectors per lane, one row at a time.  What differs from
+// rms_norm_rows:
+// - the lane count is the launch's, so that no lane is idle whatever the width;
+// - loads go through a buffer descriptor of one row (or of the weight row): a
+//   lane's address is one per-lane byte offset plus a wavefront-uniform one, no
+//   vector register carries an address across the loop over rows, and vectors
+//   behind the row's end read as zeros without a test.  (rms_norm_rows at eight
+//   vectors per lane kept 48 registers of addresses alive and spilled them.)
+//   Stores take the same descriptor but the whole offset per lane: a 16-byte
+//   buffer store whose uniform offset comes from a scalar register was seen,
+//   on MI355X, to pick up the value that the next instructions write into its
+//   first data register (about one row in four of [512, 32768] had a few
+//   elements wrong) - the compiler separates such a store from a write to its
+//   data only when that offset is a constant;
+// - the widened values are formed anew for the scaling (kept from the squares
+//   they would take 8 registers per vector);
+// - weights from memory (rows whose fp32 weights do not fit LDS) are requested
+//   WBATCH vectors at a time as raw words, the first batch in front of the
+//   reduction, and the weight type is resolved once, outside the loop over rows.
+// The sum of squares is row_sum_any's, in its order: the same bits as every
+// other form.
+// Measured on MI355X, bf16 with fp32 weights, against rms_norm_rows (us):
+//   fused [8192, 16384]  181.6 / 187.5     fused [8192, 12288]  134.4 / 138.7
+//   fused [8192, 10240]  117.8 / 119.5     fused [4096, 32768]  183.0 / 192.1
+//   plain [4096, 32768]   94.3 /  93.7 (so the plain form stays with rms_norm_rows up to there)
+// (Two halves of a workgroup on rows of their own, each with a counting
+// barrier in LDS and both sharing the staged weights, measured slower: plain
+// [4096, 32768] 100.2 us, fused 191.6 us.)
+template<typename T, int NV, int WHOME, bool THROUGH, bool ADD, int WBATCH = 4>
+__global__ __launch_bounds__(1024) void rms_norm_wide(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
+                                                      uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
+                                                      Residual<ADD> res) {
+    RMS_ARGS_NOW(gridDim.x, blockDim.x);
+    constexpr int MAX_WAVES = 1024 / kWave;
+    __shared__ float red[2 * NV * MAX_WAVES];
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
+    f32x4 *w_lo = reinterpret_cast<f32x4 *>(dyn_lds);
+    const uint32_t nvec = d / 8;
+    f32x4 *w_hi = w_lo + nvec;
+    const uint32_t bs = blockDim.x, waves = bs / kWave;
+    const uint32_t lane16 = threadIdx.x * 16;
+    constexpr uint32_t kNt = 2, kOut = THROUGH ? (16 | 2) : 2;// cache policies: nt; sc1 nt
+    const auto row_of = [&](const uint16_t *base, uint64_t row, int64_t stride) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(base + static_cast<int64_t>(row) * stride), 0, static_cast<int>(d * 2), 0x00020000);
+    };
+
+    if constexpr (WHOME == kWLds) {// the weight row, staged once as fp32
+        auto stage = [&](auto tag) {
+            typedef decltype(tag) W;
+            constexpr uint32_t kWVec = 8 * sizeof(typename W::scalar);
+            const __amdgpu_buffer_rsrc_t w_row = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(w), 0, static_cast<int>(d * sizeof(typename W::scalar)), 0x00020000);
+            typename W::raw wr[NV];
+#pragma unroll
+            for (int k = 0; k < NV; ++k) wr[k] = W::fetch(w_row, threadIdx.x * kWVec, k * bs * kWVec);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * bs + threadIdx.x;
+                float g[8];
+                W::spread(wr[k], g);
+                if (v < nvec) {
+                    w_lo[v] = f32x4{g[0], g[1], g[2], g[3]};
+                    w_hi[v] = f32x4{g[4], g[5], g[6], g[7]};
+                }
+            }
+        };
+        if (w_kind == kWKindF32) stage(WF32{});
+        else if (w_kind == kWKindF16) stage(W16<F16Ref>{});
+        else stage(W16<BF16Rne>{});
+        __syncthreads();
+    }
+
+    auto serve = [&](auto wtag) {
+        typedef decltype(wtag) W;
+        constexpr int WB = WHOME == kWLds ? 1 : (NV < WBATCH ? NV : WBATCH);
+        constexpr uint32_t kWVec = 8 * sizeof(typename W::scalar);
+        [[maybe_unused]] const __amdgpu_buffer_rsrc_t w_row =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(w), 0, static_cast<int>(d * sizeof(typename W::scalar)), 0x00020000);
+        int phase = 0;
+        for (uint64_t row = blockIdx.x; row < n; row += gridDim.x, phase ^= 1) {
+            const __amdgpu_buffer_rsrc_t xr = row_of(x, row, stride_x);
+            u32x4 cur[NV];
+#pragma unroll
+            for (int k = 0; k < NV; ++k) cur[k] = __builtin_amdgcn_raw_buffer_load_b128(xr, static_cast<int>(lane16), static_cast<int>(k * bs * 16), kNt);
+            if constexpr (ADD) {// cur += b, rounded as Add rounds, and out to c
+                const __amdgpu_buffer_rsrc_t br = row_of(res.b, row, res.stride_b), cr = row_of(res.c, row, res.stride_c);
+                u32x4 other[NV];
+#pragma unroll
+                for (int k = 0; k < NV; ++k) other[k] = __builtin_amdgcn_raw_buffer_load_b128(br, static_cast<int>(lane16), static_cast<int>(k * bs * 16), kNt);
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    float p[8], q[8];
+                    widen8<T>(cur[k], p);
+                    widen8<T>(other[k], q);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) p[i] += q[i];
+                    cur[k] = narrow8<T>(p);
+                    __builtin_amdgcn_raw_buffer_store_b128(cur[k], cr, static_cast<int>(lane16 + k * bs * 16), 0, kOut);// behind the row's end: dropped
+                }
+            }
+            [[maybe_unused]] typename W::raw wr[WB];
+            [[maybe_unused]] auto fetch_weights = [&](int k0) {
+#pragma unroll
+                for (int j = 0; j < WB; ++j) {
+                    if (k0 + j < NV) wr[j] = W::fetch(w_row, threadIdx.x * kWVec, (k0 + j) * bs * kWVec);
+                }
+            };
+            if constexpr (WHOME == kWGlobal) fetch_weights(0);
+            float part[NV];
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                float f[8];
+                widen8<T>(cur[k], f);
+                part[k] = squares8(f);// vectors behind the row's end were read as zeros
+            }
+            const float k_row = inv_rms(row_sum_any<NV>(part, red + phase * NV * MAX_WAVES, waves), d, eps);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) asm volatile("" : "+v"(cur[k]));// what follows widens the raw words anew
+
+            const __amdgpu_buffer_rsrc_t yr = row_of(y, row, stride_y);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const uint32_t v = k * bs + threadIdx.x;
+                if constexpr (WHOME == kWGlobal) {
+                    if (k != 0 && k % WB == 0) {
+                        __builtin_amdgcn_sched_barrier(0);// the batch before is used up: its registers take the next one
+                        fetch_weights(k);
+                    }
+                }
+                float f[8], g[8];
+                widen8<T>(cur[k], f);
+                if constexpr (WHOME == kWLds) {
+                    const uint32_t lv = v < nvec ? v : 0;
+                    const f32x4 a = w_lo[lv], b = w_hi[lv];
+                    g[0] = a.x, g[1] = a.y, g[2] = a.z, g[3] = a.w;
+                    g[4] = b.x, g[5] = b.y, g[6] = b.z, g[7] = b.w;
+                } else {
+                    W::spread(wr[k % WB], g);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
+                __builtin_amdgcn_raw_buffer_store_b128(narrow8<T>(f), yr, static_cast<int>(lane16 + k * bs * 16), 0, kOut);
+                if constexpr (NV >= 8) __builtin_amdgcn_sched_barrier(0);// one vector's arithmetic at a time: 128 registers per lane in all
+            }
+        }
+    };
+    if constexpr (WHOME == kWLds) {
+        serve(WF32{});
+    } else {
+        if (w_kind == kWKindF32) serve(WF32{});
+        else if (w_kind == kWKindF16) serve(W16<F16Ref>{});
+        else serve(W16<BF16Rne>{});
     }
 }
 
@@ -724,6 +899,36 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
 #undef RMS_ONCE
 #undef RMS_ONCE_GO
 
+    // Rows of more than 32 768 elements, and the fused form from 10 240: one workgroup per compute unit with as many
+    // lanes as the row has vectors for (see rms_norm_wide).
+    if (nvec > 4096 || (ADD && nvec >= 1280)) {
+        const unsigned per_lane = static_cast<unsigned>(ceil_div(nvec, 1024));               // 2 .. 8
+        const unsigned lanes = static_cast<unsigned>(ceil_div(ceil_div(nvec, per_lane), kWave)) * kWave;
+        const bool in_lds = d * sizeof(float) + 1024 <= static_cast<uint64_t>(desc.lds_per_block) && n > static_cast<uint64_t>(desc.cu_count);
+        const unsigned g = static_cast<unsigned>(n < static_cast<uint64_t>(desc.cu_count) ? n : desc.cu_count);
+#define RMS_WIDE_GO(NV, HOME, TH)                                                                                              \
+    rms_norm_wide<T, NV, HOME, TH, ADD><<<g, lanes, HOME == kWLds ? d * sizeof(float) : 0, stream>>>(                             \
+        py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res)
+#define RMS_WIDE(NV)                                        \
+    do {                                                    \
+        if (in_lds && through) RMS_WIDE_GO(NV, kWLds, true); \
+        else if (in_lds) RMS_WIDE_GO(NV, kWLds, false);      \
+        else if (through) RMS_WIDE_GO(NV, kWGlobal, true);   \
+        else RMS_WIDE_GO(NV, kWGlobal, false);               \
+    } while (0)
+        switch (per_lane) {
+            case 2: RMS_WIDE(2); break;
+            case 3: RMS_WIDE(3); break;
+            case 4: RMS_WIDE(4); break;
+            case 5: RMS_WIDE(5); break;
+            case 6: RMS_WIDE(6); break;
+            case 7: RMS_WIDE(7); break;
+            default: RMS_WIDE(8); break;
+        }
+#undef RMS_WIDE
+#undef RMS_WIDE_GO
+        return;
+    }
     // A workgroup that serves several rows fetches the weights once: into LDS
     // as fp32 when the row leaves room for at least two workgroups per compute
     // unit, else it re-reads them from memory like a one-row workgroup does.
@@ -840,8 +1045,7 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     }
     if (nvec <= 1024) RMS_LAUNCH(256, 4);
     else if (nvec <= 2048) RMS_LAUNCH(512, 4);
-    else if (nvec <= 4096) RMS_LAUNCH(1024, 4);
-    else RMS_LAUNCH(1024, 8);
+    else RMS_LAUNCH(1024, 4);
 #undef RMS_LAUNCH
 #undef RMS_GO
 }

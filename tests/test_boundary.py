@@ -18,7 +18,7 @@ INCLUDE = os.path.join(ROOT, "include")
 
 # reference include/infini_operators.h:1-19 and include/operators.h:4-7, minus the CNN-family operators
 REFERENCE_PATHS = [
-    "infini_operators.h", "operators.h", "device.h", "status.h", "data_type.h", "tensor.h", "handle.h",
+    "infini_operators.h", "operators.h", "export.h", "device.h", "status.h", "data_type.h", "tensor.h", "handle.h",
     "handle/handle_export.h", "tensor/tensor_descriptor.h",
     "ops/add/add.h", "ops/attention/attention.h", "ops/causal_softmax/causal_softmax.h", "ops/matmul/matmul.h",
     "ops/mlp/mlp.h", "ops/random_sample/random_sample.h", "ops/rearrange/rearrange.h", "ops/rms_norm/rms_norm.h",
@@ -49,6 +49,28 @@ def test_reference_header_path_stands_alone(path, tmp_path):
         res = subprocess.run([compiler, std, "-x", "c" if compiler == "gcc" else "c++", "-fsyntax-only", "-I", INCLUDE, str(tu)],
                              capture_output=True, text=True)
         assert res.returncode == 0, (path, compiler, res.stderr)
+
+
+@needs_gcc
+def test_export_header_gives_the_reference_macros(tmp_path):
+    """reference include/export.h:4-16: every operator header of the reference starts from `__export` and `__C`."""
+    tu = tmp_path / "macros.c"
+    tu.write_text('#include "ops/swiglu/swiglu.h"\n__C __export int mine(void);\nint mine(void) { return 0; }\n')
+    for compiler, lang in (("gcc", "c"), ("g++", "c++")):
+        res = subprocess.run([compiler, "-x", lang, "-Wall", "-Werror", "-fsyntax-only", "-I", INCLUDE, str(tu)], capture_output=True, text=True)
+        assert res.returncode == 0, (compiler, res.stderr)
+
+
+@needs_gcc
+def test_c_client_links_against_the_library(tmp_path):
+    """The program form of the C client (what tests/test_gpu_c_client.py runs on the GPU) links with the plain C compiler."""
+    from operators_amd import build as lib_build
+
+    assert os.path.isfile(library_path())
+    out = lib_build.build_c_client(verbose=False)
+    assert os.access(out, os.X_OK)
+    needed = subprocess.run(["readelf", "-d", out], capture_output=True, text=True, check=True).stdout
+    assert "libinfiniop.so" in needed and "libamdhip64.so" in needed
 
 
 def test_dynamic_symbol_table_is_exactly_the_header():
