@@ -14,10 +14,15 @@ five launches through the public C API on one stream.  Inputs are synthetic
 (seeded N(0,1) / U(0.5,1.5)), resident in HBM before the timed region, and the
 steps rotate over several independent buffer sets so that nothing is served
 from the 256 MB Infinity Cache.  The line printed at the end is one JSON
-object: `value` is algorithmic bytes moved per second over the whole chain;
-`roofline` describes the dominant kernel (SwiGLU) timed on its own with events
-on the launch stream; `cpu_baseline` is the CPU oracle timed on this host on a
-bounded sample of the same workload; `ops` lists every operator/configuration
+object: `value` is algorithmic bytes moved per second over the whole chain,
+W warm-up steps then K timed steps as asked for (`config.value_settled` is the
+same K steps timed again after untimed runs until the rate stands still,
+`config.value_qk_one_call` the chain when q and k are rotated by one RoPE call
+on the 72-head view); `roofline` describes the dominant kernel (SwiGLU) timed
+on its own, the same way, with events on the launch stream; `cpu_baseline` is
+the CPU oracle timed on this host on a bounded sample of the same workload;
+`config.frac_<row>` / `config.us_<row>` repeat the headline figure of the
+table's rows as flat scalars; `ops` lists every operator/configuration
 with its own time, bandwidth and fraction of the 8 TB/s peak: per row one cold
 first call (buffers never touched before; includes one-time code loading where
 the kernel has not run yet in the process), then at least 20 warm-up calls and
@@ -49,14 +54,14 @@ DOMINANT_KERNEL = "swiglu_rows<amd::BF16Rne"
 
 def measured_traffic(path=TRAFFIC_PROFILE, kernel=DOMINANT_KERNEL):
     """HBM bytes per launch of `kernel` from its row of the counter summary
-    (columns: kernel (grid), FETCH KiB, WRITE KiB, HBM bytes/launch,
+    (columns: bench row, kernel (grid), FETCH KiB, WRITE KiB, HBM bytes/launch,
     algorithmic, ratio).  No file or no row is an error: a roofline line whose
     traffic figure comes from nowhere would be worse than none."""
     if not os.path.isfile(path):
         raise FileNotFoundError(f"{path}: the hardware-counter summary the roofline's traffic figure is read from is missing")
     with open(path) as f:
         for line in f:
-            if line.startswith(kernel):
+            if kernel in line and line.rstrip()[-1:].isdigit():
                 cols = line.split()
                 return int(cols[-3])
     raise LookupError(f"{path} has no row for {kernel}")
@@ -458,7 +463,10 @@ def ops_table(ctx, args, gen):
         "N1c causal_softmax f16 [2048,512,512] (short rows: two to a wavefront)": lambda: [make_causal_softmax(ctx, 2048, 512, 512, f16, gen, "causal_softmax") for _ in range(2)],
         "N1d causal_softmax f16 [32,4095,4095] (ragged rows: every row starts at another 2-byte offset in its 128-byte line)": lambda: [make_causal_softmax(ctx, 32, 4095, 4095, f16, gen, "causal_softmax") for _ in range(2)],
         "N1e causal_softmax f16 [64,512,20480] (a chunk of 512 queries against 20480 keys: 512 lanes x 8 vectors)": lambda: [make_causal_softmax(ctx, 64, 512, 20480, f16, gen, "causal_softmax") for _ in range(2)],
-        "N1f causal_softmax f16 [64,512,65536] (rows beyond a workgroup's registers: two passes over the row)": lambda: [make_causal_softmax(ctx, 64, 512, 65536, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1f causal_softmax f16 [64,512,65536] (rows of 128 KiB held in registers as raw words, read once; the row stride is a power of two)": lambda: [make_causal_softmax(ctx, 64, 512, 65536, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1g causal_softmax f16 [64,512,40000] (the same form, 12 vectors per lane, a row stride that is no power of two)": lambda: [make_causal_softmax(ctx, 64, 512, 40000, f16, gen, "causal_softmax") for _ in range(2)],
+        "Q2 rms_norm bf16 [4096,32768] w f32 (one 1024-lane workgroup per compute unit, 128 KiB of weights in LDS)": lambda: [make_rms_norm(ctx, 4096, 32768, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * 4096 * 32768, nset))],
+        "F2 add_rms_norm bf16 [8192,16384] w f32 (fused Add + RMSNorm, wide rows)": lambda: [make_add_rms_norm(ctx, 8192, 16384, bf16, torch.float32, gen, "add_rms_norm") for _ in range(sets_needed(6 * 8192 * 16384, nset))],
     }
     if args.only and "calibration" in args.only:
         # Not an operator of the library: a plain device-to-device copy of known
@@ -688,10 +696,16 @@ def main():
     pos = torch.arange(T, device="cuda", dtype=torch.int64).view(torch.uint64)
     sets = [chain_set(ctx, T, gen, (sin_t, cos_t, pos)) for _ in range(args.sets)]
     chain_bytes = sum(l.nbytes for l in sets[0])
-    # Untimed steps first, until the rate has settled (the GPU has idled while the inputs were built, and the first
-    # tens of milliseconds of load run 1-3 % slower than what follows; see op_entry): at least 0.2 s of them, then until
-    # two runs in a row agree within 0.3 %, 2 s at most.  Then the W warm-up steps and the K timed ones, as asked.
+    # `value` is the protocol as asked: W untimed warm-up steps, then exactly K timed steps.  The GPU has idled while
+    # the inputs were built, and its first tens of milliseconds of load run 1-3 % slower than what follows (see
+    # op_entry), so the same K steps are timed once more after untimed settling and reported beside it, under names
+    # of their own (config.value_settled ...): a steady rate, not comparable with a figure taken the plain way.
+    wall, ev = time_rotating(sets, args.steps, args.warmup)
+    ms_per_step = wall / args.steps * 1e3
+    value = chain_bytes * args.steps / wall / 1e9
+
     def settle(what):
+        """Untimed runs: at least 0.2 s of them, then until two in a row agree within 0.3 % (2 s at most)."""
         spent, prev, runs = 0.0, None, 0
         while spent < 2.0:
             _, e = time_rotating(what, max(args.steps, 20), 0)
@@ -700,16 +714,30 @@ def main():
                 break
             prev = e
         return round(spent * 1e3, 1)
+
     chain_settle_ms = settle(sets)
-    wall, ev = time_rotating(sets, args.steps, args.warmup)
-    ms_per_step = wall / args.steps * 1e3
-    value = chain_bytes * args.steps / wall / 1e9
+    wall_s, ev_s = time_rotating(sets, args.steps, 0)
+    value_settled = chain_bytes * args.steps / wall_s / 1e9
+
+    # The same chain when the caller rotates q and k with ONE call: both are heads of the fused qkv buffer, so
+    # heads 0..71 of it are one strided view (four launches per step instead of five; the same bytes but for the
+    # position ids and table rows, which are then read once instead of twice).
+    qk_sets = []
+    for st in sets:
+        qkv = st[1].keep[1]
+        qk_sets.append([st[0], make_rope(ctx, qkv, 0, 72, pos, sin_t, cos_t, "rope_qk"), st[3], st[4]])
+    qk_bytes = sum(l.nbytes for l in qk_sets[0])
+    wall_qk, _ = time_rotating(qk_sets, args.steps, args.warmup)
+    del qk_sets
 
     # ---- dominant kernel on its own: SwiGLU of the chain -------------------------
     swiglu_sets = [[s[3]] for s in sets]
-    settle(swiglu_sets)
+    torch.cuda.synchronize()
+    time.sleep(0.5)  # idle, as before the chain's own run: the same protocol for the same kind of figure
     _, ev_sw = time_rotating(swiglu_sets, args.steps, args.warmup)
     sw_time = ev_sw / args.steps
+    settle(swiglu_sets)
+    _, ev_sw_s = time_rotating(swiglu_sets, args.steps, 0)
     sw_bytes = sets[0][3].nbytes
     roofline = {
         "bound": "hbm", "achieved": round(sw_bytes / sw_time / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -717,6 +745,7 @@ def main():
         "traffic": traffic,
         "kernel": f"swiglu_rows<bf16> [{T},28672] from fused [{T},57344]",
         "bytes_per_launch": sw_bytes, "us_per_launch": round(sw_time * 1e6, 2),
+        "frac_settled": round(sw_bytes / (ev_sw_s / args.steps) / 1e9 / HBM_PEAK_GBPS, 4), "us_per_launch_settled": round(ev_sw_s / args.steps * 1e6, 2),
     }
     per_op_chain = {l.name: l.nbytes for l in sets[0]}
     del sets, swiglu_sets
@@ -726,18 +755,55 @@ def main():
         "metric": "achieved_hbm_bandwidth", "value": round(value, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"C5 Llama-70B-shaped bf16 prefill chain, {T} tokens: rms_norm[{T},8192] + rope q[{T},64,128], k[{T},8,128] in qkv[{T},80,128] + swiglu[{T},28672] (fused gate/up) + add[{T},8192]",
+        "config": {"workload": f"C5 bf16 prefill chain, {T} tokens: rms_norm + rope q, k + swiglu (fused gate/up) + add",
+                   "shapes": f"rms_norm[{T},8192] w f32; rope q[{T},64,128], k[{T},8,128] in qkv[{T},80,128]; swiglu[{T},28672] of [{T},57344]; add[{T},8192]",
                    "launches_per_step": 5, "buffer_sets": args.sets, "bytes_per_step": chain_bytes, "bytes_by_op": per_op_chain,
-                   "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4), "event_ms_per_step": round(ev / args.steps * 1e3, 4), "untimed_settling_ms": chain_settle_ms},
+                   "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4), "event_ms_per_step": round(ev / args.steps * 1e3, 4),
+                   "value_settled": round(value_settled, 1), "ms_per_step_settled": round(wall_s / args.steps * 1e3, 4),
+                   "untimed_settling_ms": chain_settle_ms,
+                   "ms_per_step_qk_one_call": round(wall_qk / args.steps * 1e3, 4), "value_qk_one_call": round(qk_bytes * args.steps / wall_qk / 1e9, 1),
+                   "bytes_per_step_qk_one_call": qk_bytes},
         "roofline": roofline,
     }
     if not args.no_ops_table:
         out["ops"] = ops_table(ctx, args, gen)
+        out["config"].update(flat_fractions(out["ops"]))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(T)
         if not args.no_ops_table:
             attach_cpu(out["ops"], cpu_per_op(T))
     print(json.dumps(out))
+
+
+# Rows of the per-operator table whose figures also go, as flat scalars, into `config`
+# (what a reader of the one JSON line keeps when nested lists are dropped): key -> label prefix.
+FLAT_ROWS = {
+    "c1": "C1 rms_norm", "c2": "C2 swiglu f16 [4096,11008]", "c2_fused": "C2 swiglu f16 [4096,11008] fused", "c3": "C3 rope",
+    "c4": "C4 add f16 [8192,4096]", "c4_bcast": "C4 add f16 [8192,4096] + b", "c5_rms_norm": "C5 rms_norm", "c5_rope_q": "C5 rope_q",
+    "c5_rope_k": "C5 rope_k", "c5b_rope_qk": "C5b rope_qk", "c5_swiglu": "C5 swiglu", "c5_add": "C5 add",
+    "f1_add_rms_norm": "F1 add_rms_norm", "f2_add_rms_norm": "F2 add_rms_norm", "q1_rms_norm": "Q1 rms_norm", "q2_rms_norm": "Q2 rms_norm",
+    "n1_causal_softmax": "N1 causal_softmax", "n1c": "N1c", "n1d": "N1d", "n1e": "N1e", "n1f": "N1f", "n1g": "N1g",
+    "n2_rearrange": "N2 rearrange", "n2b_rearrange": "N2b rearrange",
+}
+
+
+def flat_fractions(rows):
+    """frac_<key> (fraction of the 8 TB/s peak) and us_<key> (microseconds per call) for the rows above; the
+    longest matching label prefix decides, as in attach_cpu.  C1 moves 135 KB: its fraction says nothing, its
+    time is the figure (frac_c1_us, as well as us_c1)."""
+    out = {}
+    for key, prefix in FLAT_ROWS.items():
+        for r in rows:
+            owners = [k for k, p in FLAT_ROWS.items() if r["config"].startswith(p)]
+            if owners and max(owners, key=lambda k: len(FLAT_ROWS[k])) == key:
+                out[f"us_{key}"] = r["us_per_call"]
+                if key == "c1":
+                    out["frac_c1_us"] = r["us_per_call"]
+                else:
+                    out[f"frac_{key}"] = r["frac_of_peak"]
+                if "copy_same_bytes_us" in r and key in ("c3", "c5_rope_k"):
+                    out[f"copy_same_bytes_us_{key}"] = r["copy_same_bytes_us"]
+    return out
 
 
 if __name__ == "__main__":

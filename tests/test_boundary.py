@@ -102,9 +102,12 @@ def test_bench_reads_its_traffic_figure_from_the_committed_profile(tmp_path):
     import bench
 
     text = open(bench.TRAFFIC_PROFILE).read()
-    row = [l for l in text.splitlines() if l.startswith(bench.DOMINANT_KERNEL)]
+    row = [l for l in text.splitlines() if bench.DOMINANT_KERNEL in l and l.startswith("C5 swiglu")]
     assert len(row) == 1
     assert bench.measured_traffic() == int(row[0].split()[-3])
+    # every row of the table carries the algorithmic bytes of its own bench row: no ratio is 0, none is far from 1
+    ratios = [float(l.split()[-1]) for l in text.splitlines() if re.search(r"\(\d+\)\s+[\d.]+\s+[\d.]+\s+\d+\s+\d+\s+[\d.]+$", l)]
+    assert len(ratios) >= 15 and all(0.99 < r < 1.06 for r in ratios), ratios
     assert 0.99 < bench.measured_traffic() / 1409286144 < 1.01  # the counters see the algorithmic bytes, no more
     with pytest.raises(FileNotFoundError):
         bench.measured_traffic(str(tmp_path / "absent.txt"))
