@@ -350,6 +350,12 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
         // here, and so is the row itself: a wavefront takes RPW consecutive rows of the whole tensor, whichever matrices
         // they lie in (the host passes the divisor of seq and the number of rows in place of the groups' figures), the
         // lanes behind the last row repeat it without storing.
+        // What this form costs against rows in whole lines, from the counters ([4096, 250, 250] against [4096, 256, 256],
+        // fp16, per launch): 1.27 times the bytes fetched (415 against 328 MB: a kept part that neither starts nor ends on
+        // a line boundary brings in two partial lines per row instead of one), 1.14 times the vector instructions, 1.29
+        // times the busy cycles.  (One end element per lane instead of two, end loads issued unconditionally beside the
+        // vector loads, 32-bit row offsets for equally spaced rows, the end stores left out altogether: each within
+        // 2 % of this, [8192, 120, 120] 13 % slower.)
         const uint32_t row_off = RAGGED ? 0u : rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
         struct Mine {
             uint16_t *row, *body;// the row's first element and its first whole vector

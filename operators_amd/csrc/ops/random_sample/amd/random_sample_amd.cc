@@ -42,7 +42,11 @@ infiniopStatus_t amdCreateRandomSampleDescriptor(AmdHandle_t handle, RandomSampl
         vecs = static_cast<uint32_t>(amd::ceil_div(voc, per_vec * kRandomSampleMaxGroups));
         groups = static_cast<uint32_t>(amd::ceil_div(voc, per_vec * vecs));
     }
-    auto *desc = new (std::nothrow) RandomSampleAmdDescriptor{DevAmdGpu, handle->device_id, elem, voc, groups, vecs};
+    void *scratch = nullptr;
+    if (amdRandomSampleScratch(handle->device_id, &scratch) != STATUS_SUCCESS) {
+        scratch = nullptr;// infiniopRandomSampleNoAlloc will say so; every other entry point works without it
+    }
+    auto *desc = new (std::nothrow) RandomSampleAmdDescriptor{DevAmdGpu, handle->device_id, elem, voc, groups, vecs, scratch};
     if (desc == nullptr) {
         return STATUS_MEMORY_NOT_ALLOCATED;
     }

@@ -40,6 +40,7 @@ struct RandomSampleAmdDescriptor {
     uint32_t voc;   // number of logits
     uint32_t groups;// workgroups of the first launch of the two-launch form; 0: never used
     uint32_t vecs;  // 8-element vectors per lane in them
+    void *scratch;  // this GPU's copy of the library's own lists (see amdRandomSampleScratch); null if it could not be found
 };
 typedef RandomSampleAmdDescriptor *RandomSampleAmdDescriptor_t;
 
@@ -54,6 +55,10 @@ infiniopStatus_t amdGetRandomSampleWorkspaceSize(RandomSampleAmdDescriptor_t des
 infiniopStatus_t amdRandomSample(RandomSampleAmdDescriptor_t desc, void *workspace, uint64_t workspace_size,
                                  void *result, void const *probs, float random_val, float topp, int topk,
                                  float temperature, void *stream);
+// The address, on GPU `device_id`, of the array the library keeps for calls that bring no workspace.  Asked of the
+// runtime once per GPU (with that GPU made current) and kept; descriptors take it at creation, so that the call
+// itself neither queries nor locks anything.
+infiniopStatus_t amdRandomSampleScratch(int device_id, void **address);
 infiniopStatus_t amdRandomSampleNoAlloc(RandomSampleAmdDescriptor_t desc, void *result, void const *probs, float random_val,
                                         float topp, int topk, float temperature, void *stream);
 infiniopStatus_t amdDestroyRandomSampleDescriptor(RandomSampleAmdDescriptor_t desc);

@@ -1345,7 +1345,8 @@ void launch_random_sample(const RandomSampleCall &c, int form, hipStream_t s) {
 // form's lists in a fixed array in device memory, one copy per GPU, held until
 // the process ends.  Host code never uses the array's name as an address (on
 // the host it is only a handle for the symbol): the address on a GPU is asked
-// for once, with that GPU current, and kept.
+// for once, with that GPU current, and kept; a descriptor takes it when it is
+// made, so the call path holds no lock and asks the runtime nothing.
 constexpr uint64_t kScratchListBytes = kRandomSampleMaxGroups * sizeof(RandomSamplePart) +
                                        static_cast<uint64_t>(kRandomSampleMaxGroups) * kRandomSamplePartCap * sizeof(uint64_t);
 constexpr uint64_t kScratchCountBytes = kRandomSampleMaxGroups * sizeof(RandomSamplePart) + static_cast<uint64_t>(kRandomSampleKeys) * sizeof(uint32_t);
@@ -1356,13 +1357,16 @@ constexpr int kMaxGpus = 64;
 std::mutex scratch_lock;
 void *scratch_on_gpu[kMaxGpus];// null until asked for
 
-// The address of this GPU's copy; `device_id` is the current device.
-infiniopStatus_t scratch_address(int device_id, void **address) {
+}// namespace
+
+// The address of a GPU's copy: asked for once per GPU, with that GPU current, at the creation of a descriptor.
+infiniopStatus_t amdRandomSampleScratch(int device_id, void **address) {
     if (device_id < 0 || device_id >= kMaxGpus) {
         return STATUS_BAD_DEVICE;
     }
     std::lock_guard<std::mutex> guard(scratch_lock);
     if (scratch_on_gpu[device_id] == nullptr) {
+        AMD_CHECK_HIP(hipSetDevice(device_id), STATUS_BAD_DEVICE);
         void *ptr = nullptr;
         AMD_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), STATUS_EXECUTION_FAILED);
         if (ptr == nullptr) {
@@ -1373,8 +1377,6 @@ infiniopStatus_t scratch_address(int device_id, void **address) {
     *address = scratch_on_gpu[device_id];
     return STATUS_SUCCESS;
 }
-
-}// namespace
 
 // RandomSample without a caller-provided workspace and without any allocation:
 // what the first launches leave for the drawing workgroup lives in this
@@ -1399,13 +1401,10 @@ infiniopStatus_t amdRandomSampleNoAlloc(RandomSampleAmdDescriptor_t desc, void *
                      desc->voc, static_cast<unsigned long long>(amdRandomSampleWorkspaceBytes(*desc)), static_cast<unsigned long long>(kScratchBytes));
         return STATUS_BAD_PARAM;
     }
-    AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
-    void *lists = nullptr;
-    const infiniopStatus_t st = scratch_address(desc->device_id, &lists);
-    if (st != STATUS_SUCCESS) {
-        return st;
+    if (desc->scratch == nullptr) {// the runtime did not give the array's address when the descriptor was made
+        return STATUS_EXECUTION_FAILED;
     }
-    return amdRandomSample(desc, lists, kScratchBytes, result, probs, random_val, topp, topk, temperature, stream);
+    return amdRandomSample(desc, desc->scratch, kScratchBytes, result, probs, random_val, topp, topk, temperature, stream);
 }
 
 // Stage 4 of RandomSample.  With topp > 0 and topk > 1 it samples, otherwise

@@ -18,12 +18,12 @@ pytestmark = pytest.mark.gpu
 SENTINEL = -777
 
 
-def draw(ctx, codes, rv, topp, topk, temp, entry):
+def draw(ctx, codes, rv, topp, topk, temp, entry, dtype="f16"):
     import torch
 
     from operators_amd.ops import RandomSamplePlan
 
-    probs = to_torch(np.ascontiguousarray(codes, np.uint16), "f16")
+    probs = to_torch(np.ascontiguousarray(codes, np.uint16), dtype)
     result = torch.full((1,), SENTINEL, dtype=torch.int64, device="cuda")
     view = result.view(torch.uint64)
     with RandomSamplePlan(ctx, view, probs, use_workspace=True) as plan:
@@ -54,6 +54,29 @@ def test_two_calls_in_a_row_second_one_smaller(ctx):
             if min(topk, voc) * voc <= 2 * 10 ** 8:  # the oracle's selection loop is O(topk * voc): seconds beyond this
                 ref = oracle.random_sample(x, rv, topp, topk, temp)
                 assert got == ref or x[got] == x[ref], (voc, rv, topp, topk, temp, got, ref)
+
+
+def test_bf16_logits_and_a_random_value_of_one(ctx):
+    """The extension type, and the draw that falls off the end of the cumulative distribution (random_val = 1: the
+    reference's loop then finds no candidate and leaves the result as it was; with one logit, sampling asked for,
+    nothing is launched at all)."""
+    rng = np.random.default_rng(79)
+    for voc in (40000, 6000, 700):
+        x = oracle.encode((rng.standard_normal(voc) * 3).astype(np.float32), "bf16")
+        for rv, topp, topk, temp in ((0.37, 0.9, 50, 0.8), (0.66, 1.0, 300, 1.0), (1.0, 0.9, 50, 0.8), (0.5, 0.0, 1, 1.0)):
+            want = draw(ctx, x, rv, topp, topk, temp, "workspace", "bf16")
+            got = draw(ctx, x, rv, topp, topk, temp, "no_alloc", "bf16")
+            assert got == want, (voc, rv, topp, topk, temp, got, want)
+    x16 = logits(rng, 33000)
+    for rv in (1.0, 1.5):
+        want = draw(ctx, x16, rv, 0.9, 50, 0.8, "workspace")
+        assert draw(ctx, x16, rv, 0.9, 50, 0.8, "no_alloc") == want
+        ref = oracle.random_sample(x16, rv, 0.9, 50, 0.8)  # None: the reference leaves the result unwritten
+        assert (want == SENTINEL) if ref is None else (want == ref or x16[want] == x16[ref]), (rv, want, ref)
+    one = logits(rng, 1)
+    for entry in ("workspace", "no_alloc"):
+        assert draw(ctx, one, 1.0, 0.9, 2, 1.0, entry) == SENTINEL  # nothing wins, nothing is written
+        assert draw(ctx, one, 0.3, 0.9, 2, 1.0, entry) == 0
 
 
 def test_repeated_calls_share_the_array_in_stream_order(ctx):
