@@ -34,3 +34,42 @@ def run(test_cases, test):
         destroy_handle(lib, handle)
     print("\033[92mTest passed!\033[0m")
     return 0
+
+
+class described:
+    """`with described(lib, t0, t1, ...) as cts:` - the tensors described to the library for the length of the block."""
+
+    def __init__(self, lib, *tensors):
+        self.lib, self.tensors = lib, tensors
+
+    def __enter__(self):
+        from operators_amd import to_tensor
+
+        self.cts = [to_tensor(t, self.lib) for t in self.tensors]
+        return self.cts
+
+    def __exit__(self, *exc):
+        from operators_amd import destroy_tensor
+
+        for ct in self.cts:
+            destroy_tensor(self.lib, ct)
+        return False
+
+
+def workspace_for(lib, query, desc, device):
+    """(pointer or None, size) of the workspace `query(desc, &size)` asks for, and the tensor that owns it."""
+    import ctypes
+
+    from operators_amd import check_error, create_workspace
+
+    size = ctypes.c_uint64(0)
+    check_error(query(desc, ctypes.byref(size)))
+    owner = create_workspace(size.value, device)
+    return (owner.data_ptr() if owner is not None else None), size.value, owner
+
+
+def laid_out(t, strides):
+    """t's values in a tensor with the given element strides (None: as it is)."""
+    from operators_amd import rearrange_tensor
+
+    return t if strides is None else rearrange_tensor(t, strides)

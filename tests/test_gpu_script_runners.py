@@ -8,7 +8,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("op", ["add", "rms_norm", "rotary_embedding", "swiglu"])
+@pytest.mark.parametrize("op", ["add", "rms_norm", "rotary_embedding", "swiglu", "causal_softmax", "rearrange", "random_sample", "matmul", "mlp"])
 def test_reference_style_cases(ctx, op, capsys):
     import torch
 
