@@ -63,8 +63,11 @@ CASES = [
     # short rows in whole lines whose matrices do not fill wavefronts (decoding: one row per matrix), any consecutive rows per wavefront
     ((37, 1, 320), None), ((9, 3, 128), None), ((50, 7, 512), None), ((5, 1, 64), (64 * 3, 64, 1)), ((33, 1, 300), None), ((3, 127, 128), None),
     ((2, 40, 4100), None), ((2, 33, 2104), None), ((2, 33, 2105), None), ((3, 50, 1080), None), ((2, 1000, 1000), None), ((1, 600, 4088), None),
-    # rows beyond what a workgroup holds in registers: two passes with 16-byte accesses (512 and 1024 lanes), padded rows
+    # rows of 32 769-131 072 elements held in registers as raw words (512 lanes x 12 / 16 / 20 vectors, 1024 lanes x 12 / 14 / 16),
+    # padded rows; beyond that, and ragged, two passes with 16-byte accesses
     ((2, 6, 65536), None), ((1, 4, 100000), None), ((2, 3, 40000), (3 * 40008, 40008, 1)), ((1, 7, 32776), None),
+    ((1, 5, 81920), None), ((2, 3, 70000), None), ((1, 4, 90000), None), ((1, 3, 131072), None), ((1, 3, 120000), None), ((1, 3, 131080), None),
+    ((1, 70, 32840), None), ((1, 40, 65544), (40 * 65600, 65600, 1)),
     # 16 385-32 768 elements: 512 lanes x 8 vectors, whole lines and ragged
     ((2, 5, 20480), None), ((1, 6, 32768), None), ((2, 4, 20001), None), ((1, 3, 32760), (3 * 32776, 32776, 1)),
     ((5, 512, 512), None), ((3, 40, 400), None), ((2, 300, 512), None), ((3, 64, 264), None), ((2, 16, 504), (16 * 520, 520, 1)), ((2, 33, 512), None),
@@ -186,6 +189,31 @@ def test_where_gpu_and_cpu_path_differ_the_gpu_is_the_exact_one(ctx, dt, shape):
     assert gpu_right >= 0.8 * n and gpu_right >= cpu_right
     assert (got == exact)[keep].mean() >= (want == exact)[keep].mean()
     assert (got == exact)[keep].mean() > 0.9995
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_long_row_forms_against_the_float64_quotient(ctx, dt):
+    """Rows of 32 769 elements and more form their exponentials with the hardware exp2 of one fused multiply-add
+    (relative error below 3e-6), the shorter ones with a corrected exponential: the same row is therefore not
+    promised the same bits through both.  What is promised, and recorded here: every output of either form is
+    within one unit in the last place of the float64 quotient narrowed by the type's rule, and the long-row form
+    hits it exactly about as often as the register form does on a row of 32 768."""
+    rng = np.random.default_rng(41)
+    rates = {}
+    for total in (32768, 40000, 65536, 100000, 131072, 200000):
+        shape = (1, 4, total)
+        y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 3, dt)
+        got, _, _ = run(ctx, y, shape, None, dt)
+        got = got.reshape(shape)
+        keep = np.broadcast_to(np.arange(total)[None, :] <= total - 4 + np.arange(4)[:, None], shape)
+        x = np.where(keep, oracle.decode(y, dt).astype(np.float64).reshape(shape), -np.inf)
+        e = np.exp(x - x.max(-1, keepdims=True))
+        exact = oracle.encode((e / e.sum(-1, keepdims=True)).astype(np.float32).ravel(), dt).reshape(shape)
+        frac, worst = check(got, exact, dt, f"[1,4,{total}] {dt} against float64", max_frac=1e-2)
+        rates[total] = 1.0 - frac
+        assert worst <= 1
+    print(f"causal softmax {dt}: share of outputs equal to the narrowed float64 quotient, by row length: " + ", ".join(f"{t}: {r:.5f}" for t, r in rates.items()))
+    assert min(rates.values()) > 0.999 and rates[32768] - min(rates.values()) < 5e-4
 
 
 def test_attention_scores_shape(ctx):

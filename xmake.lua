@@ -69,9 +69,11 @@ if has_config("amd-gpu") then
         on_install(function (target) end)
         set_languages("cxx17")
         add_includedirs("include")
-        add_files(CSRC .. "/devices/amd/*.cc", {rule = "hipcc"})
-        add_files(CSRC .. "/ops/*/amd/*.cc", {rule = "hipcc"})
-        add_files(CSRC .. "/ops/*/amd/*.hip", {rule = "hipcc"})
+        -- only the hipcc rule compiles this target's files: `rules = ` replaces the rules xmake would pick by
+        -- extension (for .cc its own C++ rule, which would compile every file a second time)
+        add_files(CSRC .. "/devices/amd/*.cc", {rules = "hipcc"})
+        add_files(CSRC .. "/ops/*/amd/*.cc", {rules = "hipcc"})
+        add_files(CSRC .. "/ops/*/amd/*.hip", {rules = "hipcc"})
     target_end()
 
 end
@@ -85,6 +87,7 @@ target("infiniop")
     set_toolset("ld", HIPCC)
     set_toolset("sh", HIPCC)
     add_shflags("--offload-arch=gfx950", {force = true})
+    add_syslinks("dl", "pthread")   -- the BLAS loader calls dlopen / dlsym; glibc before 2.34 keeps them in libdl
     add_includedirs(ROCM .. "/include")
     add_defines("__HIP_PLATFORM_AMD__")
     add_cxxflags("-fPIC", "-fvisibility=hidden")
