@@ -396,7 +396,10 @@ __global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y
 //   plain [4096, 32768]   94.3 /  93.7 (so the plain form stays with rms_norm_rows up to there)
 // (Two halves of a workgroup on rows of their own, each with a counting
 // barrier in LDS and both sharing the staged weights, measured slower: plain
-// [4096, 32768] 100.2 us, fused 191.6 us.)
+// [4096, 32768] 100.2 us, fused 191.6 us.  Each lane's weights held in its
+// registers for all of a workgroup's rows, no LDS, so that two or three
+// 512-lane workgroups fit a compute unit: plain [4096, 32768] 92.2-93.4 us
+// against 93.3, [8192, 16384] 90.6 against 89.9 - no different.)
 template<typename T, int NV, int WHOME, bool THROUGH, bool ADD, int WBATCH = 4>
 __global__ __launch_bounds__(1024) void rms_norm_wide(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                       uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
