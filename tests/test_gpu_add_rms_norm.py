@@ -58,7 +58,11 @@ def check_y(got, want, dt, what, max_frac=5e-3):
                                  # widths of common models on the looping kernels
                                  (600, 5120), (530, 7168), (300, 12288),
                                  # rows whose fp32 weights take more than 64 KiB of LDS, and the first size beyond what LDS holds
-                                 (300, 18432), (270, 32768), (265, 40704), (262, 40960)])
+                                 (300, 18432), (270, 32768), (265, 40704), (262, 40960),
+                                 # the wide-row kernel (from 10 240 elements): 2 to 8 vectors per lane, lane counts that are no power of
+                                 # two (11 000: 704 lanes), weights in LDS and from memory, fewer rows than compute units
+                                 (520, 10240), (300, 11000), (280, 14336), (290, 16384), (280, 20480), (270, 24576), (264, 36864), (300, 49152),
+                                 (258, 65536), (40, 12288)])
 def test_against_oracle_and_against_the_two_separate_calls(ctx, dt, wdt, n, d):
     a, b, w = inputs(n, d, dt, wdt, n * 11 + d)
     want_c, want_y = oracle.add_rms_norm(a, b, w, 1e-5, dt, wdt)

@@ -55,6 +55,8 @@ def test_golden_odd_sizes(ctx):
                                  (5600, 6144), (4700, 7168),
                                  # rows whose fp32 weights take more than 64 KiB of LDS (up to 160 KiB per workgroup), and the first size beyond
                                  (300, 18432), (290, 20480), (280, 24576), (270, 32768), (265, 40704), (262, 40960),
+                                 # the wide-row kernel, 5 to 8 vectors per lane: weights in LDS (33 000: 832 lanes), from memory in batches, few rows
+                                 (270, 33000), (264, 36864), (300, 49152), (260, 57344), (258, 65536), (40, 49152),
                                  # short rows, several to a wavefront (per-head norms): full and ragged last wavefronts, rows that
                                  # do not fill their lanes, an output large enough to be written through L2
                                  (5001, 128), (4096, 128), (1003, 64), (777, 256), (333, 72), (101, 16), (50, 200), (270000, 128)])
