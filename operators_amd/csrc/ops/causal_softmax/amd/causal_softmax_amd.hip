@@ -542,17 +542,17 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
     }
 }
 
-// Rows that the register kernels above do not take: longer than a workgroup
-// can hold (more than 32 768 elements), or RAGGED - rows that do not start on
-// 16-byte boundaries or whose length is no multiple of 8, which is what the
-// scores of an attention over an arbitrary number of keys look like.  Two
-// passes over the row with 16-byte accesses, UNROLL vectors per lane in flight
-// at a time: the maximum (and the minimum, for the choice of exponential)
-// together with the sum of the exponentials, then the quotients.  The first
-// pass brings the row in from memory; the second finds it in L2 or in the
-// Infinity Cache, so the exponentials are formed twice but memory is read
-// once.  (With the sum in a pass of its own, after the maximum: [64, 512,
-// 65536] fp16 2163 us against 1691 us, [64, 512, 40000] 1288 against 1001 us.)
+// Rows of more than 32 768 elements that the register kernels do not take:
+// longer than 131 072 elements, or RAGGED - rows that do not start on 16-byte
+// boundaries or whose length is no multiple of 8, which is what the scores of
+// an attention over an arbitrary number of keys look like.  Two passes over
+// the row with 16-byte accesses, UNROLL vectors per lane in flight at a time:
+// the maximum (and the minimum, for the choice of exponential) together with
+// the sum of the exponentials, then the quotients.  The first pass brings the
+// row in from memory; the second finds most of it in L2 or in the Infinity
+// Cache (the counters say 70 % at 65 536 elements: 1.15 times the algorithmic
+// traffic), so the exponentials are formed twice.  (With the sum in a pass of
+// its own, after the maximum: [64, 512, 65536] fp16 2163 us against 1691 us.)
 // Masked vectors are written as zeros without being read.  One workgroup per
 // row at a time.
 // RAGGED: the vectors are the 16-byte aligned ones from the 128-byte boundary
@@ -930,8 +930,9 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
 
     const bool even = (reinterpret_cast<uintptr_t>(data) & 1u) == 0;// elements lie on 2-byte boundaries
     const bool vec_ok = even && cover <= 4096 && d.seq < (1ull << 31) && (!ragged || d.total >= 16);
-    // Rows of more than 32 768 elements (see causal_softmax_long).  Measured on MI355X, fp16, against the element kernel:
-    //   [64, 512, 65536]  1691 us (63 %) against 7230 us     [64, 512, 40000]  1001 against 4194 us
+    // Rows of more than 32 768 elements: held in registers as raw words up to 131 072 when they lie on 16-byte
+    // boundaries (causal_softmax_held), two passes otherwise (causal_softmax_long; the element kernel took
+    // 7230 us for [64, 512, 65536] fp16, 4194 us for [64, 512, 40000]).
     const uint64_t vecs = cover;
     const bool long_ok = even && cover > 4096 && d.total + 64 < (1ull << 31) && rows < kFastDivLimit;
     if (long_ok) {

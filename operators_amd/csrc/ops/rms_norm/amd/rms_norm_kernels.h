@@ -833,7 +833,8 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     //   d = 4096:  45.5 us one pass, R = 1 (46.4 with R = 2)   46.6 us looping
     //   d = 8192:  45.6-50.3 us one pass            44.6 us looping
     //   d = 8192, fused Add: 86.5 us one pass with 1024 lanes, 88.1-89.7 with 256 or 512   89.0 us looping
-    //   d >= 16384: looping (a row's weights are 64 KiB and more: too many registers)
+    //   d >= 16384: looping (a row's weights are 64 KiB and more: too many registers); the fused form from 10240
+    //   and plain rows beyond 32768: rms_norm_wide, below
     // One pass re-reads the weight row through L2 once per R rows - at d = 8192
     // that is twice the bytes of the row itself - which is what it loses to
     // the looping form there; the fused form moves twice the data per weight.
@@ -932,11 +933,10 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
 #undef RMS_WIDE_GO
         return;
     }
-    // A workgroup that serves several rows fetches the weights once: into LDS
-    // as fp32 when the row leaves room for at least two workgroups per compute
-    // unit, else it re-reads them from memory like a one-row workgroup does.
+    // What is left: plain rows of 4097 to 32 768 elements and fused ones below 10 240.  A workgroup that serves
+    // several rows fetches the weights once, into LDS as fp32 (128 KiB at most here: it always fits the 160 KiB a
+    // gfx950 workgroup may use; above 80 KiB only one workgroup fits a compute unit).
     const uint64_t lds_bytes = d * sizeof(float);
-    const uint64_t lds_limit = static_cast<uint64_t>(desc.lds_per_block) - 1024;
     // How many workgroups per compute unit.  With the next row always in flight
     // a workgroup keeps two rows' worth of loads outstanding, and what measures
     // best is 20-32 KiB of them per compute unit, not more: bf16 rows with fp32
@@ -951,17 +951,9 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // d = 16384: 45.0-45.9 against 46.0-46.6 us).
     uint64_t per_cu = d * sizeof(uint16_t) > 12 * 1024 ? 1 : 2;
     if (!ADD && (d == 8192 || d == 16384)) per_cu = 2;
+    // (128 MiB of bf16 rows, weights in LDS against re-read through L2 per row:
+    //   d = 18432  48.0 / 58.8 us     d = 24576  48.0 / 55.1 us     d = 32768  49.5 / 54.3 us)
     int home = kWLds;
-    // LDS holds up to 160 KiB per workgroup on gfx950 (rows of up to 40 704 elements); above 80 KiB only one
-    // workgroup fits a compute unit.  128 MiB of bf16 rows, weights in LDS against re-read through L2 per row:
-    //   d = 18432  48.0 / 58.8 us     d = 24576  48.0 / 55.1 us     d = 32768  49.5 / 54.3 us
-    // The fused form has no registers for a second row at these widths, and one workgroup per unit working
-    // one row at a time is slower than two that re-read the weights (d = 18432: 108.2 / 102.9 us,
-    // d = 24576: 102.3 / 96.7 us), so it keeps its weights in LDS up to 64 KiB only.
-    if (lds_bytes > lds_limit || (ADD && lds_bytes > 64 * 1024)) {
-        home = kWGlobal;
-        per_cu = 2;
-    }
     uint64_t grid = static_cast<uint64_t>(desc.cu_count) * per_cu;
     if (n <= grid) {
         grid = n;
@@ -977,8 +969,7 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // is measurable.
     // Two register sets (the next row fetched ahead) fit the 128 registers a
     // lane of a 1024-lane workgroup may have up to 4 vectors per lane, 2 in
-    // the fused form; beyond that the second set would live in scratch
-    // memory, and those shapes work through one row at a time.
+    // the fused form.
 #define RMS_GO(BS, NV, HOME, LDS, EXACT, THROUGH)                                                                      \
     rms_norm_rows<T, BS, NV, HOME, EXACT, THROUGH, ADD, (BS * NV * (ADD ? 2 : 1) <= 4096)>                             \
         <<<static_cast<unsigned>(grid), BS, LDS, stream>>>(                                                            \
