@@ -21,6 +21,7 @@
 
 #include "../../../devices/amd/common_amd.h"
 #include "../../../devices/amd/kernel_amd.h"
+#include <algorithm>
 
 // Internal linkage: each including translation unit owns its copies, and none
 // of them appears in the library's dynamic symbol table.
@@ -367,9 +368,11 @@ __global__ __launch_bounds__(BS != 0 ? BS : 1024) void rms_norm_rows(uint16_t *y
 }
 
 // ---- wide rows ----------------------------------------------------------------
-// Rows of more than 32 768 elements, and the fused form from 10 240: one
-// workgroup per compute unit, as many lanes as the row has vectors for (up to
-// 1024), NV raw vectors per lane, one row at a time.  What differs from
+// Rows of more than 32 768 elements and the fused form from 10 240 (one
+// workgroup per compute unit, as many lanes as the row has vectors for, up to
+// 1024); the fused form between 4097 and 8191 and plain rows for which
+// rms_norm_rows has no exact launch shape (two workgroups per unit of up to
+// 512 lanes).  NV raw vectors per lane, one row at a time.  What differs from
 // rms_norm_rows:
 // - the lane count is the launch's, so that no lane is idle whatever the width;
 // - loads go through a buffer descriptor of one row (or of the weight row): a
@@ -903,13 +906,27 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
 #undef RMS_ONCE
 #undef RMS_ONCE_GO
 
-    // Rows of more than 32 768 elements, and the fused form from 10 240: one workgroup per compute unit with as many
-    // lanes as the row has vectors for (see rms_norm_wide).
-    if (nvec > 4096 || (ADD && nvec >= 1280)) {
-        const unsigned per_lane = static_cast<unsigned>(ceil_div(nvec, 1024));               // 2 .. 8
+    // rms_norm_wide.  Rows of more than 32 768 elements, and the fused form from 10 240: one workgroup per compute
+    // unit with as many lanes as the row has vectors for.  Plain rows from 6144 elements whose vector count is no
+    // multiple of 64, so that no launch shape below fits them exactly: two workgroups per unit of up to 512 lanes
+    // (128 MiB of bf16 rows, us, against the predicated ladder of rms_norm_rows:
+    //   d = 6720  45.9 / 57.5    7232  45.1 / 54.5    9280  45.2 / 49.9    10304  45.5 / 50.4    15424  45.4 / 47.4    18496  48.3 / 51.7
+    //   and rows that do not even start on 128-byte boundaries: d = 7000  56.7 / 74.4    9000  55.0 / 64.1    10000  54.6 / 62.2;
+    //   below 6144 elements the ladder is the faster one: d = 4544  48.7 against 52.8, 5184  47.2 against 51.7).
+    // The fused form between 4097 and 8191 elements: two workgroups per unit of 2 or 3 vectors per lane (128 MiB per
+    // operand, us, against rms_norm_rows: d = 4608  87.3 / 96.6    5120  88.2 / 98.7    6144  87.4 / 97.2    7168  89.1 / 91.1
+    // 7680  89.7 / 91.1; from 8704 to 10 239 rms_norm_rows is level or ahead: 9216  92.4 against 94.4).
+    const bool no_exact_shape = !ADD && nvec % kWave != 0 && nvec >= 768;
+    const bool fused_mid = ADD && nvec > 512 && nvec < 1024;
+    if (nvec > 4096 || (ADD && nvec >= 1280) || no_exact_shape || fused_mid) {
+        const bool one_per_unit = nvec > 4096 || (ADD && nvec >= 1280);
+        const unsigned per_lane = static_cast<unsigned>(one_per_unit ? ceil_div(nvec, 1024) : fused_mid ? (nvec <= 768 ? 2 : 3) : std::min<uint64_t>(4, ceil_div(nvec, 512)));// 2 .. 8
         const unsigned lanes = static_cast<unsigned>(ceil_div(ceil_div(nvec, per_lane), kWave)) * kWave;
-        const bool in_lds = d * sizeof(float) + 1024 <= static_cast<uint64_t>(desc.lds_per_block) && n > static_cast<uint64_t>(desc.cu_count);
-        const unsigned g = static_cast<unsigned>(n < static_cast<uint64_t>(desc.cu_count) ? n : desc.cu_count);
+        const uint64_t lds_need = d * sizeof(float) + 2048;
+        const unsigned per_cu = !one_per_unit && 2 * lds_need <= static_cast<uint64_t>(desc.lds_per_block) ? 2 : 1;
+        const uint64_t cap = static_cast<uint64_t>(desc.cu_count) * per_cu;
+        const bool in_lds = lds_need <= static_cast<uint64_t>(desc.lds_per_block) && n > cap;
+        const unsigned g = static_cast<unsigned>(n < cap ? n : cap);
 #define RMS_WIDE_GO(NV, HOME, TH)                                                                                              \
     rms_norm_wide<T, NV, HOME, TH, ADD><<<g, lanes, HOME == kWLds ? d * sizeof(float) : 0, stream>>>(                             \
         py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res)
