@@ -356,6 +356,11 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
         // times the busy cycles.  (One end element per lane instead of two, end loads issued unconditionally beside the
         // vector loads, 32-bit row offsets for equally spaced rows, the end stores left out altogether: each within
         // 2 % of this, [8192, 120, 120] 13 % slower.)
+        // Nor is it the arithmetic that these rows wait for: with the exponential cut to one multiply and the
+        // hardware exp2, and the quotient to one multiply - a third of the vector instructions gone, at the price of
+        // three times as many outputs one unit off the float64 quotient - [8192, 256, 256] took 276 against 274 us,
+        // [4096, 250, 250] 190 against 190, [2048, 333, 333] 157 against 157; only [16384, 64, 256] (160 against 170)
+        // and [65536, 64, 64] (168 against 178) moved.
         const uint32_t row_off = RAGGED ? 0u : rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
         struct Mine {
             uint16_t *row, *body;// the row's first element and its first whole vector
@@ -1059,6 +1064,8 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     // hand and one row's arithmetic overlaps the other's loads and stores.  1024 lanes x 4 vectors (one row per unit, its
     // phases strictly one after the other) measured, fp16: [64, 512, 20480] 644 -> 430 us (52 -> 77 %), [64, 512, 32768]
     // 945 -> 768 us, [2, 20480, 20480] 682 -> 454 us, [1, 32768, 32768] 723 -> 583 us.
+    // (causal_softmax_held with 5, 6 or 8 raw vectors per lane, three or four workgroups per unit, on these rows:
+    // [64, 512, 20480] 472 against 427 us, [64, 512, 24576] 578 against 527 us, [64, 512, 32768] 862 against 807 us.)
     // (A lane count taken from the launch, so that a row of 10240 elements gets 320 lanes x 4 vectors instead of
     // 512 x 4, measured worse, not better: [64, 512, 10240] fp16 364 against 237 us, [64, 512, 20480] 763
     // against 647 us - workgroups of 5, 10 or 12 wavefronts sit unevenly on a compute unit's four SIMDs.)
