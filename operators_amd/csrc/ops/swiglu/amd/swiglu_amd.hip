@@ -167,6 +167,17 @@ void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const v
 
     const bool vec_ok = d.di % 8 == 0 && d.stride_a % 8 == 0 && d.stride_b % 8 == 0 && d.stride_c % 8 == 0 &&
                         aligned16(c) && aligned16(a) && aligned16(b);
+    // Dense tensors are one run of rows * di elements whatever the width: vectors as far as they go, the up to 7
+    // elements behind them one by one ([4096, 11007] fp16: 42 us; 112 us element by element).
+    const bool one_run = d.rows == 1 || (d.stride_a == di && d.stride_b == di && d.stride_c == di);
+    if (!vec_ok && one_run && n >= 8 && aligned16(c) && aligned16(a) && aligned16(b)) {
+        const uint64_t whole = n / 8, want = ceil_div(whole, kWave), max_grid = max_grid_1d(kWave);
+        swiglu_vec<T, uint64_t, false><<<static_cast<unsigned>(want < max_grid ? want : max_grid), kWave, 0, stream>>>(
+            pc, pa, pb, whole, whole, 0, 0, 0, FastDiv{});
+        const uint64_t done = whole * 8;
+        if (done < n) swiglu_scalar<T><<<1, kBlock, 0, stream>>>(pc + done, pa + done, pb + done, 1, n - done, 0, 0, 0);
+        return;
+    }
     if (!vec_ok) {
         const uint64_t want = ceil_div(n, kBlock), cap = static_cast<uint64_t>(d.cu_count) * 64;
         swiglu_scalar<T><<<static_cast<unsigned>(want < cap ? want : cap), kBlock, 0, stream>>>(
@@ -179,8 +190,7 @@ void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const v
     const uint64_t want = ceil_div(nvec, kWave);
     const uint64_t max_grid = max_grid_1d(kWave);
     const unsigned grid = static_cast<unsigned>(want < max_grid ? want : max_grid);
-    // One row, or every row stride equal to the width: the tensors are dense.
-    const bool dense = d.rows == 1 || (d.stride_a == di && d.stride_b == di && d.stride_c == di);
+    const bool dense = one_run;// one row, or every row stride equal to the width
     const bool small = nvec < (1ull << 31);
     // Row-strided tensors (the halves of a fused gate/up buffer).  Rows of at least 1024 vectors: a 2-D grid of
     // single-wavefront workgroups, no lane divides anything.  Shorter rows: the same tiles over the flat (row,

@@ -55,7 +55,8 @@ def test_golden_saturation(ctx):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-@pytest.mark.parametrize("shape,fused", [((13, 4), False), ((16, 5632), False), ((33, 1000), True), ((64, 11008), True), ((5, 7), False)])
+@pytest.mark.parametrize("shape,fused", [((13, 4), False), ((16, 5632), False), ((33, 1000), True), ((64, 11008), True), ((5, 7), False),
+                                         ((1, 5), False), ((3, 1001), False), ((257, 4099), False), ((7, 1001), True)])
 def test_against_oracle(ctx, dt, shape, fused):
     import torch
 
