@@ -757,7 +757,11 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
 // from the one before it: 1453 us (74 %) against 1641 us (65 %); [64, 512,
 // 32768]: 764 against 815 us.  (Turning the order in which a workgroup's lanes
 // take the row's vectors, by 1 KiB per row, changes nothing: 1647 us - the
-// whole row is in flight at once either way.)
+// whole row is in flight at once either way.  Which rows are in flight
+// together does matter, but not in a way a rule could be made of: workgroups
+// taking row r * m mod rows instead of row r, for fourteen odd m from 3 to
+// 12 289, ran [64, 512, 65536] in 1566 (m = 513) to 1800 us (m = 1025)
+// against 1664, and [64, 512, 32768] in 796-814 against 799.)
 template<typename T, int BS, int NV, bool THROUGH>
 __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(4)))
 void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total, int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
