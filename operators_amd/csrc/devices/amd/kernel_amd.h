@@ -106,6 +106,17 @@ __device__ __forceinline__ void st16_stream(void *p, u32x4 v) {
 __device__ __forceinline__ u32x4 ld16(const void *p) {
     return *reinterpret_cast<const u32x4 *>(p);
 }
+// 16 bytes at any 2-byte boundary (gfx950 serves global accesses at any
+// alignment, at a fraction of the aligned rate): for the kernels that take
+// what the vector kernels refuse.
+typedef u32x4 __attribute__((aligned(2))) u32x4_any;
+typedef f32x4 __attribute__((aligned(4))) f32x4_any;
+__device__ __forceinline__ u32x4 ld16_any(const void *p) {
+    return *reinterpret_cast<const u32x4_any *>(p);
+}
+__device__ __forceinline__ void st16_any(void *p, u32x4 v) {
+    *reinterpret_cast<u32x4_any *>(p) = v;
+}
 __device__ __forceinline__ f32x4 ld16f(const float *p) {
     return *reinterpret_cast<const f32x4 *>(p);
 }

@@ -142,18 +142,28 @@ __global__ __launch_bounds__(LANES) void swiglu_rows(uint16_t *c, const uint16_t
     }
 }
 
-// Any width, any alignment: one element per lane per step.
+// Any width, any alignment.  A lane takes 8 consecutive elements of one row: a
+// whole group moves as 16 bytes at whatever 2-byte boundary it lies on (which
+// gfx950 serves at a fraction of the aligned rate), a row's last, partial
+// group element by element.  [4096, 11007] fp16 halves of a fused buffer:
+// 113 us with element accesses only.
 template<typename T>
 __global__ __launch_bounds__(kBlock) void swiglu_scalar(uint16_t *c, const uint16_t *a, const uint16_t *b,
                                                         uint64_t rows, uint64_t di,
                                                         int64_t stride_c, int64_t stride_a, int64_t stride_b) {
-    const uint64_t n = rows * di;
+    const uint64_t per_row = (di + 7) / 8, groups = rows * per_row;
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
-    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += step) {
-        const uint64_t row = i / di, col = i - row * di;
-        const float up = T::one(a[static_cast<int64_t>(row) * stride_a + col]);
-        const float gate = T::one(b[static_cast<int64_t>(row) * stride_b + col]);
-        c[static_cast<int64_t>(row) * stride_c + col] = T::narrow1(swiglu1_any(up, gate));
+    for (uint64_t g = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; g < groups; g += step) {
+        const uint64_t row = g / per_row, col = (g - row * per_row) * 8;
+        const uint16_t *pa = a + static_cast<int64_t>(row) * stride_a + col;
+        const uint16_t *pb = b + static_cast<int64_t>(row) * stride_b + col;
+        uint16_t *pc = c + static_cast<int64_t>(row) * stride_c + col;
+        // the ballot inside swiglu8 is over the lanes that are here: a wavefront's lanes with partial groups take the other side
+        if (col + 8 <= di) {
+            st16_any(pc, swiglu8<T>(ld16_any(pa), ld16_any(pb)));
+        } else {
+            for (uint64_t e = 0; col + e < di; ++e) pc[e] = T::narrow1(swiglu1_any(T::one(pa[e]), T::one(pb[e])));
+        }
     }
 }
 
@@ -179,7 +189,7 @@ void launch_swiglu(const SwiGLUAmdDescriptor &d, void *c, const void *a, const v
         return;
     }
     if (!vec_ok) {
-        const uint64_t want = ceil_div(n, kBlock), cap = static_cast<uint64_t>(d.cu_count) * 64;
+        const uint64_t want = ceil_div(d.rows * ceil_div(d.di, 8), kBlock), cap = max_grid_1d(kBlock);
         swiglu_scalar<T><<<static_cast<unsigned>(want < cap ? want : cap), kBlock, 0, stream>>>(
             pc, pa, pb, d.rows, d.di, d.stride_c, d.stride_a, d.stride_b);
         return;
