@@ -331,7 +331,7 @@ void causal_softmax_rows(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
 // kept length being a per-lane value; the sums are the same trees, one per
 // vector index k, added in the order the whole-wavefront tree adds its halves
 // (see segment_sum).
-template<typename T, int P, int NV, bool THROUGH, bool RAGGED>
+template<typename T, int P, int NV, bool THROUGH, bool RAGGED, bool ON16 = false>
 __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint64_t groups, uint32_t seq, uint32_t total,
                                                               int64_t stride_b, int64_t stride_i, FastDiv by_groups_per_matrix,
                                                               uint32_t groups_per_matrix) {
@@ -339,23 +339,31 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
     AMD_ARGS_NOW(y, groups, seq, total, stride_b, stride_i, arg_pair(by_groups_per_matrix), groups_per_matrix, gridDim.x);
     constexpr uint32_t RPW = kWave / P;// rows per wavefront
     const uint32_t sub = threadIdx.x % P, rr = threadIdx.x / P;
+    // ON16: RAGGED rows that all start on 16-byte boundaries.  They keep the streaming hint; on rows that do not,
+    // where neighbouring accesses share lines, it costs ([2048, 504, 504] fp16 305 with, 339 us without;
+    // [2048, 333, 333] 170 with, 159 without).
+    constexpr bool on_16 = ON16;
     const float neg_inf = -__builtin_inff();
     for (uint64_t g = blockIdx.x; g < groups; g += gridDim.x) {
         // group g of RPW rows: matrix b, rows i0 .. i0 + RPW - 1 (fewer than 2^31 groups, see FastDiv)
         const uint32_t b = fast_quotient(static_cast<uint32_t>(g), by_groups_per_matrix);
         const uint32_t i0 = (static_cast<uint32_t>(g) - b * groups_per_matrix) * RPW;
         uint16_t *base = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i0) * stride_i;// the same for every lane unless RAGGED
-        // RAGGED (see causal_softmax_rows): the vectors are the whole 16-byte aligned ones inside the row, the up to 7
-        // elements in front of them and the up to 7 behind are taken one each by the row's first lanes.  All per lane
+        // RAGGED: rows at any 2-byte boundary and of any length.  The vectors are the row's groups of 8 elements from
+        // its first element on, moved as 16 bytes at whatever boundary they lie on (gfx950 serves such accesses, at
+        // a fraction of the aligned rate); the up to 7 elements behind the last whole group are taken one each by the
+        // row's first lanes.  (Whole 16-byte aligned vectors inside the row instead, with the up to 7 elements in
+        // front of them taken one by one as well, measured the same where the mask cuts rows short and 15 % slower
+        // where it does not: [16384, 64, 250] fp16 224 against 192 us, [4096, 250, 250] 190 against 189.)  All per lane
         // here, and so is the row itself: a wavefront takes RPW consecutive rows of the whole tensor, whichever matrices
         // they lie in (the host passes the divisor of seq and the number of rows in place of the groups' figures), the
         // lanes behind the last row repeat it without storing.
         // What this form costs against rows in whole lines, from the counters ([4096, 250, 250] against [4096, 256, 256],
         // fp16, per launch): 1.27 times the bytes fetched (415 against 328 MB: a kept part that neither starts nor ends on
         // a line boundary brings in two partial lines per row instead of one), 1.14 times the vector instructions, 1.29
-        // times the busy cycles.  (One end element per lane instead of two, end loads issued unconditionally beside the
-        // vector loads, 32-bit row offsets for equally spaced rows, the end stores left out altogether: each within
-        // 2 % of this, [8192, 120, 120] 13 % slower.)
+        // times the busy cycles.  (With aligned vectors and end elements at both ends: one end element per lane
+        // instead of two, end loads issued unconditionally beside the vector loads, 32-bit row offsets for equally
+        // spaced rows, the end stores left out altogether - each within 2 %, [8192, 120, 120] 13 % slower.)
         // Nor is it the arithmetic that these rows wait for: with the exponential cut to one multiply and the
         // hardware exp2, and the quotient to one multiply - a third of the vector instructions gone, at the price of
         // three times as many outputs one unit off the float64 quotient - [8192, 256, 256] took 276 against 274 us,
@@ -363,10 +371,10 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
         // and [65536, 64, 64] (168 against 178) moved.
         const uint32_t row_off = RAGGED ? 0u : rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
         struct Mine {
-            uint16_t *row, *body;// the row's first element and its first whole vector
+            uint16_t *row;       // the row's first element
             uint32_t row_keep;   // columns kept of the row
-            uint32_t head, nvec; // elements in front of the vectors, vectors
-            uint32_t keep;       // columns kept of the vectors
+            uint32_t nvec;       // whole groups of 8 elements
+            uint32_t keep;       // columns kept of those groups
             bool valid;
         };
         const Mine mine = [&]() {
@@ -377,35 +385,33 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
                 const uint32_t rb = fast_quotient(rc, by_groups_per_matrix), ri = rc - rb * seq;
                 uint16_t *row = y + static_cast<int64_t>(rb) * stride_b + static_cast<int64_t>(ri) * stride_i;
                 const uint32_t row_keep = total - seq + ri + 1;
-                const uint32_t head = (8u - static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u) / 2) & 7u;
-                const uint32_t nvec = (total - head) / 8;
-                const uint32_t past = row_keep > head ? row_keep - head : 0u;
-                return Mine{row, row + head, row_keep, head, nvec, past < nvec * 8 ? past : nvec * 8, valid};
+                const uint32_t nvec = total / 8;
+                return Mine{row, row_keep, nvec, row_keep < nvec * 8 ? row_keep : nvec * 8, valid};
             } else {
                 const uint32_t row_keep = total - seq + i0 + rr + 1;
-                return Mine{base, base, row_keep, 0u, total / 8, row_keep, true};
+                return Mine{base, row_keep, total / 8, row_keep, true};
             }
         }();
-        const uint32_t row_keep = mine.row_keep, head = mine.head, nvec = mine.nvec, keep = mine.keep;
+        const uint32_t row_keep = mine.row_keep, nvec = mine.nvec, keep = mine.keep;
         [[maybe_unused]] uint16_t *const row = mine.row;
         [[maybe_unused]] const bool valid = mine.valid;
-        if constexpr (RAGGED) base = mine.body;
+        if constexpr (RAGGED) base = mine.row;
         const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = RAGGED && keep == 0 ? 0u : (keep - 1) / 8;
         u32x4 cur[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = sub + k * P;
-            cur[k] = ld16_stream(reinterpret_cast<const uint8_t *>(base) + row_off + (v < last_vec ? v : last_vec) * 16);
+            const uint8_t *at = reinterpret_cast<const uint8_t *>(base) + row_off + (v < last_vec ? v : last_vec) * 16;
+            cur[k] = RAGGED && !on_16 ? ld16_any(at) : ld16_stream(at);
         }
-        // the row's elements in front of its vectors (lane sub takes column sub) and behind them
+        // the row's elements behind its whole groups (lane sub takes the sub-th of them)
         [[maybe_unused]] uint32_t col_t = 0;
-        [[maybe_unused]] bool mine_h = false, mine_t = false, kept_h = false, kept_t = false;
-        [[maybe_unused]] float x_h = 0.0f, x_t = 0.0f;
+        [[maybe_unused]] bool mine_t = false, kept_t = false;
+        [[maybe_unused]] float x_t = 0.0f;
         if constexpr (RAGGED) {
-            col_t = head + nvec * 8 + sub;
-            mine_h = sub < head, mine_t = col_t < total;// P >= 8 lanes, at most 7 elements at either end
-            kept_h = mine_h && sub < row_keep, kept_t = mine_t && col_t < row_keep;
-            if (kept_h) x_h = T::one(row[sub]);
+            col_t = nvec * 8 + sub;
+            mine_t = col_t < total;// P >= 8 lanes, at most 7 elements
+            kept_t = mine_t && col_t < row_keep;
             if (kept_t) x_t = T::one(row[col_t]);
         }
 
@@ -443,23 +449,22 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
             }
         }
         if constexpr (RAGGED) {
-            if (kept_h) mx = fmaxf(mx, x_h), mn = fminf(mn, x_h);
             if (kept_t) mx = fmaxf(mx, x_t), mn = fminf(mn, x_t);
         }
         mx = segment_max<P>(mx);
 
         const float lowest = mn - mx;// +inf - max for a lane without kept elements: passes the test below
         const bool lean = __builtin_amdgcn_ballot_w64(!(lowest >= kLeanExpLimit)) == 0;
-        [[maybe_unused]] float e_h = 0.0f, e_t = 0.0f;
+        [[maybe_unused]] float e_t = 0.0f;
         if constexpr (RAGGED) {
             if (lean) {
-                e_h = exp_nonpositive(x_h - mx), e_t = exp_nonpositive(x_t - mx);
+                e_t = exp_nonpositive(x_t - mx);
             } else {
-                float slow[8] = {x_h, x_t, mx, mx, mx, mx, mx, mx};
+                float slow[8] = {x_t, mx, mx, mx, mx, mx, mx, mx};
                 exp_any8(slow, mx);
-                e_h = slow[0], e_t = slow[1];
+                e_t = slow[0];
             }
-            e_h = kept_h ? e_h : 0.0f, e_t = kept_t ? e_t : 0.0f;
+            e_t = kept_t ? e_t : 0.0f;
         }
         float tree[NV];
 #pragma unroll
@@ -493,7 +498,7 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
                 for (int e = 0; e < 8; ++e) part += f[k][e];
             }
             if constexpr (RAGGED) {
-                if (k == 0) part += e_h + e_t;
+                if (k == 0) part += e_t;
             }
             tree[k] = segment_sum<P>(part);
         }
@@ -531,7 +536,10 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
                 }
             }
             if constexpr (RAGGED) {
-                if (valid && v < nvec) st16_stream(base + v * 8, packed);
+                if (valid && v < nvec) {
+                    if (on_16) st16_stream(base + v * 8, packed);
+                    else st16_any(base + v * 8, packed);
+                }
             } else {
                 if (v < nvec) out.st16(row_off + v * 16, packed);
             }
@@ -541,7 +549,6 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
                 const float q = e * rcp;
                 return static_cast<uint16_t>(T::narrow2_fast(__builtin_fmaf(__builtin_fmaf(-sum, q, e), rcp, q), 0.0f) & 0xFFFFu);
             };
-            if (valid && mine_h) row[sub] = kept_h ? one(e_h) : uint16_t{0};
             if (valid && mine_t) row[col_t] = kept_t ? one(e_t) : uint16_t{0};
         }
     }
@@ -1028,15 +1035,17 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
             const uint32_t gpm = static_cast<uint32_t>(d.seq / rpw);
             const uint64_t capg = static_cast<uint64_t>(d.cu_count) * 2048;
             const unsigned g = static_cast<unsigned>(std::min(groups, capg));
-#define CS_SHORT_GO(P, NV, TH, RG)                                                                                             \
-    causal_softmax_short<T, P, NV, TH, RG><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
-                                                                    d.stride_b, d.stride_i, RG ? by_seq : fast_div(gpm), RG ? static_cast<uint32_t>(rows) : gpm)
+#define CS_SHORT_GO(P, NV, TH, RG, ON16)                                                                                       \
+    causal_softmax_short<T, P, NV, TH, RG, ON16><<<g, kWave, 0, stream>>>(py, groups, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), \
+                                                                          d.stride_b, d.stride_i, RG ? by_seq : fast_div(gpm), RG ? static_cast<uint32_t>(rows) : gpm)
 #define CS_SHORT(P, NV)                                                                                                        \
     do {                                                                                                                       \
-        if (through && together) CS_SHORT_GO(P, NV, true, false);                                                              \
-        else if (through) CS_SHORT_GO(P, NV, true, true);                                                                      \
-        else if (together) CS_SHORT_GO(P, NV, false, false);                                                                   \
-        else CS_SHORT_GO(P, NV, false, true);                                                                                  \
+        if (through && together) CS_SHORT_GO(P, NV, true, false, false);                                                       \
+        else if (through && aligned) CS_SHORT_GO(P, NV, true, true, true);                                                     \
+        else if (through) CS_SHORT_GO(P, NV, true, true, false);                                                               \
+        else if (together) CS_SHORT_GO(P, NV, false, false, false);                                                            \
+        else if (aligned) CS_SHORT_GO(P, NV, false, true, true);                                                               \
+        else CS_SHORT_GO(P, NV, false, true, false);                                                                           \
     } while (0)
             switch (lanes * 10 + per_lane) {
                 case 81: CS_SHORT(8, 1); break;
