@@ -45,17 +45,29 @@ template<> struct Unit<4> { typedef uint32_t type; };
 template<> struct Unit<2> { typedef uint16_t type; };
 template<> struct Unit<1> { typedef uint8_t type; };
 
+// ANY: rows of at least 16 bytes whose length, strides or bases are no multiples of 16.  The row still moves in
+// 16-byte units, at whatever byte boundary they lie on (gfx950 serves such accesses, at a fraction of the
+// aligned rate), and the last unit of a row is the row's last 16 bytes, overlapping the one before it: a
+// copy may write a byte twice.  bf16 [8192, 64, 127] out of [8192, 80, 127]: 141 us in 2-byte units.
+typedef u32x4 __attribute__((aligned(1))) u32x4_bytes;
+__device__ __forceinline__ uint32_t unit_offset_any(uint32_t col, uint32_t last_offset) {
+    const uint32_t at = col * 16;
+    return at < last_offset ? at : last_offset;
+}
+
 // blockIdx.y walks the rows, blockIdx.x the units of a row: rows of at least a
 // wavefront of units.  The row's offsets are found by splitting the row number
 // by the merged outer extents - once per workgroup row, on the scalar unit,
 // since the row number is uniform, and by multiplication (see FastDiv).
 // BUFST (16-byte units, large outputs): stores are written through L2 as
 // buffer stores relative to the start of the destination row (see StreamOut).
-template<int BYTES, bool BUFST, int LANES>
-__global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row) {
+template<int BYTES, bool BUFST, int LANES, bool ANY = false>
+__global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t rows, uint32_t units_per_row,
+                                                        uint32_t last_offset) {
     typedef typename Unit<BYTES>::type U;
+    static_assert(!ANY || (BYTES == 16 && !BUFST), "ANY: 16-byte units at any boundary, plain stores");
     // every argument up front (see AMD_ARGS_NOW; the number of rows to step by is not needed before the first load is out)
-    AMD_ARGS_NOW(dst, src, rows, units_per_row, ARGS_OF_DIMS(d));
+    AMD_ARGS_NOW(dst, src, rows, units_per_row, last_offset, ARGS_OF_DIMS(d));
     const uint32_t col = blockIdx.x * LANES + threadIdx.x;
     if (col >= units_per_row) return;
     for (uint64_t r = blockIdx.y; r < rows; r += gridDim.y) {
@@ -71,11 +83,16 @@ __global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint
                 os += static_cast<int64_t>(i) * d.src_stride[k];
             }
         }
-        const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
-        if constexpr (BUFST) {
-            StreamOut<true>(dst + od).st16(col * 16, v);
+        if constexpr (ANY) {
+            const uint32_t at = unit_offset_any(col, last_offset);
+            *reinterpret_cast<u32x4_bytes *>(dst + od + at) = *reinterpret_cast<const u32x4_bytes *>(src + os + at);
         } else {
-            __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+            const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
+            if constexpr (BUFST) {
+                StreamOut<true>(dst + od).st16(col * 16, v);
+            } else {
+                __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+            }
         }
     }
 }
@@ -85,11 +102,12 @@ __global__ __launch_bounds__(LANES) void rearrange_rows(uint8_t *dst, const uint
 // allows, which makes the divisions cheap.  BUFST (16-byte units only): the
 // whole destination lies within 4 GiB of its base and no stride is negative,
 // so stores go out as buffer stores relative to the base (see StreamOut).
-template<int BYTES, typename Idx, bool BUFST, bool FAST>
+template<int BYTES, typename Idx, bool BUFST, bool FAST, bool ANY = false>
 __global__ __launch_bounds__(Lanes<BYTES>::value) void rearrange_flat(uint8_t *dst, const uint8_t *src, OuterDims d, uint64_t total_units, Idx units_per_row,
-                                                                    FastDiv by_row) {
+                                                                    FastDiv by_row, uint32_t last_offset) {
     typedef typename Unit<BYTES>::type U;
-    AMD_ARGS_NOW(dst, src, total_units, units_per_row, arg_pair(by_row), gridDim.x, ARGS_OF_DIMS(d));
+    static_assert(!ANY || (BYTES == 16 && !BUFST), "ANY: 16-byte units at any boundary, plain stores");
+    AMD_ARGS_NOW(dst, src, total_units, units_per_row, arg_pair(by_row), last_offset, gridDim.x, ARGS_OF_DIMS(d));
     // one pass for anything a single launch can span (2^32 work-items); the loop covers the rest
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * Lanes<BYTES>::value;
     for (uint64_t idx64 = static_cast<uint64_t>(blockIdx.x) * Lanes<BYTES>::value + threadIdx.x; idx64 < total_units; idx64 += step) {
@@ -125,20 +143,26 @@ __global__ __launch_bounds__(Lanes<BYTES>::value) void rearrange_flat(uint8_t *d
                 }
             }
         }
-        const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
-        if constexpr (BUFST) {
-            StreamOut<true>(dst).st16(static_cast<uint32_t>(od) + static_cast<uint32_t>(col) * 16, v);
+        if constexpr (ANY) {
+            const uint32_t at = unit_offset_any(static_cast<uint32_t>(col), last_offset);
+            *reinterpret_cast<u32x4_bytes *>(dst + od + at) = *reinterpret_cast<const u32x4_bytes *>(src + os + at);
         } else {
-            __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+            const U v = __builtin_nontemporal_load(reinterpret_cast<const U *>(src + os) + col);
+            if constexpr (BUFST) {
+                StreamOut<true>(dst).st16(static_cast<uint32_t>(od) + static_cast<uint32_t>(col) * 16, v);
+            } else {
+                __builtin_nontemporal_store(v, reinterpret_cast<U *>(dst + od) + col);
+            }
         }
     }
 }
 
-template<int BYTES>
+template<int BYTES, bool ANY = false>
 void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, const void *src, hipStream_t stream) {
     auto *pd = static_cast<uint8_t *>(dst);
     auto *ps = static_cast<const uint8_t *>(src);
-    const uint64_t upr = desc.row_bytes / BYTES;
+    const uint64_t upr = ANY ? ceil_div(desc.row_bytes, BYTES) : desc.row_bytes / BYTES;
+    const uint32_t last_offset = ANY ? static_cast<uint32_t>(desc.row_bytes - 16) : 0;// ANY: rows of 16 bytes to 4 GiB
     constexpr int kBlock = Lanes<BYTES>::value;
     const bool large = desc.rows * desc.row_bytes >= kWriteThroughBytes;// worth writing through L2
     // where the destination ends, in bytes from its base, when no stride is negative
@@ -168,12 +192,12 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         const bool half = !wave_rows && ceil_div(upr, 128) * 128 < ceil_div(upr, 256) * 256;
         const int lanes = wave_rows ? kWave : (half ? 128 : 256);
         const dim3 grid(static_cast<unsigned>(ceil_div(upr, lanes)), static_cast<unsigned>(desc.rows < 65535 ? desc.rows : 65535));
-        const bool bufst = BYTES == 16 && large && desc.row_bytes < (1ull << 32);
+        const bool bufst = BYTES == 16 && !ANY && large && desc.row_bytes < (1ull << 32);
         const uint32_t upr32 = static_cast<uint32_t>(upr);
 #define REARRANGE_ROWS_OF(LANES)                                                                                           \
     do {                                                                                                                   \
-        if (bufst) rearrange_rows<BYTES, BYTES == 16, LANES><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32);     \
-        else rearrange_rows<BYTES, false, LANES><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32);                 \
+        if (bufst) rearrange_rows<BYTES, BYTES == 16 && !ANY, LANES, ANY><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32, last_offset); \
+        else rearrange_rows<BYTES, false, LANES, ANY><<<grid, LANES, 0, stream>>>(pd, ps, d, desc.rows, upr32, last_offset); \
     } while (0)
         if constexpr (BYTES == 16) {
             if (wave_rows) {
@@ -189,13 +213,13 @@ void launch(const RearrangeAmdDescriptor &desc, const OuterDims &d, void *dst, c
         const uint64_t want = ceil_div(total, kBlock);
         const uint64_t blocks = want < max_grid_1d(kBlock) ? want : max_grid_1d(kBlock);
         const unsigned grid = static_cast<unsigned>(blocks);
-        const bool bufst = BYTES == 16 && large && forward && dst_span < (1ull << 32);
+        const bool bufst = BYTES == 16 && !ANY && large && forward && dst_span < (1ull << 32);
         if (total < kFastDivLimit) {
             const FastDiv by_row = fast_div(static_cast<uint32_t>(upr));
-            if (bufst) rearrange_flat<BYTES, uint32_t, BYTES == 16, true><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row);
-            else rearrange_flat<BYTES, uint32_t, false, true><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row);
+            if (bufst) rearrange_flat<BYTES, uint32_t, BYTES == 16 && !ANY, true, ANY><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row, last_offset);
+            else rearrange_flat<BYTES, uint32_t, false, true, ANY><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, static_cast<uint32_t>(upr), by_row, last_offset);
         } else {
-            rearrange_flat<BYTES, uint64_t, false, false><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, upr, FastDiv{});
+            rearrange_flat<BYTES, uint64_t, false, false, ANY><<<grid, kBlock, 0, stream>>>(pd, ps, d, total, upr, FastDiv{}, last_offset);
         }
     }
 }
@@ -226,7 +250,13 @@ infiniopStatus_t amdRearrange(RearrangeAmdDescriptor_t desc, void *dst, void con
     }
     AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (align % 16 == 0) launch<16>(*desc, d, dst, src, s);
+    // Rows that all start and end on 128-byte boundaries stream past the caches; rows that share lines with their
+    // neighbours go through them, in 16-byte units at whatever boundary (bf16 [8192, 64, hd] out of [8192, 80, hd],
+    // us, streaming hints against none: hd 104  78.7 / 37.7, hd 120  77.8 / 56.5, hd 200  123 / 102, hd 504  245 / 241;
+    // [16384, 4104] out of a pitch of 4120  47.5 / 46.7).
+    const bool any_ok = desc->row_bytes >= 16 && desc->row_bytes < (1ull << 32);
+    if (align % 16 == 0 && (align % 128 == 0 || !any_ok)) launch<16>(*desc, d, dst, src, s);
+    else if (any_ok) launch<16, true>(*desc, d, dst, src, s);
     else if (align % 8 == 0) launch<8>(*desc, d, dst, src, s);
     else if (align % 4 == 0) launch<4>(*desc, d, dst, src, s);
     else if (align % 2 == 0) launch<2>(*desc, d, dst, src, s);

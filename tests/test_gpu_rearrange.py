@@ -65,6 +65,16 @@ CASES = [
     # 128 MiB outputs: large enough for the write-through store path of both kernels
     ("bf16", (8192, 64, 128), (80 * 128, 128, 1), (128, 8192 * 128, 1)),     # q heads -> [head, token, dim], 256-byte rows
     ("f16", (4096, 16384), (16384, 1), (16392, 1)),                          # long rows into a padded destination
+    # rows of 16 bytes and more that do not lie on 16-byte boundaries: 16-byte units at any boundary, the last one overlapping
+    ("u8", (37, 17), (19, 1), (23, 1)),                                      # one whole unit and an overlapping one, odd pitches
+    ("u8", (5, 3, 16), (3 * 17, 17, 1), (48, 16, 1)),                        # rows of exactly one unit at odd addresses
+    ("u8", (11, 255), (300, 1), (257, 1)),
+    ("f16", (513, 127), (131, 1), (127, 1)),                                 # 254-byte rows, the flat form
+    ("bf16", (64, 8, 127), (10 * 127, 127, 1), (127, 64 * 127, 1)),          # heads of odd width -> [head, token, dim]
+    ("f16", (9, 4095), (4099, 1), (4095, 1)),                                # rows of more than a wavefront of units: the row form
+    ("f16", (3, 20001), (20003, 1), (20001, 1)),
+    ("f16", (300, 120), (128, 1), (120, 1)),                                 # on 16-byte but not on 128-byte boundaries
+    ("f32", (70, 33), (35, 1), (33, 1)),
 ]
 
 
@@ -86,7 +96,7 @@ def test_against_oracle(ctx, case):
 
 
 def test_misaligned_base_pointers(ctx):
-    """Views that start 2 bytes into their buffers fall back to narrower units."""
+    """Views that start 2 bytes into their buffers: 16-byte units at that boundary; what lies in front of and between the rows stays."""
     import torch
 
     rng = np.random.default_rng(950)
