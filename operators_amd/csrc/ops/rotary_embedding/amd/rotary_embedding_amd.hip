@@ -188,24 +188,48 @@ __global__ __launch_bounds__(BS) void rope_once(uint16_t *__restrict__ t, const 
     }
 }
 
-// Any even head_dim, any strides and alignment: one lane per pair.
+// Any even head_dim, any strides and alignment.  A lane takes 8 consecutive
+// elements (4 pairs) of one head: a whole group moves as 16 bytes at whatever
+// 2-byte boundary it lies on, with its 2 x 8 table values as 16-byte loads at
+// their 4-byte boundary (gfx950 serves such accesses, at a fraction of the
+// aligned rate); a head's last, partial group pair by pair.  [8192, 64, 128]
+// bf16 one element into its buffer: 119 us with one lane per pair.
 template<typename T>
 __global__ __launch_bounds__(kBlock) void rope_pairs(uint16_t *t, const uint64_t *pos, const float *sin_t, const float *cos_t,
-                                                     uint64_t total_pairs, uint64_t heads, uint64_t head_dim,
+                                                     uint64_t total_groups, uint64_t heads, uint64_t head_dim,
                                                      int64_t stride_token, int64_t stride_head) {
-    const uint64_t half = head_dim / 2;
+    const uint64_t per_head = (head_dim + 7) / 8;
     const uint64_t step = static_cast<uint64_t>(gridDim.x) * kBlock;
-    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < total_pairs; i += step) {
-        const uint64_t k = i % half;
-        const uint64_t th = i / half;
-        const uint64_t h = th % heads, token = th / heads;
-        uint16_t *p = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(h) * stride_head + 2 * k;
-        const uint64_t row = pos[token] * head_dim + 2 * k;
-        const float a = T::one(p[0]), b = T::one(p[1]);
-        const float ac = a * cos_t[row], bs = b * sin_t[row];
-        const float as = a * sin_t[row + 1], bc = b * cos_t[row + 1];
-        p[0] = T::narrow1(ac - bs);
-        p[1] = T::narrow1(as + bc);
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < total_groups; i += step) {
+        const uint64_t th = i / per_head, col = (i - th * per_head) * 8;
+        const uint64_t token = th / heads, h = th - token * heads;
+        uint16_t *p = t + static_cast<int64_t>(token) * stride_token + static_cast<int64_t>(h) * stride_head + col;
+        const uint64_t row = pos[token] * head_dim + col;
+        if (col + 8 <= head_dim) {
+            float f[8], r[8];
+            widen8<T>(ld16_any(p), f);
+            const f32x4 s_lo = *reinterpret_cast<const f32x4_any *>(sin_t + row), s_hi = *reinterpret_cast<const f32x4_any *>(sin_t + row + 4);
+            const f32x4 c_lo = *reinterpret_cast<const f32x4_any *>(cos_t + row), c_hi = *reinterpret_cast<const f32x4_any *>(cos_t + row + 4);
+            const float sn[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+            const float cs[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+#pragma unroll
+            for (int k = 0; k < 8; k += 2) {
+                const float a = f[k], b = f[k + 1];
+                const float ac = a * cs[k], bs = b * sn[k];
+                const float as = a * sn[k + 1], bc = b * cs[k + 1];
+                r[k] = ac - bs;
+                r[k + 1] = as + bc;
+            }
+            st16_any(p, narrow8<T>(r));
+        } else {
+            for (uint64_t k = 0; col + k < head_dim; k += 2) {
+                const float a = T::one(p[k]), b = T::one(p[k + 1]);
+                const float ac = a * cos_t[row + k], bs = b * sin_t[row + k];
+                const float as = a * sin_t[row + k + 1], bc = b * cos_t[row + k + 1];
+                p[k] = T::narrow1(ac - bs);
+                p[k + 1] = T::narrow1(as + bc);
+            }
+        }
     }
 }
 
@@ -311,10 +335,10 @@ void launch_rope(const RoPEAmdDescriptor &d, void *t, const void *pos_ids, const
                         aligned16(t) && aligned16(sin_table) && aligned16(cos_table) &&
                         d.heads < (1ull << 31) && d.head_dim < (1ull << 31) && elems / 8 < (1ull << 38);
     if (!vec_ok) {
-        const uint64_t pairs = elems / 2;
-        const uint64_t want = ceil_div(pairs, kBlock), cap = static_cast<uint64_t>(d.cu_count) * 64;
+        const uint64_t groups = d.tokens * d.heads * ceil_div(d.head_dim, 8);
+        const uint64_t want = ceil_div(groups, kBlock), cap = max_grid_1d(kBlock);
         rope_pairs<T><<<static_cast<unsigned>(want < cap ? want : cap), kBlock, 0, stream>>>(
-            pt, pos, sn, cs, pairs, d.heads, d.head_dim, d.stride_token, d.stride_head);
+            pt, pos, sn, cs, groups, d.heads, d.head_dim, d.stride_token, d.stride_head);
         return;
     }
     if (elems / 8 < (1ull << 31)) launch_vec<T, uint32_t>(d, pt, pos, sn, cs, stream);
