@@ -104,18 +104,22 @@ def test_in_place(ctx, which):
     assert_codes_equal(to_codes(tc), want, "f16", what=f"in place on {which}")
 
 
-def test_misaligned_pointers_take_the_element_path(ctx):
+@pytest.mark.parametrize("n", [5, 5000, 5003, 1 << 20])
+def test_misaligned_pointers(ctx, n):
+    """Operands that start on different 2-byte boundaries: the same vectors as 16-byte accesses at those
+    boundaries, the last few elements one by one; what lies in front of and behind c stays."""
     import torch
 
     rng = np.random.default_rng(6)
-    n = 5000
     a = oracle.encode(rng.standard_normal(n + 3).astype(np.float32), "f16")
     b = oracle.encode(rng.standard_normal(n + 5).astype(np.float32), "f16")
     ta, tb = to_torch(a, "f16")[3:], to_torch(b, "f16")[5:]  # 2-byte aligned only
-    tc = torch.empty(n + 1, dtype=torch.float16, device="cuda")[1:]
+    whole = torch.full((n + 2,), 7.0, dtype=torch.float16, device="cuda")
+    tc = whole[1:n + 1]
     ctx.add(tc, ta, tb)
     torch.cuda.synchronize()
     assert_codes_equal(to_codes(tc), oracle.add(a[3:].copy(), b[5:].copy(), (n,), "f16"), "f16", what="misaligned")
+    assert whole[0] == 7.0 and whole[n + 1] == 7.0
 
 
 def test_more_than_2_to_31_elements_uses_64_bit_indexing(ctx):
