@@ -925,7 +925,16 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
         return;
     }
     if (nvec > 256 && nvec <= 512 && once_fits(256, 1)) {
-        RMS_ONCE(256, 2, 1);
+        // fp32 weights are twice the row's own bytes through L2: two rows per workgroup share them where the
+        // lanes are not all busy anyway (64 MiB of bf16 rows, us, one row per workgroup / two: d = 2304  52.1 / 47.6,
+        // 2560  49.9 / 46.9, 3072  49.2 / 46.5, 3584  48.4 / 46.6, 3840  48.8 / 47.0; 4096  45.7 / 46.3; with 16-bit
+        // weights one row per workgroup runs all of these in 44.3-45.1; the fused form loses by two: 3072  90.0 / 93.5)
+        bool pair = false;
+        if constexpr (!ADD) pair = w_kind == kWKindF32 && nvec < 512 && once_fits(256, 2);
+        if constexpr (!ADD) {
+            if (pair) RMS_ONCE(256, 2, 2);
+        }
+        if (!pair) RMS_ONCE(256, 2, 1);
         return;
     }
     if constexpr (ADD) {
