@@ -936,7 +936,12 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const bool in_lines = aligned && d.stride_i % 64 == 0 && d.stride_b % 64 == 0 && (reinterpret_cast<uintptr_t>(data) & 127u) == 0;// rows start on 128-byte boundaries
     // Vectors per row that the kernel must have room for.  The ragged form takes up to 56 elements behind them one by one
     // (see causal_softmax_rows), which rows in whole lines also use when that spares them the next larger form.
-    const auto form_of = [](uint64_t vectors) { return vectors <= 64 ? 0 : 64 - __builtin_clzll(vectors - 1) - 6; };// 64, 128, 256, ... vectors
+    const auto form_of = [](uint64_t vectors) {// the vectors the launch shape for that many has room for (the ladder at the end of this function)
+        for (const uint64_t room : {64, 128, 192, 256, 384, 512, 640, 768, 1024, 1280, 1536, 1792, 2048, 2560, 3072}) {
+            if (vectors <= room) return room;
+        }
+        return uint64_t{4096};
+    };
     const uint64_t spared = d.total <= 56 ? 1 : ceil_div(d.total - 56, 8);
     const bool ragged = !in_lines || form_of(spared) < form_of(nvec);
     const uint64_t cover = ragged ? spared : nvec;
@@ -1087,16 +1092,32 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     // and the plain form, which used to take those on 16-byte boundaries):
     //   [32, 4095, 4095]  285 (1033)   [32, 1024, 4099]  85 (392)   [64, 512, 1027]  24 (78)   [256, 128, 333]  18 (45)
     //   [32, 4088, 4088]  278 (360)    [32, 4100, 4104]  281 (450)  [32, 2048, 2056]  74 (100)  [128, 1000, 1000]  72 (83)
+    // Lanes x vectors per lane: the tightest fit, with the fewer lanes where two fit equally.  Every shape that covers
+    // the row was timed at 28 row lengths, square causal matrices [h, n, n] and chunks of 512 queries [h, 512, n], fp16
+    // (us, this ladder against the powers of two - 64 x 8, 256 x 2, 256 x 4, 512 x 4, 512 x 8 - it replaces):
+    //   n = 1536   75 /  77      2560  206 / 229     3500  285 / 323     5000  271 / 312     6144  257 / 272
+    //   n = 9000  256 / 365     10240  256 / 331    12288  220 / 257    14000  204 / 228    20480  213 / 225   (square)
+    //   n = 2560  167 / 179      5120  165 / 180     9216  160 / 207    10240  166 / 192    12288  171 / 183   (512 queries)
+    // (512 lanes x 7 vectors is the one shape to stay away from: 354-611 us where 512 x 6 and 512 x 8 take 308-429.)
+    const bool mostly_masked = d.seq * 2 > d.total;// a causal square: half of every matrix is masked
     if (cover <= 64) CS_LAUNCH(64, 1);
     else if (cover <= 128) CS_LAUNCH(64, 2);
-    else if (cover <= 256 && cover > 192 && !ragged && !T::kPackedMinMax) CS_LAUNCH(128, 2);// bf16 rows of 2048 in whole lines: 257 against 269 us
-                                                                                              // (fp16 264 / 269 at seq 2048, 158 / 155 at seq 512; 1536 columns 173 / 150; ragged 2047: 299 / 281)
+    else if (cover <= 192) CS_LAUNCH(64, 3);
+    else if (cover <= 256 && !ragged && !T::kPackedMinMax) CS_LAUNCH(128, 2);// bf16 rows of 2048 in whole lines: 257 against 269 us
+                                                                              // (fp16 264 / 269 at seq 2048, 158 / 155 at seq 512; ragged 2047: 299 / 281)
     else if (cover <= 256) CS_LAUNCH(64, 4);
-    else if (cover <= 384) CS_LAUNCH(64, 8);
-    else if (cover <= 512) CS_LAUNCH(256, 2);// four wavefronts x 2 vectors.  [32, 4096, 4096] fp16 / bf16: 261 / 256 us; two x 4: 261 / 260; one x 8: 265 / 269.
-                                            // [64, 512, 4096]: 80 / 80, 82 / 83, 83 / 88.  At 384 vectors one wavefront x 8 is 1-2 % ahead; 512 lanes x 1 vector: 348 / 339 us.
+    else if (cover <= 384) CS_LAUNCH(64, 6);
+    else if (cover <= 512 && mostly_masked) CS_LAUNCH(128, 4);// [33, 4000, 4000] 260 against 273 us with 256 x 2; [32, 4096, 4096] 259-261 either way
+    else if (cover <= 512) CS_LAUNCH(256, 2);                 // [128, 512, 4096] 155 against 163 us with 128 x 4
+    else if (cover <= 640) CS_LAUNCH(128, 5);
+    else if (cover <= 768) CS_LAUNCH(256, 3);
     else if (cover <= 1024) CS_LAUNCH(256, 4);
-    else if (cover <= 2048) CS_LAUNCH(512, 4);
+    else if (cover <= 1280) CS_LAUNCH(256, 5);
+    else if (cover <= 1536) CS_LAUNCH(256, 6);
+    else if (cover <= 1792) CS_LAUNCH(256, 7);
+    else if (cover <= 2048) CS_LAUNCH(256, 8);
+    else if (cover <= 2560) CS_LAUNCH(512, 5);
+    else if (cover <= 3072) CS_LAUNCH(512, 6);
     else CS_LAUNCH(512, 8);
 #undef CS_LAUNCH
 #undef CS_GO
