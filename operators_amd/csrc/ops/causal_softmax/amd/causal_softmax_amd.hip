@@ -916,7 +916,8 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
     // Rows of up to 3072 elements are taken by single wavefronts (no barrier, no
-    // LDS), longer ones by 128, 256 or 512 lanes.  Measured on MI355X, fp16 / bf16 (rows of 4096 with one wavefront):
+    // LDS), longer ones by 128, 256 or 512 lanes (the ladder at the end of this function).  Measured on MI355X,
+    // fp16 / bf16 (rows of 4096 with one wavefront):
     //   [32, 4096, 4096]   one workgroup per row 264 / 261-266 us (76 %), 256 workgroups per
     //                      compute unit 267 / 267-274, 64 per unit 293 / 292-299; 128 or 256
     //                      lanes per row 264-288 / 261-270
