@@ -769,7 +769,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
 // taking row r * m mod rows instead of row r, for fourteen odd m from 3 to
 // 12 289, ran [64, 512, 65536] in 1566 (m = 513) to 1800 us (m = 1025)
 // against 1664, and [64, 512, 32768] in 796-814 against 799.)
-template<typename T, int BS, int NV, bool THROUGH>
+template<typename T, int BS, int NV, bool THROUGH, bool TURN>
 __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(4)))
 void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total, int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
     AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
@@ -784,7 +784,21 @@ void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
         uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
         const uint32_t keep = total - seq + i + 1;
         const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = (keep - 1) / 8;
-        auto vector_at = [&](int k) { return static_cast<uint32_t>(k * BS + threadIdx.x); };
+        // TURN: rows that start inside a 128-byte line.  Lanes take the vectors turned by the row's distance from
+        // the line's start, the first few lanes of the first turn the last vectors there is room for, so that a
+        // wavefront's 1 KiB per instruction is whole lines ([34, 512, 45000] fp16 657 -> 526 us, [47, 512, 33000]
+        // 674 -> 585).  A form of its own: on rows in whole lines it costs 1-1.5 %, and the 20-vector form has no
+        // register left for it.
+        static_assert(!TURN || NV < 20, "no register left for the turn");
+        [[maybe_unused]] const uint32_t turn = TURN ? static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 127u) / 16 : 0u;
+        auto vector_at = [&](int k) {
+            if constexpr (TURN) {
+                const uint32_t s = static_cast<uint32_t>(k * BS + threadIdx.x) - turn;
+                return k == 0 && static_cast<int32_t>(s) < 0 ? s + NV * BS : s;
+            } else {
+                return static_cast<uint32_t>(k * BS + threadIdx.x);
+            }
+        };
         u32x4 cur[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -961,17 +975,21 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         const bool thr = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
         const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
         if (aligned && nvec <= 16 * 1024) {// up to 131 072 elements: held in registers, read once (see causal_softmax_held)
-            const unsigned lanes = nvec <= 20 * 512 ? 512 : 1024;
+            // rows off the 128-byte boundaries skip the 20-vector form, which has no turned variant
+            const uint64_t most_512 = in_lines ? 20 * 512 : 16 * 512;
+            const unsigned lanes = nvec <= most_512 ? 512 : 1024;
             const unsigned g = static_cast<unsigned>(std::min<uint64_t>(rows, amd::max_grid_1d(lanes)));
-#define CS_HELD_GO(BS, NV, TH) causal_softmax_held<T, BS, NV, TH><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)
-#define CS_HELD(BS, NV)               \
-    do {                              \
-        if (thr) CS_HELD_GO(BS, NV, true); \
-        else CS_HELD_GO(BS, NV, false);    \
+#define CS_HELD_GO(BS, NV, TH, TURN) causal_softmax_held<T, BS, NV, TH, TURN><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)
+#define CS_HELD(BS, NV)                                                 \
+    do {                                                                \
+        if (thr && (in_lines || NV >= 20)) CS_HELD_GO(BS, NV, true, false); \
+        else if (thr) CS_HELD_GO(BS, NV, true, (NV < 20));              \
+        else if (in_lines || NV >= 20) CS_HELD_GO(BS, NV, false, false); \
+        else CS_HELD_GO(BS, NV, false, (NV < 20));                      \
     } while (0)
             if (nvec <= 12 * 512) CS_HELD(512, 12);
             else if (nvec <= 16 * 512) CS_HELD(512, 16);
-            else if (nvec <= 20 * 512) CS_HELD(512, 20);
+            else if (nvec <= most_512) CS_HELD(512, 20);
             else if (nvec <= 12 * 1024) CS_HELD(1024, 12);
             else if (nvec <= 14 * 1024) CS_HELD(1024, 14);
             else CS_HELD(1024, 16);
