@@ -462,7 +462,7 @@ def ops_table(ctx, args, gen):
         "N1b causal_softmax bf16 [32,4096,4096] (the Attention row's softmax on its own)": lambda: [make_causal_softmax(ctx, 32, 4096, 4096, bf16, gen, "causal_softmax") for _ in range(2)],
         "N1c causal_softmax f16 [2048,512,512] (short rows: two to a wavefront)": lambda: [make_causal_softmax(ctx, 2048, 512, 512, f16, gen, "causal_softmax") for _ in range(2)],
         "N1d causal_softmax f16 [32,4095,4095] (ragged rows: every row starts at another 2-byte offset in its 128-byte line)": lambda: [make_causal_softmax(ctx, 32, 4095, 4095, f16, gen, "causal_softmax") for _ in range(2)],
-        "N1e causal_softmax f16 [64,512,20480] (a chunk of 512 queries against 20480 keys: 512 lanes x 8 vectors)": lambda: [make_causal_softmax(ctx, 64, 512, 20480, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1e causal_softmax f16 [64,512,20480] (a chunk of 512 queries against 20480 keys: 512 lanes x 5 vectors)": lambda: [make_causal_softmax(ctx, 64, 512, 20480, f16, gen, "causal_softmax") for _ in range(2)],
         "N1f causal_softmax f16 [64,512,65536] (rows of 128 KiB held in registers as raw words, read once; the row stride is a power of two)": lambda: [make_causal_softmax(ctx, 64, 512, 65536, f16, gen, "causal_softmax") for _ in range(2)],
         "N1g causal_softmax f16 [64,512,40000] (the same form, 12 vectors per lane, a row stride that is no power of two)": lambda: [make_causal_softmax(ctx, 64, 512, 40000, f16, gen, "causal_softmax") for _ in range(2)],
         "Q2 rms_norm bf16 [4096,32768] w f32 (one 1024-lane workgroup per compute unit, 128 KiB of weights in LDS)": lambda: [make_rms_norm(ctx, 4096, 32768, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * 4096 * 32768, nset))],
