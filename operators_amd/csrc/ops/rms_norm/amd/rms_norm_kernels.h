@@ -875,6 +875,9 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // One pass re-reads the weight row through L2 once per R rows - at d = 8192
     // that is twice the bytes of the row itself - which is what it loses to
     // the looping form there; the fused form moves twice the data per weight.
+    // (Every one-pass shape of 64-512 lanes x 1-4 vectors x 1, 2 or 4 rows that covers the row, timed at eleven
+    // widths from 768 to 4096, plain with fp32 and with 16-bit weights and fused: the best of them is 0-3 % ahead
+    // of the shapes below, 384 x 1 x 2 at d = 2560 with fp32 weights 45.2 against 47.1 us being the largest gap.)
 #define RMS_ONCE_GO(BS, NV, R, E, TH)                                                                              \
     rms_norm_once<T, BS, NV, R, E, TH, ADD><<<static_cast<unsigned>(ceil_div(n, R)), BS, 0, stream>>>(              \
         py, px, w, w_kind, n, static_cast<uint32_t>(d), desc.stride_y, desc.stride_x, desc.epsilon, res)
