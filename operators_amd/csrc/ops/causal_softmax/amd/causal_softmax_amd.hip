@@ -769,7 +769,7 @@ __global__ __launch_bounds__(BS) void causal_softmax_long(uint16_t *y, uint64_t 
 // taking row r * m mod rows instead of row r, for fourteen odd m from 3 to
 // 12 289, ran [64, 512, 65536] in 1566 (m = 513) to 1800 us (m = 1025)
 // against 1664, and [64, 512, 32768] in 796-814 against 799.)
-template<typename T, int BS, int NV, bool THROUGH, bool TURN>
+template<typename T, int BS, int NV, bool THROUGH, bool TURN, bool RAGGED = false>
 __global__ __launch_bounds__(BS) __attribute__((amdgpu_waves_per_eu(4)))
 void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t total, int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
     AMD_ARGS_NOW(y, rows, seq, total, stride_b, stride_i, arg_pair(by_seq), gridDim.x);
@@ -777,20 +777,43 @@ void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
     constexpr float kL2e = 1.44269502162933349609375f;
     __shared__ float red[4 * WAVES];
     const float neg_inf = -__builtin_inff();
-    const uint32_t nvec = total / 8;
+    static_assert(!RAGGED || TURN, "rows at any 2-byte boundary are turned to line boundaries as well");
     int phase = 0;
     for (uint64_t r = blockIdx.x; r < rows; r += gridDim.x, phase ^= 1) {
         const uint32_t b = fast_quotient(static_cast<uint32_t>(r), by_seq), i = static_cast<uint32_t>(r) - b * seq;// fewer than 2^31 rows (see FastDiv)
         uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
-        const uint32_t keep = total - seq + i + 1;
-        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = (keep - 1) / 8;
+        // RAGGED: rows at any 2-byte boundary and of any length.  The vectors are the whole 16-byte aligned ones
+        // inside the row (its body); the up to 7 elements in front of them and the up to 7 behind are taken one each
+        // by the first 16 lanes of the workgroup, with 2-byte accesses, and enter the maximum, the sum and the
+        // quotients beside those lanes' vectors ([39, 512, 40001] fp16 614 us in two passes -> 5xx us).
+        const uint32_t row_keep = total - seq + i + 1;
+        uint32_t head = 0, nvec = total / 8, keep = row_keep;
+        uint16_t *body = row;
+        if constexpr (RAGGED) {
+            head = (8u - static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 15u) / 2) & 7u;
+            body = row + head;
+            nvec = (total - head) / 8;
+            const uint32_t past_head = row_keep > head ? row_keep - head : 0u;
+            keep = past_head < nvec * 8 ? past_head : nvec * 8;
+        }
+        const uint32_t keep_vecs = (keep + 7) / 8, tail = keep & 7u, last_vec = RAGGED && keep == 0 ? 0u : (keep - 1) / 8;
+        [[maybe_unused]] uint32_t end_col = 0;// this lane's column of the row, if end_mine
+        [[maybe_unused]] bool end_mine = false, end_kept = false;
+        [[maybe_unused]] float end_x = 0.0f, end_e = 0.0f;
+        if constexpr (RAGGED) {
+            const uint32_t t = threadIdx.x;
+            end_col = t < 8 ? t : head + nvec * 8 + (t - 8);
+            end_mine = t < 8 ? t < head : (t < 16 && end_col < total);
+            end_kept = end_mine && end_col < row_keep;
+            if (end_kept) end_x = T::one(row[end_col]);
+        }
         // TURN: rows that start inside a 128-byte line.  Lanes take the vectors turned by the row's distance from
         // the line's start, the first few lanes of the first turn the last vectors there is room for, so that a
         // wavefront's 1 KiB per instruction is whole lines ([34, 512, 45000] fp16 657 -> 526 us, [47, 512, 33000]
         // 674 -> 585).  A form of its own: on rows in whole lines it costs 1-1.5 %, and the 20-vector form has no
         // register left for it.
         static_assert(!TURN || NV < 20, "no register left for the turn");
-        [[maybe_unused]] const uint32_t turn = TURN ? static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row) & 127u) / 16 : 0u;
+        [[maybe_unused]] const uint32_t turn = TURN ? static_cast<uint32_t>(reinterpret_cast<uintptr_t>(body) & 127u) / 16 : 0u;
         auto vector_at = [&](int k) {
             if constexpr (TURN) {
                 const uint32_t s = static_cast<uint32_t>(k * BS + threadIdx.x) - turn;
@@ -803,7 +826,7 @@ void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = vector_at(k);
-            cur[k] = ld16_stream(row + static_cast<uint64_t>(v < last_vec ? v : last_vec) * 8);// masked vectors re-read the last kept one
+            cur[k] = ld16_stream(body + static_cast<uint64_t>(v < last_vec ? v : last_vec) * 8);// masked vectors re-read the last kept one
         }
         // the maximum; the one vector that straddles the mask enters element by element
         float mx = neg_inf;
@@ -836,6 +859,9 @@ void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
             }
         }
         if constexpr (T::kPackedMinMax) mx = fmaxf(mx, fmaxf(T::first(mx2), T::second(mx2)));
+        if constexpr (RAGGED) {
+            if (end_kept) mx = fmaxf(mx, end_x);
+        }
         mx = block_max<WAVES>(mx, red, phase);
         // exp(x - max) as exp2(x * log2(e) - max * log2(e)); a row whose maximum is +-inf goes the plain way (inf - inf must give NaN)
         const bool finite_max = __builtin_fabsf(mx) < __builtin_inff();
@@ -868,11 +894,15 @@ void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
             }
             part += ((e8[0] + e8[1]) + (e8[2] + e8[3])) + ((e8[4] + e8[5]) + (e8[6] + e8[7]));
         }
+        if constexpr (RAGGED) {
+            if (end_kept) end_e = __builtin_amdgcn_exp2f(finite_max ? __builtin_fmaf(end_x, kL2e, -m2) : (end_x - mx) * kL2e);
+            part += end_e;// 0 for the lanes without a kept end element
+        }
         const float sum = block_sum<WAVES>(part, red + 2 * WAVES, phase);
         const float rcp = 1.0f / sum;
 #pragma unroll
         for (int k = 0; k < NV; ++k) asm volatile("" : "+v"(cur[k]));
-        const StreamOut<THROUGH> out(row);
+        const StreamOut<THROUGH> out(body);
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = vector_at(k);
@@ -896,6 +926,9 @@ void causal_softmax_held(uint16_t *y, uint64_t rows, uint32_t seq, uint32_t tota
                 }
             }
             if (v < nvec) out.st16(v * 16, packed);
+        }
+        if constexpr (RAGGED) {
+            if (end_mine) row[end_col] = end_kept ? static_cast<uint16_t>(T::narrow2_fast(end_e * rcp, 0.0f) & 0xFFFFu) : uint16_t{0};
         }
     }
 }
@@ -974,18 +1007,21 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     if (long_ok) {
         const bool thr = rows * d.total * sizeof(uint16_t) >= kWriteThroughBytes;
         const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
-        if (aligned && nvec <= 16 * 1024) {// up to 131 072 elements: held in registers, read once (see causal_softmax_held)
-            // rows off the 128-byte boundaries skip the 20-vector form, which has no turned variant
+        if (nvec <= 16 * 1024) {// up to 131 072 elements: held in registers, read once (see causal_softmax_held)
+            // rows off the 128-byte boundaries skip the 20-vector form, which has no turned variant; rows off the
+            // 16-byte boundaries, or whose length is no multiple of 8, take the ragged one (its body is never longer)
             const uint64_t most_512 = in_lines ? 20 * 512 : 16 * 512;
             const unsigned lanes = nvec <= most_512 ? 512 : 1024;
             const unsigned g = static_cast<unsigned>(std::min<uint64_t>(rows, amd::max_grid_1d(lanes)));
-#define CS_HELD_GO(BS, NV, TH, TURN) causal_softmax_held<T, BS, NV, TH, TURN><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)
-#define CS_HELD(BS, NV)                                                 \
-    do {                                                                \
-        if (thr && (in_lines || NV >= 20)) CS_HELD_GO(BS, NV, true, false); \
-        else if (thr) CS_HELD_GO(BS, NV, true, (NV < 20));              \
-        else if (in_lines || NV >= 20) CS_HELD_GO(BS, NV, false, false); \
-        else CS_HELD_GO(BS, NV, false, (NV < 20));                      \
+#define CS_HELD_GO(BS, NV, TH, TURN, RG) causal_softmax_held<T, BS, NV, TH, TURN, RG><<<g, BS, 0, stream>>>(py, rows, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by)
+#define CS_HELD(BS, NV)                                                              \
+    do {                                                                             \
+        if (thr && (in_lines || NV >= 20)) CS_HELD_GO(BS, NV, true, false, false);  \
+        else if (thr && aligned) CS_HELD_GO(BS, NV, true, (NV < 20), false);         \
+        else if (thr) CS_HELD_GO(BS, NV, true, (NV < 20), (NV < 20));                \
+        else if (in_lines || NV >= 20) CS_HELD_GO(BS, NV, false, false, false);      \
+        else if (aligned) CS_HELD_GO(BS, NV, false, (NV < 20), false);               \
+        else CS_HELD_GO(BS, NV, false, (NV < 20), (NV < 20));                        \
     } while (0)
             if (nvec <= 12 * 512) CS_HELD(512, 12);
             else if (nvec <= 16 * 512) CS_HELD(512, 16);

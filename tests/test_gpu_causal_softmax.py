@@ -93,7 +93,10 @@ def test_against_oracle(ctx, dt, case):
                                                (2, (2, 4, 33333), 33339), (0, (3, 21, 77), 77), (6, (40, 3, 5), 5), (4, (2, 6, 520), 523),
                                                # up to 56 elements behind a workgroup's vectors are taken one by one, also for rows in whole lines
                                                (0, (2, 10, 4152), 4160), (0, (3, 12, 2104), 2112), (3, (2, 12, 2105), 2111), (0, (2, 7, 32800), 32832),
-                                               (5, (2, 9, 32830), 32831), (1, (3, 10, 16), 16), (0, (3, 10, 15), 15), (3, (2, 16, 17), 19), (0, (2, 70, 568), 576)])
+                                               (5, (2, 9, 32830), 32831), (1, (3, 10, 16), 16), (0, (3, 10, 15), 15), (3, (2, 16, 17), 19), (0, (2, 70, 568), 576),
+                                               # long rows at any boundary, held in registers: body vectors turned to line boundaries, ends one by one
+                                               (3, (1, 3, 65537), 65541), (1, (1, 2, 100001), 100003), (7, (1, 3, 131073), 131075), (0, (1, 5, 40001), 40001),
+                                               (4, (1, 3, 81913), 81920)])
 def test_ragged_rows_leave_their_neighbours_alone(ctx, dt, start, shape, pitch):
     """Rows that start anywhere and end anywhere, inside a buffer of other data:
     `start` elements in front of the first row, `pitch - total` between rows.
@@ -200,7 +203,7 @@ def test_long_row_forms_against_the_float64_quotient(ctx, dt):
     hits it exactly about as often as the register form does on a row of 32 768."""
     rng = np.random.default_rng(41)
     rates = {}
-    for total in (32768, 40000, 65536, 100000, 131072, 200000):
+    for total in (32768, 40000, 40001, 65536, 65537, 100000, 131072, 200000):
         shape = (1, 4, total)
         y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 3, dt)
         got, _, _ = run(ctx, y, shape, None, dt)
