@@ -342,7 +342,8 @@ template<typename T, int P, int NV, bool THROUGH, bool RAGGED, bool ON16 = false
 __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint64_t groups, uint32_t seq, uint32_t total,
                                                               int64_t stride_b, int64_t stride_i, FastDiv by_groups_per_matrix,
                                                               uint32_t groups_per_matrix) {
-    static_assert(NV >= 1 && NV <= 3 && P * NV <= kWave, "up to three vector indices, added as the whole-wavefront tree adds them");
+    static_assert((NV >= 1 && NV <= 3 && P * NV <= kWave) || (P == 32 && NV == 4),
+                  "up to three vector indices, added as the whole-wavefront tree adds them; or two rows of 65-128 vectors, added as a wavefront of its own adds a row's two vectors per lane");
     AMD_ARGS_NOW(y, groups, seq, total, stride_b, stride_i, arg_pair(by_groups_per_matrix), groups_per_matrix, gridDim.x);
     constexpr uint32_t RPW = kWave / P;// rows per wavefront
     const uint32_t sub = threadIdx.x % P, rr = threadIdx.x / P;
@@ -474,6 +475,9 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
             e_t = kept_t ? e_t : 0.0f;
         }
         float tree[NV];
+        // 32 x 4: a wavefront of its own (causal_softmax_rows, 64 lanes x 2 vectors) would give lane l the vectors l and
+        // l + 64 and add their elements in one running sum; here they are lane sub's vectors k and k + 2
+        [[maybe_unused]] float run[2] = {0.0f, 0.0f};
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const uint32_t v = sub + k * P;
@@ -499,20 +503,31 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
                     for (int e = 0; e < 8; ++e) f[k][e] = static_cast<uint32_t>(e) < tail ? f[k][e] : 0.0f;
                 }
             }
-            float part = 0.0f;
-            if (v < keep_vecs) {
+            if constexpr (NV == 4) {
+                if (v < keep_vecs) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) part += f[k][e];
+                    for (int e = 0; e < 8; ++e) run[k & 1] += f[k][e];
+                }
+                if constexpr (RAGGED) {
+                    if (k == 0) run[0] += e_t;
+                }
+            } else {
+                float part = 0.0f;
+                if (v < keep_vecs) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) part += f[k][e];
+                }
+                if constexpr (RAGGED) {
+                    if (k == 0) part += e_t;
+                }
+                tree[k] = segment_sum<P>(part);
             }
-            if constexpr (RAGGED) {
-                if (k == 0) part += e_t;
-            }
-            tree[k] = segment_sum<P>(part);
         }
         // the order in which the whole-wavefront tree adds these groups of lanes: upper to lower, pairwise
         float sum = tree[0];
         if constexpr (NV == 2) sum = tree[1] + tree[0];
         if constexpr (NV == 3) sum = tree[2] + (tree[1] + tree[0]);
+        if constexpr (NV == 4) sum = segment_sum<P>(run[1]) + segment_sum<P>(run[0]);
         const float rcp = 1.0f / sum;
 
         const StreamOut<THROUGH> out(RAGGED ? y : base);// RAGGED: not used, every lane has a base of its own
@@ -1071,7 +1086,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
     //   [32768, 128, 128]  1385 -> 291 us                    [131072, 64, 64]  2765 -> 324 us
     // with 2048 wavefronts per compute unit striding over the groups (128 / 512 / 8192 per unit: 382 / 348 / 351 us
     // at 256 columns with 32 lanes per row).
-    if ((aligned || d.total >= 16) && nvec <= 64 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
+    if ((aligned || d.total >= 16) && nvec <= 96 && rows < kFastDivLimit && d.stride_i >= 0 && static_cast<uint64_t>(d.stride_i) * 16 + d.total * 2 < (1ull << 31)) {
         // Lanes per row x vectors per lane: the pair that wastes the fewest lanes, the fewer lanes per row (more
         // rows per wavefront) when two waste the same, among those whose rows per wavefront divide the matrix's
         // row count.  More than one vector per lane spares the rows that the mask cuts short the work of the
@@ -1085,8 +1100,13 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         unsigned lanes = 0, per_lane = 0;
         const auto pick = [&]() {
             for (const unsigned p : {8u, 16u, 32u}) {
-                for (const unsigned v : {1u, 2u, 3u}) {
-                    const bool fits = p * v >= nvec && p * v <= kWave && (!together || d.seq % (kWave / p) == 0);// ragged rows: any consecutive rows
+                for (const unsigned v : {1u, 2u, 3u, 4u}) {
+                    // (32 x 4: rows of 513-768 elements two to a wavefront.  Against a wavefront each - causal_softmax_rows,
+                    // 64 x 2 - fp16, us: [2978, 520, 520] 569 / 638, [2427, 576, 576] 442 / 552, [1966, 640, 640] 426 / 515,
+                    // [1365, 768, 768] 404 / 449; beyond, the wavefront each is level or ahead: [1333, 777, 777] 555 / 544,
+                    // [1003, 896, 896] 417 / 416, [805, 1000, 1000] 461 / 457, [768, 1024, 1024] 389 / 376.)
+                    const bool room = v == 4 ? p == 32 : p * v <= kWave;
+                    const bool fits = p * v >= nvec && room && (!together || d.seq % (kWave / p) == 0);// ragged rows: any consecutive rows
                     if (fits && (lanes == 0 || p * v < lanes * per_lane)) lanes = p, per_lane = v;
                 }
             }
@@ -1122,6 +1142,7 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
                 case 162: CS_SHORT(16, 2); break;
                 case 163: CS_SHORT(16, 3); break;
                 case 321: CS_SHORT(32, 1); break;
+                case 324: CS_SHORT(32, 4); break;
                 default: CS_SHORT(32, 2); break;
             }
 #undef CS_SHORT

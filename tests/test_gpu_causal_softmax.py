@@ -302,13 +302,13 @@ def test_infinities_and_long_tails_in_long_rows(ctx):
 
 
 def test_short_rows_give_the_bits_of_a_wavefront_per_row(ctx):
-    """Rows of up to 512 elements share a wavefront (8, 16 or 32 lanes each) when
+    """Rows of up to 1024 elements share a wavefront (8, 16 or 32 lanes each) when
     the rows of a group lie within 2 GiB of each other; rows 256 MiB apart get a
     wavefront each.  Both forms add in the same order: same data, same bits."""
     import torch
 
     for dt, tdt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
-        for total in (64, 72, 128, 136, 192, 200, 256, 264, 320, 384, 512):
+        for total in (64, 72, 128, 136, 192, 200, 256, 264, 320, 384, 512, 520, 576, 640, 768, 896, 1000, 1024):
             seq = 8
             rng = np.random.default_rng(900 + total)
             vals = rng.standard_normal((1, seq, total)).astype(np.float32) * 3
