@@ -465,6 +465,8 @@ def ops_table(ctx, args, gen):
         "N1e causal_softmax f16 [64,512,20480] (a chunk of 512 queries against 20480 keys: 512 lanes x 5 vectors)": lambda: [make_causal_softmax(ctx, 64, 512, 20480, f16, gen, "causal_softmax") for _ in range(2)],
         "N1f causal_softmax f16 [64,512,65536] (rows of 128 KiB held in registers as raw words, read once; the row stride is a power of two)": lambda: [make_causal_softmax(ctx, 64, 512, 65536, f16, gen, "causal_softmax") for _ in range(2)],
         "N1g causal_softmax f16 [64,512,40000] (the same form, 12 vectors per lane, a row stride that is no power of two)": lambda: [make_causal_softmax(ctx, 64, 512, 40000, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1h causal_softmax f16 [21,5000,5000] (a prompt of 5000 tokens: ragged rows, 128 lanes x 5 vectors)": lambda: [make_causal_softmax(ctx, 21, 5000, 5000, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1i causal_softmax f16 [39,512,40001] (long rows at odd 2-byte boundaries, held in registers, ends one element per lane)": lambda: [make_causal_softmax(ctx, 39, 512, 40001, f16, gen, "causal_softmax") for _ in range(2)],
         "Q2 rms_norm bf16 [4096,32768] w f32 (one 1024-lane workgroup per compute unit, 128 KiB of weights in LDS)": lambda: [make_rms_norm(ctx, 4096, 32768, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * 4096 * 32768, nset))],
         "F2 add_rms_norm bf16 [8192,16384] w f32 (fused Add + RMSNorm, wide rows)": lambda: [make_add_rms_norm(ctx, 8192, 16384, bf16, torch.float32, gen, "add_rms_norm") for _ in range(sets_needed(6 * 8192 * 16384, nset))],
     }
@@ -782,7 +784,7 @@ FLAT_ROWS = {
     "c4": "C4 add f16 [8192,4096]", "c4_bcast": "C4 add f16 [8192,4096] + b", "c5_rms_norm": "C5 rms_norm", "c5_rope_q": "C5 rope_q",
     "c5_rope_k": "C5 rope_k", "c5b_rope_qk": "C5b rope_qk", "c5_swiglu": "C5 swiglu", "c5_add": "C5 add",
     "f1_add_rms_norm": "F1 add_rms_norm", "f2_add_rms_norm": "F2 add_rms_norm", "q1_rms_norm": "Q1 rms_norm", "q2_rms_norm": "Q2 rms_norm",
-    "n1_causal_softmax": "N1 causal_softmax", "n1c": "N1c", "n1d": "N1d", "n1e": "N1e", "n1f": "N1f", "n1g": "N1g",
+    "n1_causal_softmax": "N1 causal_softmax", "n1c": "N1c", "n1d": "N1d", "n1e": "N1e", "n1f": "N1f", "n1g": "N1g", "n1h": "N1h", "n1i": "N1i",
     "n2_rearrange": "N2 rearrange", "n2b_rearrange": "N2b rearrange",
 }
 
