@@ -1097,6 +1097,13 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipS
         bool together = in_lines;// rows in whole lines: RPW rows of one matrix per wavefront; others: the ragged form, which measures
                                        // better for them also where they lie on 16-byte boundaries ([2048, 504, 504] fp16 345 against 411 us,
                                        // [8192, 120, 120] 89 against 164 us; in whole lines it is the other way round: [2048, 512, 512] 335 against 277 us)
+        // (Contiguous rows at odd boundaries through LDS instead - a wavefront loads a run of 8 to 16 rows as the
+        // aligned 16-byte vectors that it is, cuts the rows out of LDS with 16-byte LDS accesses and writes the run
+        // back in whole vectors - measured level at best, fp16, us, rows addressed in memory / through LDS in chunks
+        // of 8 / of 16 rows: [4096, 250, 250] 181 / 196 / 175, [2048, 333, 333] 160 / 192 / 201, [2048, 500, 500]
+        // 342 / 326 / 521, [16384, 64, 250] 190 / 207 / 204; with the next run's loads issued before the work on
+        // this one, 200 and more.  The three phases of a run follow each other within a wavefront, and LDS bounds
+        // the wavefronts that can be in different phases.)
         unsigned lanes = 0, per_lane = 0;
         const auto pick = [&]() {
             for (const unsigned p : {8u, 16u, 32u}) {
