@@ -669,53 +669,65 @@ __global__ __launch_bounds__(BS) void rms_norm_once(uint16_t *y, const uint16_t 
 // consecutive rows; the sum of squares is the first steps of the wavefront
 // tree (amd::segment_sum), which adds the same values in the same order as
 // the full tree would with zeros in the absent lanes - so these rows, too,
-// give the bits every other form gives.
-template<typename T, int P, bool THROUGH, bool ADD>
+// give the bits every other form gives.  A turn of the wavefront takes U such
+// groups of rows, with the loads of all of them in flight together.
+template<typename T, int P, int U, bool THROUGH, bool ADD>
 __global__ __launch_bounds__(kWave) void rms_norm_short(uint16_t *y, const uint16_t *x, const void *w, int w_kind,
                                                         uint64_t n, uint32_t d, int64_t stride_y, int64_t stride_x, float eps,
                                                         Residual<ADD> res) {
     RMS_ARGS_NOW(gridDim.x);
-    constexpr uint32_t RPW = kWave / P;// rows per wavefront
+    constexpr uint32_t RPW = kWave / P;// rows per wavefront and group; U groups per turn
     const uint32_t nvec = d / 8;
     const uint32_t sub = threadIdx.x % P, rr = threadIdx.x / P;
     const uint32_t lv = sub < nvec ? sub : 0;
-    const uint64_t hop = static_cast<uint64_t>(gridDim.x) * RPW;
-    uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * RPW;
+    const uint64_t hop = static_cast<uint64_t>(gridDim.x) * RPW * U;
+    uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * RPW * U;
     if (row0 >= n) return;
-    // absent rows re-read the group's first one; nothing of them is stored
-    const auto row_of = [&](uint64_t first) { return first + rr < n ? first + rr : first; };
+    // absent rows re-read the turn's first one; nothing of them is stored
+    const auto row_of = [&](uint64_t first, int u) { return first + u * RPW + rr < n ? first + u * RPW + rr : first; };
     // The first rows are asked for in front of the weights: 16-bit weights are widened as soon as they arrive,
     // and with the weights asked for first that wait stood in front of the rows' request - two memory latencies
     // in a row for a wavefront that serves one group of rows ([524288, 128] bf16 with bf16 weights 47.2 us, with
     // fp32 weights, which need no widening, 42.0).
-    u32x4 xv = ld16_stream(x + static_cast<int64_t>(row_of(row0)) * stride_x + static_cast<uint64_t>(lv) * 8);
-    [[maybe_unused]] u32x4 bv{};
-    if constexpr (ADD) bv = ld16_stream(res.b + static_cast<int64_t>(row_of(row0)) * res.stride_b + static_cast<uint64_t>(lv) * 8);
+    u32x4 xv[U];
+    [[maybe_unused]] u32x4 bv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        xv[u] = ld16_stream(x + static_cast<int64_t>(row_of(row0, u)) * stride_x + static_cast<uint64_t>(lv) * 8);
+        if constexpr (ADD) bv[u] = ld16_stream(res.b + static_cast<int64_t>(row_of(row0, u)) * res.stride_b + static_cast<uint64_t>(lv) * 8);
+    }
     float g[8];
     load_w8(w, w_kind, lv, g);
     while (true) {
-        const bool have = row0 + rr < n && sub < nvec;
-        if constexpr (ADD) {// the row becomes a + b, rounded as Add rounds, and goes out to c
-            float p[8], q[8];
-            widen8<T>(xv, p);
-            widen8<T>(bv, q);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) p[i] += q[i];
-            xv = narrow8<T>(p);
-            const StreamOut<THROUGH> cr(res.c + static_cast<int64_t>(row0) * res.stride_c);
-            if (have) cr.st16(rr * static_cast<uint32_t>(res.stride_c) * 2 + sub * 16, xv);
+        for (int u = 0; u < U; ++u) {
+            const uint64_t first = row0 + u * RPW;
+            const bool have = first + rr < n && sub < nvec;
+            if constexpr (ADD) {// the row becomes a + b, rounded as Add rounds, and goes out to c
+                float p[8], q[8];
+                widen8<T>(xv[u], p);
+                widen8<T>(bv[u], q);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) p[i] += q[i];
+                xv[u] = narrow8<T>(p);
+                const StreamOut<THROUGH> cr(res.c + static_cast<int64_t>(first) * res.stride_c);
+                if (have) cr.st16(rr * static_cast<uint32_t>(res.stride_c) * 2 + sub * 16, xv[u]);
+            }
+            float f[8];
+            widen8<T>(xv[u], f);
+            const float k_row = inv_rms(segment_sum<P>(sub < nvec ? squares8(f) : 0.0f), d, eps);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
+            const StreamOut<THROUGH> yr(y + static_cast<int64_t>(first) * stride_y);
+            if (have) yr.st16(rr * static_cast<uint32_t>(stride_y) * 2 + sub * 16, narrow8<T>(f));
         }
-        float f[8];
-        widen8<T>(xv, f);
-        const float k_row = inv_rms(segment_sum<P>(sub < nvec ? squares8(f) : 0.0f), d, eps);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = (k_row * f[i]) * g[i];
-        const StreamOut<THROUGH> yr(y + static_cast<int64_t>(row0) * stride_y);
-        if (have) yr.st16(rr * static_cast<uint32_t>(stride_y) * 2 + sub * 16, narrow8<T>(f));
         row0 += hop;
         if (row0 >= n) break;
-        xv = ld16_stream(x + static_cast<int64_t>(row_of(row0)) * stride_x + static_cast<uint64_t>(lv) * 8);
-        if constexpr (ADD) bv = ld16_stream(res.b + static_cast<int64_t>(row_of(row0)) * res.stride_b + static_cast<uint64_t>(lv) * 8);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            xv[u] = ld16_stream(x + static_cast<int64_t>(row_of(row0, u)) * stride_x + static_cast<uint64_t>(lv) * 8);
+            if constexpr (ADD) bv[u] = ld16_stream(res.b + static_cast<int64_t>(row_of(row0, u)) * res.stride_b + static_cast<uint64_t>(lv) * 8);
+        }
     }
 }
 
@@ -911,20 +923,35 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     if constexpr (ADD) near = near && res.stride_c >= 0 && res.stride_c < (1 << 26);
     if (nvec <= 32 && near) {
         const unsigned lanes = nvec <= 8 ? 8 : (nvec <= 16 ? 16 : 32);
-        const uint64_t want = ceil_div(n, kWave / lanes), cap = amd::max_grid_1d(kWave);
+        // A wavefront has one 16-byte load per lane in flight, and the compute unit's wavefronts together must cover
+        // the memory latency: rows that leave a quarter or more of their lanes idle (72, 80, 96, 160, 192 elements)
+        // take two groups of rows per turn.  Measured, [64 Mi / d, d] bf16 with fp32 weights, us, one / two / four
+        // groups: d = 72: 58.9 / 49.3 / 48.4, 80: 53.9 / 46.7 / 47.3, 96: 46.2 / 45.3 / 46.9, 160: 53.7 / 47.2 / 47.1,
+        // 192: 46.9 / 45.1 / 47.4; rows that fill their lanes lose by it (112: 42.7 / 45.2, 128: 41.9 / 43.6,
+        // 256: 41.4 / 43.4), and so does the fused form, which has two loads per lane in flight as it is
+        // (80: 66.2 / 68.8, 160: 65.7 / 68.1).
+        const unsigned turns = !ADD && nvec * 4 <= lanes * 3 ? 2 : 1;
+        const uint64_t want = ceil_div(n, kWave / lanes * turns), cap = amd::max_grid_1d(kWave);
         const unsigned grid = static_cast<unsigned>(want < cap ? want : cap);
+#define RMS_SHORT_GO(P, U, TH)                                                                                      \
+    rms_norm_short<T, P, U, TH, ADD><<<grid, kWave, 0, stream>>>(py, px, w, w_kind, n, static_cast<uint32_t>(d),    \
+                                                                 desc.stride_y, desc.stride_x, desc.epsilon, res)
 #define RMS_SHORT(P)                                                                                                   \
     do {                                                                                                               \
-        if (through)                                                                                                   \
-            rms_norm_short<T, P, true, ADD><<<grid, kWave, 0, stream>>>(py, px, w, w_kind, n, static_cast<uint32_t>(d), \
-                                                                        desc.stride_y, desc.stride_x, desc.epsilon, res); \
-        else                                                                                                           \
-            rms_norm_short<T, P, false, ADD><<<grid, kWave, 0, stream>>>(py, px, w, w_kind, n, static_cast<uint32_t>(d), \
-                                                                         desc.stride_y, desc.stride_x, desc.epsilon, res); \
+        if constexpr (!ADD) {                                                                                          \
+            if (turns == 2) {                                                                                          \
+                if (through) RMS_SHORT_GO(P, 2, true);                                                                 \
+                else RMS_SHORT_GO(P, 2, false);                                                                        \
+                break;                                                                                                 \
+            }                                                                                                          \
+        }                                                                                                              \
+        if (through) RMS_SHORT_GO(P, 1, true);                                                                         \
+        else RMS_SHORT_GO(P, 1, false);                                                                                \
     } while (0)
         if (lanes == 8) RMS_SHORT(8);
         else if (lanes == 16) RMS_SHORT(16);
         else RMS_SHORT(32);
+#undef RMS_SHORT_GO
 #undef RMS_SHORT
         return;
     }
@@ -932,6 +959,16 @@ void launch_rms_norm(const RowsShape &desc, void *y, const void *x, const void *
     // hold the looping kernels below take over.
     const auto once_fits = [&](unsigned lanes, unsigned rows) { return ceil_div(n, rows) <= amd::max_grid_1d(lanes); };
     if (nvec <= 64 && once_fits(64, 1)) {
+        // (rows of 264-384 elements leave a quarter and more of the wavefront idle: two rows per wavefront, as above;
+        // [64 Mi / d, d] bf16, us, one / two rows: d = 320: 51.7 / 43.4, 384: 45.1 / 43.4, 448: 41.7 / 44.0, 512: 41.1 / 44.3)
+        bool two = false;
+        if constexpr (!ADD) two = nvec <= 48 && once_fits(64, 2);
+        if constexpr (!ADD) {
+            if (two) {
+                RMS_ONCE(64, 1, 2);
+                return;
+            }
+        }
         RMS_ONCE(64, 1, 1);
         return;
     }

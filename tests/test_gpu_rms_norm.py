@@ -59,7 +59,10 @@ def test_golden_odd_sizes(ctx):
                                  (270, 33000), (264, 36864), (300, 49152), (260, 57344), (258, 65536), (40, 49152),
                                  # short rows, several to a wavefront (per-head norms): full and ragged last wavefronts, rows that
                                  # do not fill their lanes, an output large enough to be written through L2
-                                 (5001, 128), (4096, 128), (1003, 64), (777, 256), (333, 72), (101, 16), (50, 200), (270000, 128)])
+                                 (5001, 128), (4096, 128), (1003, 64), (777, 256), (333, 72), (101, 16), (50, 200), (270000, 128),
+                                 # rows that leave a quarter and more of their lanes idle: two groups of rows per turn of a wavefront
+                                 # (one, odd and large row counts; 320 and 384: two rows per one-wavefront workgroup)
+                                 (1001, 80), (7, 96), (1, 160), (5, 192), (9, 24), (430000, 80), (1003, 320), (3, 384), (1, 320)])
 def test_against_oracle(ctx, dt, wdt, n, d):
     rng = np.random.default_rng(n * 7 + d)
     x = oracle.encode(rng.standard_normal((n, d)).astype(np.float32), dt)
@@ -84,6 +87,11 @@ def test_row_strides_of_x_and_y_are_independent(ctx):
     w = oracle.encode(rng.uniform(0.5, 1.5, 128).astype(np.float32), "f32")
     want = oracle.rms_norm(x, w, 1e-6, "bf16", "f32")
     check(run(ctx, x, w, 1e-6, "bf16", "f32", x_stride=640, y_stride=256), want, "bf16", "strided short rows")
+    # and with two groups of rows per turn: heads of 80 out of every 400 elements, written 88 apart
+    x = oracle.encode(rng.standard_normal((1003, 80)).astype(np.float32), "f16")
+    w = oracle.encode(rng.uniform(0.5, 1.5, 80).astype(np.float32), "f16")
+    want = oracle.rms_norm(x, w, 1e-6, "f16", "f16")
+    check(run(ctx, x, w, 1e-6, "f16", "f16", x_stride=400, y_stride=88), want, "f16", "strided short rows, two groups per turn")
 
 
 def test_in_place(ctx):
