@@ -376,7 +376,10 @@ __global__ __launch_bounds__(kWave) void causal_softmax_short(uint16_t *y, uint6
         // hardware exp2, and the quotient to one multiply - a third of the vector instructions gone, at the price of
         // three times as many outputs one unit off the float64 quotient - [8192, 256, 256] took 276 against 274 us,
         // [4096, 250, 250] 190 against 190, [2048, 333, 333] 157 against 157; only [16384, 64, 256] (160 against 170)
-        // and [65536, 64, 64] (168 against 178) moved.
+        // and [65536, 64, 64] (168 against 178) moved.  Nor the memory latency: with the loads of a wavefront's next
+        // group in flight during the work on this one (12 more registers, 6 wavefronts per SIMD in place of 7)
+        // [8192, 256, 256] took 282 against 274 us, [4096, 250, 250] 184 against 189, [2048, 504, 504] 325 against 301,
+        // [16384, 64, 250] 203 against 187.
         const uint32_t row_off = RAGGED ? 0u : rr * static_cast<uint32_t>(stride_i) * 2;// bytes from base to this lane's row
         struct Mine {
             uint16_t *row;       // the row's first element
