@@ -178,7 +178,8 @@ def make_causal_softmax(ctx, heads, seq, total, dtype, gen, name):
     plan = CausalSoftmaxPlan(ctx, y)
     kept = seq * (total - seq) + seq * (seq + 1) // 2  # elements read per matrix; every element is written
     nbytes = heads * (kept + seq * total) * y.element_size()
-    return Launch(name, ctx.lib.infiniopCausalSoftmax, (plan.desc, None, 0, y.data_ptr()), nbytes, (plan, y))
+    ws = plan.workspace.data_ptr() if plan.workspace is not None else None  # few very long rows only; 0 bytes otherwise
+    return Launch(name, ctx.lib.infiniopCausalSoftmax, (plan.desc, ws, plan.workspace_size, y.data_ptr()), nbytes, (plan, y))
 
 
 def make_random_sample(ctx, voc, topk, gen, name, use_workspace=True, topp=0.9, temperature=0.8):
@@ -467,6 +468,7 @@ def ops_table(ctx, args, gen):
         "N1g causal_softmax f16 [64,512,40000] (the same form, 12 vectors per lane, a row stride that is no power of two)": lambda: [make_causal_softmax(ctx, 64, 512, 40000, f16, gen, "causal_softmax") for _ in range(2)],
         "N1h causal_softmax f16 [21,5000,5000] (a prompt of 5000 tokens: ragged rows, 128 lanes x 5 vectors)": lambda: [make_causal_softmax(ctx, 21, 5000, 5000, f16, gen, "causal_softmax") for _ in range(2)],
         "N1i causal_softmax f16 [39,512,40001] (long rows at odd 2-byte boundaries, held in registers, ends one element per lane)": lambda: [make_causal_softmax(ctx, 39, 512, 40001, f16, gen, "causal_softmax") for _ in range(2)],
+        "N1j causal_softmax bf16 [32,1,131072] (decoding over 131072 keys, 32 heads: every row split over 8 workgroups, two launches, through the workspace)": lambda: [make_causal_softmax(ctx, 32, 1, 131072, bf16, gen, "causal_softmax") for _ in range(sets_needed(4 * 32 * 131072, nset))],
         "Q2 rms_norm bf16 [4096,32768] w f32 (one 1024-lane workgroup per compute unit, 128 KiB of weights in LDS)": lambda: [make_rms_norm(ctx, 4096, 32768, bf16, torch.float32, gen, "rms_norm") for _ in range(sets_needed(4 * 4096 * 32768, nset))],
         "F2 add_rms_norm bf16 [8192,16384] w f32 (fused Add + RMSNorm, wide rows)": lambda: [make_add_rms_norm(ctx, 8192, 16384, bf16, torch.float32, gen, "add_rms_norm") for _ in range(sets_needed(6 * 8192 * 16384, nset))],
     }

@@ -237,7 +237,10 @@ typedef CausalSoftmaxDescriptor *infiniopCausalSoftmaxDescriptor_t;
 /* replaces include/ops/causal_softmax/causal_softmax.h:13-15 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateCausalSoftmaxDescriptor(
     infiniopHandle_t handle, infiniopCausalSoftmaxDescriptor_t *desc_ptr, infiniopTensorDescriptor_t y_desc);
-/* replaces include/ops/causal_softmax/causal_softmax.h:17 - always 0 bytes */
+/* replaces include/ops/causal_softmax/causal_softmax.h:17 - 0 bytes, except for very few very long rows
+ * (decoding over 131 072 keys and more with up to a few dozen heads): 16 bytes per 16 384 columns of every
+ * row, through which the workgroups that share a row exchange its maximum and sum.  A call that comes
+ * without that workspace is served all the same, a workgroup per row. */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetCausalSoftmaxWorkspaceSize(infiniopCausalSoftmaxDescriptor_t desc, uint64_t *size);
 /* replaces include/ops/causal_softmax/causal_softmax.h:19-23 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCausalSoftmax(

@@ -26,8 +26,14 @@ struct AttentionPlan {
     uint64_t q_bytes;     // 0 when q is used where it lies
     uint64_t scores_bytes;// [n_q_head, seq, total]
     uint64_t result_bytes;// [n_q_head, seq, head_dim]
+    uint64_t softmax_bytes;// what CausalSoftmax asks for (few long rows: decoding over a long context), behind the rest on a 16-byte boundary
     uint64_t k_offset_bytes, v_offset_bytes;// position `pos` in the caches
 };
+
+uint64_t softmax_offset(const AttentionPlan &p) { return (p.q_bytes + p.scores_bytes + p.result_bytes + 15) / 16 * 16; }
+uint64_t workspace_bytes(const AttentionPlan &p) {
+    return p.softmax_bytes != 0 ? softmax_offset(p) + p.softmax_bytes : p.q_bytes + p.scores_bytes + p.result_bytes;
+}
 
 void destroy_all(AttentionPlan *p) {
     if (p->store_k) infiniopDestroyRearrangeDescriptor(p->store_k);
@@ -107,7 +113,7 @@ INFINIOP_C infiniopStatus_t infiniopCreateAttentionDescriptor(infiniopHandle_t h
     const DataLayout dt = q_desc->dt;
     const uint64_t es = dt.size;
 
-    auto *p = new (std::nothrow) AttentionPlan{handle->device, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
+    auto *p = new (std::nothrow) AttentionPlan{handle->device, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, 0};
     if (p == nullptr) {
         return STATUS_MEMORY_NOT_ALLOCATED;
     }
@@ -139,6 +145,7 @@ INFINIOP_C infiniopStatus_t infiniopCreateAttentionDescriptor(infiniopHandle_t h
     // causal softmax in place on scores seen as [heads, seq, total]
     infiniopTensorDescriptor_t scores_by_head = d.dense(dt, heads, seq, total);
     if (ok()) st = infiniopCreateCausalSoftmaxDescriptor(handle, &p->softmax, scores_by_head);
+    if (ok()) st = infiniopGetCausalSoftmaxWorkspaceSize(p->softmax, &p->softmax_bytes);
 
     // result[kv, group*seq, hd] = scores[kv, group*seq, total] @ V[kv, total, hd]
     infiniopTensorDescriptor_t v_full = d.make(v_cache_desc->dt, kv_heads, total, hd, v_cache_desc->strides[0], v_cache_desc->strides[1], 1);
@@ -165,7 +172,7 @@ INFINIOP_C infiniopStatus_t infiniopGetAttentionWorkspaceSize(infiniopAttentionD
         return STATUS_BAD_PARAM;
     }
     auto *p = reinterpret_cast<AttentionPlan *>(desc);
-    *size = p->q_bytes + p->scores_bytes + p->result_bytes;
+    *size = workspace_bytes(*p);
     return STATUS_SUCCESS;
 }
 
@@ -175,7 +182,7 @@ INFINIOP_C infiniopStatus_t infiniopAttention(infiniopAttentionDescriptor_t desc
         return STATUS_BAD_PARAM;
     }
     auto *p = reinterpret_cast<AttentionPlan *>(desc);
-    const uint64_t need = p->q_bytes + p->scores_bytes + p->result_bytes;
+    const uint64_t need = workspace_bytes(*p);
     if (workspace_size < need || (workspace == nullptr && need > 0)) {
         return STATUS_MEMORY_NOT_ALLOCATED;// the reference's answer to a short workspace (attention/operator.cc:264-266)
     }
@@ -185,6 +192,7 @@ INFINIOP_C infiniopStatus_t infiniopAttention(infiniopAttentionDescriptor_t desc
     char *q_packed = static_cast<char *>(workspace);
     char *scores = q_packed + p->q_bytes;
     char *result = scores + p->scores_bytes;
+    char *softmax_parts = p->softmax_bytes != 0 ? static_cast<char *>(workspace) + softmax_offset(*p) : nullptr;
 
     infiniopStatus_t st = infiniopRearrange(p->store_k, static_cast<char *>(k_cache) + p->k_offset_bytes, k, stream);
     if (st == STATUS_SUCCESS) st = infiniopRearrange(p->store_v, static_cast<char *>(v_cache) + p->v_offset_bytes, v, stream);
@@ -193,7 +201,7 @@ INFINIOP_C infiniopStatus_t infiniopAttention(infiniopAttentionDescriptor_t desc
         q = q_packed;
     }
     if (st == STATUS_SUCCESS) st = infiniopMatmul(p->scores, nullptr, 0, scores, q, k_cache, stream);
-    if (st == STATUS_SUCCESS) st = infiniopCausalSoftmax(p->softmax, nullptr, 0, scores, stream);
+    if (st == STATUS_SUCCESS) st = infiniopCausalSoftmax(p->softmax, softmax_parts, p->softmax_bytes, scores, stream);
     if (st == STATUS_SUCCESS) st = infiniopMatmul(p->weighted, nullptr, 0, result, scores, v_cache, stream);
     if (st == STATUS_SUCCESS) st = infiniopRearrange(p->unpack_out, out, result, stream);
     return st;

@@ -39,11 +39,12 @@ infiniopStatus_t amdCreateCausalSoftmaxDescriptor(AmdHandle_t handle, CausalSoft
     return STATUS_SUCCESS;
 }
 
-infiniopStatus_t amdGetCausalSoftmaxWorkspaceSize(CausalSoftmaxAmdDescriptor_t, uint64_t *size) {
+// 0 for every shape but few long rows, whose parts exchange a maximum and a sum each (see causal_softmax_parts).
+infiniopStatus_t amdGetCausalSoftmaxWorkspaceSize(CausalSoftmaxAmdDescriptor_t desc, uint64_t *size) {
     if (size == nullptr) {
         return STATUS_BAD_PARAM;
     }
-    *size = 0;
+    *size = desc->batch * desc->seq * causal_softmax_parts(*desc) * sizeof(CausalSoftmaxPart);
     return STATUS_SUCCESS;
 }
 

@@ -19,6 +19,31 @@ struct CausalSoftmaxAmdDescriptor {
 };
 typedef CausalSoftmaxAmdDescriptor *CausalSoftmaxAmdDescriptor_t;
 
+// Very few very long rows - decoding over a context of 128 Ki keys and more has one query row per head - leave
+// most compute units idle at a workgroup per row.  Such a call splits every row into parts of
+// kCausalSoftmaxPartColumns columns, a workgroup each, in two launches that exchange the parts' maxima and sums
+// through the workspace (causal_softmax_split_stats, causal_softmax_split_apply).  That reads the rows twice and
+// costs a second launch, so it pays only where the rows are few: measured on MI355X, bf16, a workgroup per row /
+// split, us: [8, 1, 131072] 16.0 / 10.9, [32, 1, 131072] 18.0 / 12.9, [64, 1, 131072] 18.7 / 19.7,
+// [128, 1, 131072] 21.1 / 34.2, [16, 1, 262144] 45.3 / 12.9, [64, 1, 262144] 47.3 / 34.3, [128, 1, 262144]
+// 49.5 / 61.9; [64, 1, 65536] 12.2 / 12.9, [64, 1, 32768] 7.0 / 11.6.  Without the workspace the call is served a
+// workgroup per row, as every other shape is.
+struct CausalSoftmaxPart {
+    float max, min, sum, unused;// of the part's kept columns; the sum is of exp(x - max)
+};
+constexpr uint64_t kCausalSoftmaxPartColumns = 16384;
+// Parts per row when the descriptor's shape takes the split form, else 0.
+inline uint32_t causal_softmax_parts(const CausalSoftmaxAmdDescriptor &d) {
+    const uint64_t rows = d.batch * d.seq, units = static_cast<uint64_t>(d.cu_count);
+    if (rows == 0 || d.total < 8 * kCausalSoftmaxPartColumns || d.total >= (1ull << 31)) return 0;
+    if (d.total % 8 != 0 || d.stride_i % 8 != 0 || d.stride_b % 8 != 0) return 0;// rows of whole 16-byte vectors
+    const uint64_t parts = (d.total + kCausalSoftmaxPartColumns - 1) / kCausalSoftmaxPartColumns;
+    if (parts > 64) return 0;// a wavefront puts a row's parts together, one per lane
+    // up to a workgroup per compute unit; rows beyond 131 072 columns, which a workgroup on its own reads twice, up to a row per four units
+    const bool few = rows * parts <= units || (parts > 8 && rows * 4 <= units);
+    return few ? static_cast<uint32_t>(parts) : 0;
+}
+
 infiniopStatus_t amdCreateCausalSoftmaxDescriptor(AmdHandle_t handle, CausalSoftmaxAmdDescriptor_t *desc_ptr,
                                                   infiniopTensorDescriptor_t y_desc);
 infiniopStatus_t amdGetCausalSoftmaxWorkspaceSize(CausalSoftmaxAmdDescriptor_t desc, uint64_t *size);

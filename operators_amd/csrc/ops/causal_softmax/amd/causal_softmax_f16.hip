@@ -5,6 +5,6 @@
 
 using namespace causal_softmax_kernels;
 
-void causal_softmax_launch_f16(const CausalSoftmaxAmdDescriptor &desc, void *data, hipStream_t stream) {
-    launch_causal_softmax<amd::F16Ref>(desc, data, stream);
+void causal_softmax_launch_f16(const CausalSoftmaxAmdDescriptor &desc, void *data, CausalSoftmaxPart *parts, hipStream_t stream) {
+    launch_causal_softmax<amd::F16Ref>(desc, data, parts, stream);
 }

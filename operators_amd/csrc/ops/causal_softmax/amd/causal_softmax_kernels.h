@@ -982,9 +982,152 @@ __global__ __launch_bounds__(256) void causal_softmax_generic(uint16_t *y, uint6
     }
 }
 
+// ---- few long rows: a row split over several workgroups, two launches --------------
+// Decoding over a long context is one query row per head: 64 rows of 131 072 columns keep 64 of 256 compute
+// units busy at a workgroup per row.  Here workgroup (part, row) takes kCausalSoftmaxPartColumns columns of the
+// row - 512 lanes x 4 vectors, held in registers.  The first launch leaves each part's maximum, minimum and sum
+// of exp(x - maximum) over its kept columns in the workspace; the second reads the row's parts (the same few
+// values in every workgroup of the row, combined in the same order), rescales the sums to the row's maximum and
+// writes its own columns: exp(x - maximum) / sum, the exponentials and the quotient those of the other forms.
+// Rows start on 16-byte boundaries and are whole vectors long (the host sees to it).
+constexpr int kSplitLanes = 512, kSplitVecs = 4;
+static_assert(kSplitLanes * kSplitVecs * 8 == kCausalSoftmaxPartColumns, "a part is what one workgroup holds");
+
 template<typename T>
-void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, hipStream_t stream) {
+__global__ __launch_bounds__(kSplitLanes) void causal_softmax_split_stats(const uint16_t *y, CausalSoftmaxPart *parts, uint32_t seq, uint32_t total,
+                                                                           int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
+    AMD_ARGS_NOW(y, parts, seq, total, stride_b, stride_i, arg_pair(by_seq));
+    constexpr int BS = kSplitLanes, NV = kSplitVecs, WAVES = BS / kWave;
+    __shared__ float red[6 * WAVES];
+    const uint32_t part = blockIdx.x, r = blockIdx.y;
+    const uint32_t b = fast_quotient(r, by_seq), i = r - b * seq;
+    const uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
+    const uint32_t keep = total - seq + i + 1;
+    const uint32_t from = part * static_cast<uint32_t>(kCausalSoftmaxPartColumns);
+    CausalSoftmaxPart *mine = parts + static_cast<size_t>(r) * gridDim.x + part;
+    const float neg_inf = -__builtin_inff();
+    if (from >= keep) {// nothing of this part is kept (uniform over the workgroup)
+        if (threadIdx.x == 0) *mine = CausalSoftmaxPart{neg_inf, __builtin_inff(), 0.0f, 0.0f};
+        return;
+    }
+    const uint32_t upto = keep - from < kCausalSoftmaxPartColumns ? keep : from + static_cast<uint32_t>(kCausalSoftmaxPartColumns);
+    float f[NV][8];
+    float mx = neg_inf, mn = __builtin_inff();
+    u32x4 x[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const uint32_t c0 = from + (k * BS + threadIdx.x) * 8;
+        x[k] = ld16_stream(row + (c0 < upto ? c0 : from));
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const uint32_t c0 = from + (k * BS + threadIdx.x) * 8;
+        widen8<T>(x[k], f[k]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (c0 + e < upto) mx = fmaxf(mx, f[k][e]), mn = fminf(mn, f[k][e]);
+        }
+    }
+    mx = block_max<WAVES>(mx, red, 0);
+    mn = -block_max<WAVES>(-mn, red + 2 * WAVES, 0);
+    const bool lean = mn - mx >= kLeanExpLimit;// uniform; false for infinities and for a part without a finite element
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const uint32_t c0 = from + (k * BS + threadIdx.x) * 8;
+        if (c0 >= upto) continue;
+        if (lean) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[k][e] = exp_nonpositive(f[k][e] - mx);
+        } else {
+            float slow[8];// an array of its own for the call: f stays in registers
+#pragma unroll
+            for (int e = 0; e < 8; ++e) slow[e] = f[k][e];
+            exp_any8(slow, mx);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[k][e] = slow[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += c0 + e < upto ? f[k][e] : 0.0f;
+    }
+    sum = block_sum<WAVES>(sum, red + 4 * WAVES, 0);
+    if (threadIdx.x == 0) *mine = CausalSoftmaxPart{mx, mn, sum, 0.0f};
+}
+
+template<typename T>
+__global__ __launch_bounds__(kSplitLanes) void causal_softmax_split_apply(uint16_t *y, const CausalSoftmaxPart *parts, uint32_t seq, uint32_t total,
+                                                                           int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
+    AMD_ARGS_NOW(y, parts, seq, total, stride_b, stride_i, arg_pair(by_seq));
+    constexpr int BS = kSplitLanes, NV = kSplitVecs;
+    const uint32_t part = blockIdx.x, r = blockIdx.y;
+    const uint32_t b = fast_quotient(r, by_seq), i = r - b * seq;
+    uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
+    const uint32_t keep = total - seq + i + 1;
+    const uint32_t from = part * static_cast<uint32_t>(kCausalSoftmaxPartColumns);
+    const uint32_t upto = from >= keep ? from : keep - from < kCausalSoftmaxPartColumns ? keep : from + static_cast<uint32_t>(kCausalSoftmaxPartColumns);
+    u32x4 x[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {// in flight while the row's parts are put together
+        const uint32_t c0 = from + (k * BS + threadIdx.x) * 8;
+        x[k] = c0 < upto ? ld16_stream(row + c0) : u32x4{0, 0, 0, 0};
+    }
+    // the row's maximum and its sum from its parts: lane p of every wavefront takes part p (at most 64 of them) and
+    // the wavefront trees put them together - the same values in the same order in every workgroup of the row
+    const CausalSoftmaxPart *of_row = parts + static_cast<size_t>(r) * gridDim.x;
+    const float neg_inf = -__builtin_inff();
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    CausalSoftmaxPart q{neg_inf, __builtin_inff(), 0.0f, 0.0f};
+    if (lane < gridDim.x) q = of_row[lane];
+    const float top = wave_max(q.max);
+    // a part at the row's maximum counts as it is (also where both are infinite); one without a kept or a
+    // finite element counts nothing beside a finite maximum
+    const float sum = wave_sum(q.max == top ? q.sum : q.max == neg_inf ? 0.0f : q.sum * expf(q.max - top));
+    const float my_min = __shfl(q.min, static_cast<int>(part));
+    const float rcp = 1.0f / sum;
+    const bool lean = my_min - top >= kLeanExpLimit;// uniform over the workgroup
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const uint32_t c0 = from + (k * BS + threadIdx.x) * 8;
+        if (c0 >= total) continue;
+        u32x4 packed{0, 0, 0, 0};
+        if (c0 < upto) {
+            float f[8], o[8];
+            widen8<T>(x[k], f);
+            if (lean) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[e] = exp_nonpositive(f[e] - top);
+            } else {
+                exp_any8(f, top);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float q = f[e] * rcp;
+                o[e] = c0 + e < upto ? __builtin_fmaf(__builtin_fmaf(-sum, q, f[e]), rcp, q) : 0.0f;
+            }
+            packed = narrow8_unit_range<T>(o);
+            if (c0 + 8 > upto) {// the masked end of the straddling vector is zero whatever the row turned into
+                uint32_t w[4] = {packed.x, packed.y, packed.z, packed.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (c0 + e >= upto) w[e / 2] &= (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                }
+                packed = u32x4{w[0], w[1], w[2], w[3]};
+            }
+        }
+        st16_stream(row + c0, packed);
+    }
+}
+
+template<typename T>
+void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, CausalSoftmaxPart *parts, hipStream_t stream) {
     auto *py = static_cast<uint16_t *>(data);
+    if (parts != nullptr) {// few long rows, and the caller brought the workspace: a row's parts on workgroups of their own
+        const dim3 grid(causal_softmax_parts(d), static_cast<unsigned>(d.batch * d.seq));
+        const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
+        causal_softmax_split_stats<T><<<grid, kSplitLanes, 0, stream>>>(py, parts, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by);
+        causal_softmax_split_apply<T><<<grid, kSplitLanes, 0, stream>>>(py, parts, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by);
+        return;
+    }
     const uint64_t rows = d.batch * d.seq;
     const uint64_t nvec = d.total / 8;
     // Rows of up to 3072 elements are taken by single wavefronts (no barrier, no

@@ -253,9 +253,16 @@ class CausalSoftmaxPlan(_Plan):
         size = ctypes.c_uint64(0)
         check_error(self.lib.infiniopGetCausalSoftmaxWorkspaceSize(desc, ctypes.byref(size)))
         self.workspace_size = size.value
+        # 0 for every shape but few long rows (decoding over a long context), whose parts meet in the workspace
+        self.workspace = None
+        if self.workspace_size:
+            import torch
 
-    def __call__(self, y, stream=None):
-        check_error(self.lib.infiniopCausalSoftmax(self.desc, None, self.workspace_size, y.data_ptr(), stream))
+            self.workspace = torch.empty(self.workspace_size, dtype=torch.uint8, device=y.device)
+
+    def __call__(self, y, stream=None, use_workspace=True):
+        ws = self.workspace.data_ptr() if (self.workspace is not None and use_workspace) else None
+        check_error(self.lib.infiniopCausalSoftmax(self.desc, ws, self.workspace_size if ws else 0, y.data_ptr(), stream))
         return y
 
 
@@ -380,9 +387,9 @@ class Context:
             torch.cuda.synchronize()  # the plan's workspace must outlive the work queued on it
             return res
 
-    def causal_softmax(self, y, stream=None):
+    def causal_softmax(self, y, stream=None, use_workspace=True):
         with CausalSoftmaxPlan(self, y) as plan:
-            return plan(y, stream)
+            return plan(y, stream, use_workspace)
 
     def rope(self, t, pos_ids, sin_table, cos_table, stream=None):
         with RoPEPlan(self, t, pos_ids, sin_table, cos_table) as plan:

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 TOL = {"f16": 1e-3, "bf16": 1e-2}
 
 
-def run(ctx, codes, shape, strides, dt):
+def run(ctx, codes, shape, strides, dt, use_workspace=True):
     import torch
 
     if strides is None:
@@ -21,7 +21,7 @@ def run(ctx, codes, shape, strides, dt):
     else:
         t, buf = strided_like(codes, shape, strides, dt)
     before = to_codes(buf)
-    ctx.causal_softmax(t)
+    ctx.causal_softmax(t, use_workspace=use_workspace)
     torch.cuda.synchronize()
     return to_codes(t), before, to_codes(buf)
 
@@ -194,9 +194,11 @@ def test_where_gpu_and_cpu_path_differ_the_gpu_is_the_exact_one(ctx, dt, shape):
     assert (got == exact)[keep].mean() > 0.9995
 
 
+@pytest.mark.parametrize("use_workspace", [False, True])
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-def test_long_row_forms_against_the_float64_quotient(ctx, dt):
-    """Rows of 32 769 elements and more form their exponentials with the hardware exp2 of one fused multiply-add
+def test_long_row_forms_against_the_float64_quotient(ctx, dt, use_workspace):
+    """(With the workspace these few rows are split over several workgroups each; without it a workgroup takes a row.)
+    Rows of 32 769 elements and more form their exponentials with the hardware exp2 of one fused multiply-add
     (relative error below 3e-6), the shorter ones with a corrected exponential: the same row is therefore not
     promised the same bits through both.  What is promised, and recorded here: every output of either form is
     within one unit in the last place of the float64 quotient narrowed by the type's rule, and the long-row form
@@ -206,7 +208,7 @@ def test_long_row_forms_against_the_float64_quotient(ctx, dt):
     for total in (32768, 40000, 40001, 65536, 65537, 100000, 131072, 200000):
         shape = (1, 4, total)
         y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 3, dt)
-        got, _, _ = run(ctx, y, shape, None, dt)
+        got, _, _ = run(ctx, y, shape, None, dt, use_workspace)
         got = got.reshape(shape)
         keep = np.broadcast_to(np.arange(total)[None, :] <= total - 4 + np.arange(4)[:, None], shape)
         x = np.where(keep, oracle.decode(y, dt).astype(np.float64).reshape(shape), -np.inf)
@@ -285,8 +287,9 @@ def test_infinities_and_long_tails_in_ragged_rows(ctx, dt, start, shape):
     assert not buf[:start].any() and not buf[start + batch * seq * total:].any()
 
 
-def test_infinities_and_long_tails_in_long_rows(ctx):
-    """The same special values in rows of 50 000 elements (the two-pass form)."""
+@pytest.mark.parametrize("use_workspace", [False, True])
+def test_infinities_and_long_tails_in_long_rows(ctx, use_workspace):
+    """The same special values in rows of 50 000 elements (held in registers)."""
     rng = np.random.default_rng(79)
     vals = rng.standard_normal((2, 6, 50000)).astype(np.float32) * 2
     vals[0, :, 3] = -np.inf
@@ -296,9 +299,87 @@ def test_infinities_and_long_tails_in_long_rows(ctx):
     vals[1, 5, :30000] = -60000.0
     y = oracle.encode(vals, "f16")
     want = oracle.causal_softmax(y.copy(), "f16")
-    got, _, _ = run(ctx, y, y.shape, None, "f16")
+    got, _, _ = run(ctx, y, y.shape, None, "f16", use_workspace)
     check(got, want, "f16", "infinities and tails, long rows", max_frac=2e-2)
     assert np.isnan(oracle.decode(got, "f16")[0, 4, 0])
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(8, 1, 131072), (32, 1, 131072), (3, 2, 262144), (5, 1, 131072), (2, 1, 200000), (1, 20, 147456), (16, 2, 163848)])
+def test_few_long_rows_split_over_workgroups(ctx, dt, shape):
+    """Decoding over a long context (131 072 keys and more): one query row, or a few, per head.  With the workspace the
+    library asks for, every row is split into parts of 16 384 columns on workgroups of their own (two launches);
+    without it a workgroup takes a row.  Both against the oracle, and against each other: within one unit, nearly all equal."""
+    from operators_amd.ops import CausalSoftmaxPlan
+
+    rng = np.random.default_rng(shape[0] * 131 + shape[2])
+    y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 3, dt)
+    with CausalSoftmaxPlan(ctx, to_torch(y, dt).reshape(shape)) as plan:
+        assert plan.workspace_size == shape[0] * shape[1] * -(-shape[2] // 16384) * 16
+    b, s_, t = shape
+    want = oracle.causal_softmax(y.copy(), dt)
+    split, _, _ = run(ctx, y, shape, None, dt, True)
+    whole, _, _ = run(ctx, y, shape, None, dt, False)
+    # the CPU path adds a row's exponentials one after the other in fp32: the longer the row, the more of its
+    # quotients land on the other side of a rounding boundary (3 % of bf16 outputs at 131 072 columns, 8 % at
+    # 262 144) - one unit at most, and the float64 quotient below says which side is right
+    loose = 0.2
+    check(split, want, dt, f"{shape} {dt} split", max_frac=loose)
+    check(whole, want, dt, f"{shape} {dt} a workgroup per row", max_frac=loose)
+    check(split, whole, dt, f"{shape} {dt} split against a workgroup per row", max_frac=2e-3)
+    # what both are held to: the float64 quotient narrowed by the type's rule
+    keep = np.broadcast_to(np.arange(t)[None, :] <= t - s_ + np.arange(s_)[:, None], shape)
+    x = np.where(keep, oracle.decode(y, dt).astype(np.float64).reshape(shape), -np.inf)
+    e = np.exp(x - x.max(-1, keepdims=True))
+    exact = oracle.encode((e / e.sum(-1, keepdims=True)).astype(np.float32).ravel(), dt).reshape(shape)
+    frac, worst = check(split.reshape(shape), exact, dt, f"{shape} {dt} split against float64", max_frac=1e-3)
+    assert worst <= 1
+    for i in range(s_):
+        assert not split.reshape(shape)[:, i, t - s_ + i + 1:].any(), "the masked part is exact zeros"
+
+
+@pytest.mark.parametrize("use_workspace", [False, True])
+def test_infinities_and_long_tails_in_few_very_long_rows(ctx, use_workspace):
+    """Special values where rows are split over workgroups: parts that are -inf throughout, a row that is, a part that
+    holds the row's only large value, parts more than 126 below the row's maximum, +inf, NaN."""
+    rng = np.random.default_rng(83)
+    vals = rng.standard_normal((2, 5, 140000)).astype(np.float32) * 2
+    vals[0, :, 3] = -np.inf
+    vals[0, 1, 16384:49152] = -np.inf
+    vals[0, 4, :] = -np.inf
+    vals[1, :, 139990] = -300.0
+    vals[1, 3, 70000] = 200.0
+    vals[1, 2, :100000] = -60000.0
+    vals[1, 0, 20000] = np.inf
+    vals[1, 1, 90000] = np.nan
+    y = oracle.encode(vals, "f16")
+    want = oracle.causal_softmax(y.copy(), "f16")
+    got, _, _ = run(ctx, y, y.shape, None, "f16", use_workspace)
+    check(got, want, "f16", "infinities and tails, few very long rows", max_frac=0.2)
+    out = oracle.decode(got, "f16")
+    assert np.isnan(out[0, 4, 0]) and np.isnan(out[1, 0, 5]) and np.isnan(out[1, 1, 5])
+
+
+def test_split_form_is_for_few_long_rows_only(ctx):
+    """No workspace is asked for where a workgroup per row fills the chip, where rows are short, or where rows are
+    not whole 16-byte vectors; and a strided view of few long rows takes the split form like a dense one."""
+    import torch
+
+    from operators_amd.ops import CausalSoftmaxPlan
+
+    for shape in [(32, 4096, 4096), (200, 1, 262144), (64, 1, 131072), (8, 1, 131064), (8, 1, 140001), (8, 1, 65536)]:
+        with CausalSoftmaxPlan(ctx, torch.empty(shape, dtype=torch.float16, device="cuda")) as plan:
+            assert plan.workspace_size == 0, shape
+    rng = np.random.default_rng(5)
+    shape, strides = (6, 2, 140000), (2 * 140008 + 16, 140008, 1)
+    y = oracle.encode(rng.standard_normal(shape).astype(np.float32) * 2, "f16")
+    want = oracle.causal_softmax(y.copy(), "f16")
+    got, before, after = run(ctx, y, shape, strides, "f16", True)
+    check(got, want, "f16", "strided few long rows, split", max_frac=0.2)
+    mask = np.zeros(before.size, bool)
+    idx = (np.arange(6)[:, None, None] * strides[0] + np.arange(2)[None, :, None] * strides[1] + np.arange(140000)[None, None, :]).ravel()
+    mask[idx] = True
+    assert np.array_equal(before[~mask], after[~mask]), "the gaps between the rows are left alone"
 
 
 def test_short_rows_give_the_bits_of_a_wavefront_per_row(ctx):
