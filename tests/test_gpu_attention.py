@@ -88,6 +88,40 @@ def test_against_float64_attention(ctx):
     assert np.all(np.abs(got - out) <= 1e-2 * np.abs(out) + 6 * 2.0 ** -10 * np.abs(V).max())
 
 
+def test_decoding_over_a_long_context(ctx):
+    """One new token against 131 071 cached ones: the scores are 8 rows of 131 072 columns, which CausalSoftmax
+    splits over workgroups through its share of Attention's workspace.  Against plain float64 attention."""
+    import torch
+
+    from operators_amd.ops import AttentionPlan
+
+    heads, kv_heads, seq, hd, pos, cap = 8, 2, 1, 64, 131071, 131072
+    rng = np.random.default_rng(78)
+    enc = lambda s: oracle.encode(rng.standard_normal(s).astype(np.float32), "f16")  # noqa: E731
+    q, k, v, kc, vc = enc((heads, seq, hd)), enc((kv_heads, seq, hd)), enc((kv_heads, seq, hd)), enc((kv_heads, cap, hd)), enc((kv_heads, cap, hd))
+    tout = torch.zeros((seq, heads, hd), dtype=torch.float16, device="cuda")
+    tq, tk, tv, tkc, tvc = (to_torch(x, "f16") for x in (q, k, v, kc, vc))
+    with AttentionPlan(ctx, tout, tq, tk, tv, tkc, tvc, pos) as plan:
+        scores, result, parts = heads * seq * cap * 2, heads * seq * hd * 2, heads * seq * (cap // 16384) * 16
+        assert plan.workspace_size == scores + result + parts  # (scores + result is a multiple of 16 here)
+    ctx.attention(tout, tq, tk, tv, tkc, tvc, pos)
+    torch.cuda.synchronize()
+    f = lambda x: oracle.decode(x, "f16").astype(np.float64)  # noqa: E731
+    K, V = f(kc), f(vc)
+    K[:, pos:pos + seq], V[:, pos:pos + seq] = f(k), f(v)
+    assert np.array_equal(to_codes(tkc)[:, pos], k[:, 0]) and np.array_equal(to_codes(tvc)[:, pos], v[:, 0]), "cache contents"
+    out = np.zeros((seq, heads, hd))
+    for h in range(heads):
+        s_ = f(q)[h] @ K[h // (heads // kv_heads)].T / np.sqrt(hd)
+        s_ = oracle.decode(oracle.encode(s_.astype(np.float32), "f16"), "f16").astype(np.float64)  # the scores are stored as fp16
+        p = np.exp(s_ - s_.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        p = oracle.decode(oracle.encode(p.astype(np.float32), "f16"), "f16").astype(np.float64)  # and so are the weights
+        out[:, h] = p @ V[h // (heads // kv_heads)]
+    got = f(to_codes(tout))
+    assert np.all(np.abs(got - out) <= 1e-2 * np.abs(out) + 6 * 2.0 ** -10 * np.abs(V).max())
+
+
 def test_status_codes_and_workspace(ctx):
     import torch
 
