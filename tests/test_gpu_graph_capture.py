@@ -106,3 +106,44 @@ def test_random_sample_replays_from_a_hip_graph(ctx):
         torch.cuda.synchronize()
         assert int(result.item()) == want[replay], replay
     plan.close()
+
+
+def test_split_causal_softmax_replays_from_a_hip_graph(ctx):
+    """The two launches that share very few very long rows among workgroups (their partial maxima and sums meet in
+    the workspace), captured once: every replay works on whatever the scores buffer holds and must give the bits of
+    an eager call on the same scores."""
+    import torch
+
+    from operators_amd.ops import CausalSoftmaxPlan
+
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(6)
+    draws = [(torch.randn((8, 1, 131072), device="cuda", generator=gen) * 3).to(torch.float16) for _ in range(3)]
+    scores = draws[0].clone()
+    plan = CausalSoftmaxPlan(ctx, scores)
+    assert plan.workspace_size > 0
+    want = []
+    for d in draws:
+        scores.copy_(d)
+        plan(scores)
+        torch.cuda.synchronize()
+        want.append(scores.clone())
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        scores.copy_(draws[0])
+        with torch.cuda.graph(graph, stream=side):
+            plan(scores, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for replay in range(6):
+        i = replay % len(draws)
+        plan.workspace.random_(0, 256)  # eager work between replays: the parts of the replay before are gone
+        scores.copy_(draws[i])
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(scores.view(torch.int16), want[i].view(torch.int16)), replay
+    plan.close()
