@@ -984,33 +984,33 @@ __global__ __launch_bounds__(256) void causal_softmax_generic(uint16_t *y, uint6
 
 // ---- few long rows: a row split over several workgroups, two launches --------------
 // Decoding over a long context is one query row per head: 64 rows of 131 072 columns keep 64 of 256 compute
-// units busy at a workgroup per row.  Here workgroup (part, row) takes kCausalSoftmaxPartColumns columns of the
-// row - 512 lanes x 4 vectors, held in registers.  The first launch leaves each part's maximum, minimum and sum
+// units busy at a workgroup per row.  Here workgroup (part, row) takes BS * 32 columns of the
+// row - BS lanes x 4 vectors, held in registers.  The first launch leaves each part's maximum, minimum and sum
 // of exp(x - maximum) over its kept columns in the workspace; the second reads the row's parts (the same few
 // values in every workgroup of the row, combined in the same order), rescales the sums to the row's maximum and
 // writes its own columns: exp(x - maximum) / sum, the exponentials and the quotient those of the other forms.
 // Rows start on 16-byte boundaries and are whole vectors long (the host sees to it).
-constexpr int kSplitLanes = 512, kSplitVecs = 4;
-static_assert(kSplitLanes * kSplitVecs * 8 == kCausalSoftmaxPartColumns, "a part is what one workgroup holds");
+constexpr int kSplitVecs = 4;
 
-template<typename T>
-__global__ __launch_bounds__(kSplitLanes) void causal_softmax_split_stats(const uint16_t *y, CausalSoftmaxPart *parts, uint32_t seq, uint32_t total,
+template<typename T, int BS>
+__global__ __launch_bounds__(BS) void causal_softmax_split_stats(const uint16_t *y, CausalSoftmaxPart *parts, uint32_t seq, uint32_t total,
                                                                            int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
     AMD_ARGS_NOW(y, parts, seq, total, stride_b, stride_i, arg_pair(by_seq));
-    constexpr int BS = kSplitLanes, NV = kSplitVecs, WAVES = BS / kWave;
+    constexpr int NV = kSplitVecs, WAVES = BS / kWave;
+    constexpr uint32_t kColumns = BS * NV * 8;
     __shared__ float red[6 * WAVES];
     const uint32_t part = blockIdx.x, r = blockIdx.y;
     const uint32_t b = fast_quotient(r, by_seq), i = r - b * seq;
     const uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
     const uint32_t keep = total - seq + i + 1;
-    const uint32_t from = part * static_cast<uint32_t>(kCausalSoftmaxPartColumns);
+    const uint32_t from = part * kColumns;
     CausalSoftmaxPart *mine = parts + static_cast<size_t>(r) * gridDim.x + part;
     const float neg_inf = -__builtin_inff();
     if (from >= keep) {// nothing of this part is kept (uniform over the workgroup)
         if (threadIdx.x == 0) *mine = CausalSoftmaxPart{neg_inf, __builtin_inff(), 0.0f, 0.0f};
         return;
     }
-    const uint32_t upto = keep - from < kCausalSoftmaxPartColumns ? keep : from + static_cast<uint32_t>(kCausalSoftmaxPartColumns);
+    const uint32_t upto = keep - from < kColumns ? keep : from + kColumns;
     float f[NV][8];
     float mx = neg_inf, mn = __builtin_inff();
     u32x4 x[NV];
@@ -1054,17 +1054,18 @@ __global__ __launch_bounds__(kSplitLanes) void causal_softmax_split_stats(const 
     if (threadIdx.x == 0) *mine = CausalSoftmaxPart{mx, mn, sum, 0.0f};
 }
 
-template<typename T>
-__global__ __launch_bounds__(kSplitLanes) void causal_softmax_split_apply(uint16_t *y, const CausalSoftmaxPart *parts, uint32_t seq, uint32_t total,
+template<typename T, int BS>
+__global__ __launch_bounds__(BS) void causal_softmax_split_apply(uint16_t *y, const CausalSoftmaxPart *parts, uint32_t seq, uint32_t total,
                                                                            int64_t stride_b, int64_t stride_i, FastDiv by_seq) {
     AMD_ARGS_NOW(y, parts, seq, total, stride_b, stride_i, arg_pair(by_seq));
-    constexpr int BS = kSplitLanes, NV = kSplitVecs;
+    constexpr int NV = kSplitVecs;
+    constexpr uint32_t kColumns = BS * NV * 8;
     const uint32_t part = blockIdx.x, r = blockIdx.y;
     const uint32_t b = fast_quotient(r, by_seq), i = r - b * seq;
     uint16_t *row = y + static_cast<int64_t>(b) * stride_b + static_cast<int64_t>(i) * stride_i;
     const uint32_t keep = total - seq + i + 1;
-    const uint32_t from = part * static_cast<uint32_t>(kCausalSoftmaxPartColumns);
-    const uint32_t upto = from >= keep ? from : keep - from < kCausalSoftmaxPartColumns ? keep : from + static_cast<uint32_t>(kCausalSoftmaxPartColumns);
+    const uint32_t from = part * kColumns;
+    const uint32_t upto = from >= keep ? from : keep - from < kColumns ? keep : from + kColumns;
     u32x4 x[NV];
 #pragma unroll
     for (int k = 0; k < NV; ++k) {// in flight while the row's parts are put together
@@ -1124,8 +1125,14 @@ void launch_causal_softmax(const CausalSoftmaxAmdDescriptor &d, void *data, Caus
     if (parts != nullptr) {// few long rows, and the caller brought the workspace: a row's parts on workgroups of their own
         const dim3 grid(causal_softmax_parts(d), static_cast<unsigned>(d.batch * d.seq));
         const FastDiv by = fast_div(static_cast<uint32_t>(d.seq));
-        causal_softmax_split_stats<T><<<grid, kSplitLanes, 0, stream>>>(py, parts, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by);
-        causal_softmax_split_apply<T><<<grid, kSplitLanes, 0, stream>>>(py, parts, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by);
+#define CS_SPLIT(BS)                                                                                                                                          \
+    do {                                                                                                                                                      \
+        causal_softmax_split_stats<T, BS><<<grid, BS, 0, stream>>>(py, parts, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by); \
+        causal_softmax_split_apply<T, BS><<<grid, BS, 0, stream>>>(py, parts, static_cast<uint32_t>(d.seq), static_cast<uint32_t>(d.total), d.stride_b, d.stride_i, by); \
+    } while (0)
+        if (causal_softmax_part_lanes(d) == 128) CS_SPLIT(128);
+        else CS_SPLIT(512);
+#undef CS_SPLIT
         return;
     }
     const uint64_t rows = d.batch * d.seq;

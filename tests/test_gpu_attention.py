@@ -102,7 +102,7 @@ def test_decoding_over_a_long_context(ctx):
     tout = torch.zeros((seq, heads, hd), dtype=torch.float16, device="cuda")
     tq, tk, tv, tkc, tvc = (to_torch(x, "f16") for x in (q, k, v, kc, vc))
     with AttentionPlan(ctx, tout, tq, tk, tv, tkc, tvc, pos) as plan:
-        scores, result, parts = heads * seq * cap * 2, heads * seq * hd * 2, heads * seq * (cap // 16384) * 16
+        scores, result, parts = heads * seq * cap * 2, heads * seq * hd * 2, heads * seq * (cap // 4096) * 16
         assert plan.workspace_size == scores + result + parts  # (scores + result is a multiple of 16 here)
     ctx.attention(tout, tq, tk, tv, tkc, tvc, pos)
     torch.cuda.synchronize()
