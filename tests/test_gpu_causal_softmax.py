@@ -305,7 +305,8 @@ def test_infinities_and_long_tails_in_long_rows(ctx, use_workspace):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-@pytest.mark.parametrize("shape", [(8, 1, 131072), (32, 1, 131072), (3, 2, 262144), (5, 1, 131072), (2, 1, 200000), (1, 20, 147456), (16, 2, 163848)])
+@pytest.mark.parametrize("shape", [(8, 1, 131072), (32, 1, 131072), (3, 2, 262144), (5, 1, 131072), (2, 1, 200000), (1, 20, 147456), (16, 2, 163848),
+                                   (1, 40, 131080)])  # the last part holds 8 columns, all of them masked in the first 31 rows
 def test_few_long_rows_split_over_workgroups(ctx, dt, shape):
     """Decoding over a long context (131 072 keys and more): one query row, or a few, per head.  With the workspace the
     library asks for, every row is split into parts of 16 384 (or 4096) columns on workgroups of their own (two launches);
