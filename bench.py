@@ -271,6 +271,27 @@ def make_attention(ctx, heads, kv_heads, seq, hd, dtype, gen, name):
     return Launch(name, ctx.lib.infiniopAttention, args, nbytes, (plan, qkv, k_cache, v_cache, out), flops)
 
 
+def make_attention_decode(ctx, heads, kv_heads, cached, hd, dtype, gen, name):
+    """One new token at position `cached`: the K and V caches hold cached + 1 rows after the call.  HBM-bound: what has
+    to move is K and V once."""
+    import torch
+
+    from operators_amd.ops import AttentionPlan
+
+    qkv = _randn((1, heads + 2 * kv_heads, hd), dtype, gen)
+    q = qkv[:, :heads, :].permute(1, 0, 2)
+    k = qkv[:, heads:heads + kv_heads, :].permute(1, 0, 2)
+    v = qkv[:, heads + kv_heads:, :].permute(1, 0, 2)
+    k_cache = _randn((kv_heads, cached + 1, hd), dtype, gen)
+    v_cache = _randn((kv_heads, cached + 1, hd), dtype, gen)
+    out = torch.empty((1, heads, hd), dtype=dtype, device="cuda")
+    plan = AttentionPlan(ctx, out, q, k, v, k_cache, v_cache, cached)
+    nbytes = (qkv.numel() + out.numel() + 2 * k_cache.numel()) * qkv.element_size()
+    args = (plan.desc, plan.workspace.data_ptr(), plan.workspace_size, out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            k_cache.data_ptr(), v_cache.data_ptr())
+    return Launch(name, ctx.lib.infiniopAttention, args, nbytes, (plan, qkv, k_cache, v_cache, out))
+
+
 def make_matmul(ctx, m, k, n, dtype, gen, name):
     import torch
 
@@ -451,6 +472,7 @@ def ops_table(ctx, args, gen):
         f"M1 matmul bf16 [{T},8192] x [8192,57344]": lambda: [make_matmul(ctx, T, 8192, 57344, bf16, gen, "matmul") for _ in range(2)],
         f"M2 mlp bf16 tokens {T}, d 8192, di 28672 (matmul + swiglu + matmul, residual)": lambda: [make_mlp(ctx, T, 8192, 28672, bf16, gen, "mlp") for _ in range(2)],
         "A1 attention bf16 prefill: 64 q heads, 8 kv heads, seq 4096, head_dim 128 (2 rearranges + matmul + causal softmax + matmul + rearrange)": lambda: [make_attention(ctx, 64, 8, 4096, 128, bf16, gen, "attention") for _ in range(2)],
+        "A2 attention bf16 decoding: 64 q heads, 8 kv heads, one token over 32767 cached ones, head_dim 128 (both products by this library's own kernels, bound by reading K and V once)": lambda: [make_attention_decode(ctx, 64, 8, 32767, 128, bf16, gen, "attention") for _ in range(sets_needed(2 * 8 * 32768 * 128 * 2, nset))],
         # sampling: one workgroup, latency-bound (64-300 KB of logits); the bandwidth columns say nothing here
         "S1 random_sample f16 voc 32000, top-k 50, top-p 0.9, temperature 0.8": lambda: [make_random_sample(ctx, 32000, 50, gen, "random_sample") for _ in range(MAX_SETS)],
         "S2 random_sample f16 voc 32000, greedy": lambda: [make_random_sample(ctx, 32000, 1, gen, "random_sample") for _ in range(MAX_SETS)],

@@ -27,11 +27,14 @@ struct AttentionPlan {
     uint64_t scores_bytes;// [n_q_head, seq, total]
     uint64_t result_bytes;// [n_q_head, seq, head_dim]
     uint64_t softmax_bytes;// what CausalSoftmax asks for (few long rows: decoding over a long context), behind the rest on a 16-byte boundary
+    uint64_t weighted_bytes;// what the second Matmul asks for (decoding: its sum over the keys is split over workgroups), behind that
     uint64_t k_offset_bytes, v_offset_bytes;// position `pos` in the caches
 };
 
 uint64_t softmax_offset(const AttentionPlan &p) { return (p.q_bytes + p.scores_bytes + p.result_bytes + 15) / 16 * 16; }
+uint64_t weighted_offset(const AttentionPlan &p) { return (softmax_offset(p) + p.softmax_bytes + 15) / 16 * 16; }
 uint64_t workspace_bytes(const AttentionPlan &p) {
+    if (p.weighted_bytes != 0) return weighted_offset(p) + p.weighted_bytes;
     return p.softmax_bytes != 0 ? softmax_offset(p) + p.softmax_bytes : p.q_bytes + p.scores_bytes + p.result_bytes;
 }
 
@@ -113,7 +116,7 @@ INFINIOP_C infiniopStatus_t infiniopCreateAttentionDescriptor(infiniopHandle_t h
     const DataLayout dt = q_desc->dt;
     const uint64_t es = dt.size;
 
-    auto *p = new (std::nothrow) AttentionPlan{handle->device, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, 0};
+    auto *p = new (std::nothrow) AttentionPlan{handle->device, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, 0, 0};
     if (p == nullptr) {
         return STATUS_MEMORY_NOT_ALLOCATED;
     }
@@ -151,6 +154,7 @@ INFINIOP_C infiniopStatus_t infiniopCreateAttentionDescriptor(infiniopHandle_t h
     infiniopTensorDescriptor_t v_full = d.make(v_cache_desc->dt, kv_heads, total, hd, v_cache_desc->strides[0], v_cache_desc->strides[1], 1);
     infiniopTensorDescriptor_t result_grouped = d.dense(dt, kv_heads, group * seq, hd);
     if (ok()) st = infiniopCreateMatmulDescriptor(handle, &p->weighted, result_grouped, 1.0f, scores_grouped, v_full, 0.0f);
+    if (ok()) st = infiniopGetMatmulWorkspaceSize(p->weighted, &p->weighted_bytes);
     p->result_bytes = heads * seq * hd * es;
 
     // out[seq, heads, hd] = result[heads, seq, hd] with its first two dimensions exchanged
@@ -193,6 +197,7 @@ INFINIOP_C infiniopStatus_t infiniopAttention(infiniopAttentionDescriptor_t desc
     char *scores = q_packed + p->q_bytes;
     char *result = scores + p->scores_bytes;
     char *softmax_parts = p->softmax_bytes != 0 ? static_cast<char *>(workspace) + softmax_offset(*p) : nullptr;
+    char *weighted_parts = p->weighted_bytes != 0 ? static_cast<char *>(workspace) + weighted_offset(*p) : nullptr;
 
     infiniopStatus_t st = infiniopRearrange(p->store_k, static_cast<char *>(k_cache) + p->k_offset_bytes, k, stream);
     if (st == STATUS_SUCCESS) st = infiniopRearrange(p->store_v, static_cast<char *>(v_cache) + p->v_offset_bytes, v, stream);
@@ -202,7 +207,7 @@ INFINIOP_C infiniopStatus_t infiniopAttention(infiniopAttentionDescriptor_t desc
     }
     if (st == STATUS_SUCCESS) st = infiniopMatmul(p->scores, nullptr, 0, scores, q, k_cache, stream);
     if (st == STATUS_SUCCESS) st = infiniopCausalSoftmax(p->softmax, softmax_parts, p->softmax_bytes, scores, stream);
-    if (st == STATUS_SUCCESS) st = infiniopMatmul(p->weighted, nullptr, 0, result, scores, v_cache, stream);
+    if (st == STATUS_SUCCESS) st = infiniopMatmul(p->weighted, weighted_parts, p->weighted_bytes, result, scores, v_cache, stream);
     if (st == STATUS_SUCCESS) st = infiniopRearrange(p->unpack_out, out, result, stream);
     return st;
 }

@@ -83,11 +83,13 @@ infiniopStatus_t amdCreateMatmulDescriptor(AmdHandle_t handle, MatmulAmdDescript
     return STATUS_SUCCESS;
 }
 
-infiniopStatus_t amdGetMatmulWorkspaceSize(MatmulAmdDescriptor_t, uint64_t *size) {
+infiniopStatus_t amdGetMatmulWorkspaceSize(MatmulAmdDescriptor_t desc, uint64_t *size) {
     if (size == nullptr) {
         return STATUS_BAD_PARAM;
     }
-    *size = 0;// as in the reference (matmul_cuda.cc:35-38); the BLAS library manages its own scratch
+    // 0 as in the reference (matmul_cuda.cc:35-38; the BLAS library manages its own scratch), except for the one
+    // shape this library splits along k itself; a call that comes without that workspace goes to the BLAS library
+    *size = amd_matmul_long_k_workspace(*desc);
     return STATUS_SUCCESS;
 }
 

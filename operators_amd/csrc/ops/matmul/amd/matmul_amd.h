@@ -58,4 +58,16 @@ infiniopStatus_t amdMatmul(MatmulAmdDescriptor_t desc, void *workspace, uint64_t
                            void *c, void const *a, void const *b, void *stream);
 infiniopStatus_t amdDestroyMatmulDescriptor(MatmulAmdDescriptor_t desc);
 
+// Few columns against very many rows of 32-512 contiguous elements (the scores of an attention while decoding):
+// this library's own kernel, bound by reading a once (matmul_skinny.hip).  a, b, c as the descriptor's
+// column-major problem has them; false when the call is not of that shape (nothing launched then).
+bool amd_matmul_skinny(const MatmulAmdDescriptor &desc, void *c, const void *a, const void *b, hipStream_t stream);
+// Few columns and up to 256 rows summed over very many k (the weighted values of an attention while decoding):
+// k split over workgroups, their partial sums through the workspace (matmul_long_k.hip).  The first gives the
+// bytes of workspace the descriptor's shape needs for it (0: not a shape for it); the second is false when the
+// call is not of that shape or came without that workspace (nothing launched then).
+uint64_t amd_matmul_long_k_workspace(const MatmulAmdDescriptor &desc);
+bool amd_matmul_long_k(const MatmulAmdDescriptor &desc, void *workspace, uint64_t workspace_size, void *c, const void *a, const void *b,
+                       hipStream_t stream);
+
 #endif

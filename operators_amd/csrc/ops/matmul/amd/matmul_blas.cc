@@ -80,21 +80,27 @@ HandlePool &pool() {
 
 }// namespace
 
-infiniopStatus_t amdMatmul(MatmulAmdDescriptor_t desc, void *, uint64_t, void *c, void const *a, void const *b, void *stream) {
+infiniopStatus_t amdMatmul(MatmulAmdDescriptor_t desc, void *workspace, uint64_t workspace_size, void *c, void const *a, void const *b, void *stream) {
     if (c == nullptr || a == nullptr || b == nullptr) {
         return STATUS_BAD_PARAM;
     }
     if (desc->m == 0 || desc->n == 0 || desc->batch == 0) {
         return STATUS_SUCCESS;
     }
-    if (!blas().ok) {
-        return STATUS_EXECUTION_FAILED;
-    }
     AMD_CHECK_HIP(hipSetDevice(desc->device_id), STATUS_BAD_DEVICE);
     if (desc->operands_swapped) {
         void const *t = a;
         a = b;
         b = t;
+    }
+    // the two products of an attention while decoding are not shapes for a library GEMM
+    if (amd_matmul_skinny(*desc, c, a, b, static_cast<hipStream_t>(stream)) ||
+        amd_matmul_long_k(*desc, workspace, workspace_size, c, a, b, static_cast<hipStream_t>(stream))) {
+        AMD_CHECK_HIP(hipGetLastError(), STATUS_EXECUTION_FAILED);
+        return STATUS_SUCCESS;
+    }
+    if (!blas().ok) {
+        return STATUS_EXECUTION_FAILED;
     }
     rocblas_datatype type;
     switch (desc->elem) {

@@ -155,9 +155,16 @@ class MatmulPlan(_Plan):
         size = ctypes.c_uint64(0)
         check_error(self.lib.infiniopGetMatmulWorkspaceSize(desc, ctypes.byref(size)))
         self.workspace_size = size.value
+        # 0 but for few columns summed over very many k (the weighted values of a decoding attention)
+        self.workspace = None
+        if self.workspace_size:
+            import torch
 
-    def __call__(self, c, a, b, stream=None):
-        check_error(self.lib.infiniopMatmul(self.desc, None, self.workspace_size, c.data_ptr(), a.data_ptr(), b.data_ptr(), stream))
+            self.workspace = torch.empty(self.workspace_size, dtype=torch.uint8, device=c.device)
+
+    def __call__(self, c, a, b, stream=None, use_workspace=True):
+        ws = self.workspace.data_ptr() if (self.workspace is not None and use_workspace) else None
+        check_error(self.lib.infiniopMatmul(self.desc, ws, self.workspace_size if ws else 0, c.data_ptr(), a.data_ptr(), b.data_ptr(), stream))
         return c
 
 

@@ -90,7 +90,8 @@ def test_against_float64_attention(ctx):
 
 def test_decoding_over_a_long_context(ctx):
     """One new token against 131 071 cached ones: the scores are 8 rows of 131 072 columns, which CausalSoftmax
-    splits over workgroups through its share of Attention's workspace.  Against plain float64 attention."""
+    splits over workgroups through its share of Attention's workspace; both products are this library's own kernels
+    (the second through its share of the workspace).  Against plain float64 attention."""
     import torch
 
     from operators_amd.ops import AttentionPlan
@@ -103,7 +104,8 @@ def test_decoding_over_a_long_context(ctx):
     tq, tk, tv, tkc, tvc = (to_torch(x, "f16") for x in (q, k, v, kc, vc))
     with AttentionPlan(ctx, tout, tq, tk, tv, tkc, tvc, pos) as plan:
         scores, result, parts = heads * seq * cap * 2, heads * seq * hd * 2, heads * seq * (cap // 4096) * 16
-        assert plan.workspace_size == scores + result + parts  # (scores + result is a multiple of 16 here)
+        weighted = kv_heads * (cap // 512) * hd * 8 * 4  # the second Matmul's partial sums: chunks of 512 keys, 8 columns of fp32 per chunk
+        assert plan.workspace_size == scores + result + parts + weighted  # (every part is a multiple of 16 here)
     ctx.attention(tout, tq, tk, tv, tkc, tvc, pos)
     torch.cuda.synchronize()
     f = lambda x: oracle.decode(x, "f16").astype(np.float64)  # noqa: E731

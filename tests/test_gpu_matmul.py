@@ -80,6 +80,79 @@ def test_against_oracle(ctx, dt, case):
     check(got, ref, exact, mag, a_shape[-1], dt, f"case {case} {dt}")
 
 
+# The two products of an attention while decoding, which this library serves with kernels of its own instead of the
+# BLAS library's: scores = q @ K^T (few queries against many keys: matmul_skinny) and out = weights @ V (a sum over many
+# keys: matmul_long_k, through the workspace Matmul then asks for).
+# batch, queries, head_dim, keys, cache rows (the caches are [batch, rows, head_dim]: K^T and V are views of them)
+DECODE_CASES = [(8, 8, 128, 4096, 4096), (2, 8, 128, 33000, 33008), (3, 5, 64, 1031, 2048), (2, 16, 256, 2049, 2056), (1, 1, 32, 1024, 1024),
+                (2, 3, 96, 3001, 3008), (2, 8, 512, 1500, 1504), (2, 7, 16, 50001, 50008), (1, 8, 8, 1500, 1504), (4, 4, 128, 131072, 131072)]
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("case", range(len(DECODE_CASES)))
+@pytest.mark.parametrize("alpha,beta", [(0.125, 0.0), (0.5, 0.25)])
+def test_the_products_of_a_decoding_attention(ctx, dt, case, alpha, beta):
+    import torch
+
+    from operators_amd.ops import MatmulPlan
+
+    batch, nq, hd, keys, rows = DECODE_CASES[case]
+    rng = np.random.default_rng(3000 + case)
+    q = make((batch, nq, hd), dt, rng, False)
+    cache = make((batch, rows, hd), dt, rng, False)
+    weights = make((batch, nq, keys), dt, rng, True)
+    tq, tcache, tw = to_torch(q, dt), to_torch(cache, dt), to_torch(weights, dt)
+    fq, fc, fw = as_f64(q, dt), as_f64(cache, dt)[:, :keys], as_f64(weights, dt)
+
+    # scores [batch, queries, keys] = alpha * q @ K^T + beta * scores, K^T a view of the cache
+    s0 = make((batch, nq, keys), dt, rng, False)
+    ts = to_torch(s0, dt)
+    k_t = tcache[:, :keys, :].transpose(1, 2)
+    ctx.matmul(ts, tq, k_t, alpha, beta)
+    torch.cuda.synchronize()
+    exact = alpha * np.matmul(fq, fc.transpose(0, 2, 1)) + beta * as_f64(s0, dt)
+    mag = abs(alpha) * np.matmul(np.abs(fq), np.abs(fc).transpose(0, 2, 1)) + abs(beta) * np.abs(as_f64(s0, dt))
+    g = as_f64(to_codes(ts), dt)
+    assert np.all(np.abs(g - exact) <= 0.5 * ULP[dt] * np.abs(exact) + 4 * hd * 2.0 ** -24 * mag + 1e-30), f"scores case {case} {dt}"
+
+    # out [batch, queries, head_dim] = alpha * weights @ V + beta * out, with the workspace and without (the BLAS library then)
+    o0 = make((batch, nq, hd), dt, rng, False)
+    v = tcache[:, :keys, :]
+    exact = alpha * np.matmul(fw, fc) + beta * as_f64(o0, dt)
+    mag = abs(alpha) * np.matmul(np.abs(fw), np.abs(fc)) + abs(beta) * np.abs(as_f64(o0, dt))
+    for use_workspace in (True, False):
+        to = to_torch(o0, dt)
+        with MatmulPlan(ctx, to, tw, v, alpha, beta) as plan:
+            fits = hd in (8, 16, 32, 64, 128, 256) and nq <= 8 and keys >= 1024
+            assert (plan.workspace_size > 0) == fits, (case, plan.workspace_size)
+            plan(to, tw, v, None, use_workspace)
+        torch.cuda.synchronize()
+        g = as_f64(to_codes(to), dt)
+        assert np.all(np.abs(g - exact) <= 0.5 * ULP[dt] * np.abs(exact) + 4 * keys * 2.0 ** -24 * mag + 1e-30), f"weighted values case {case} {dt} workspace {use_workspace}"
+
+
+def test_decoding_products_with_special_values(ctx):
+    """An infinity or a NaN in one key's values, or in one weight, reaches exactly the outputs it reaches in the float64
+    product - also where the key count is odd and the last pair of keys is half empty."""
+    import torch
+
+    rng = np.random.default_rng(9)
+    batch, nq, hd, keys = 2, 5, 128, 2047
+    cache = rng.standard_normal((batch, keys, hd)).astype(np.float32)
+    weights = rng.random((batch, nq, keys), dtype=np.float32)
+    cache[0, 2046, 3] = np.inf   # the last key (odd count: alone in its pair)
+    cache[1, 100, 7] = np.nan
+    weights[1, 2, 5] = np.inf
+    tc, tw = to_torch(oracle.encode(cache, "f16"), "f16"), to_torch(oracle.encode(weights, "f16"), "f16")
+    to = torch.zeros((batch, nq, hd), dtype=torch.float16, device="cuda")
+    ctx.matmul(to, tw, tc)
+    torch.cuda.synchronize()
+    with np.errstate(invalid="ignore", over="ignore"):
+        exact = np.matmul(as_f64(oracle.encode(weights, "f16"), "f16"), as_f64(oracle.encode(cache, "f16"), "f16"))
+    got = as_f64(to_codes(to), "f16")
+    assert np.array_equal(np.isnan(got), np.isnan(exact)) and np.array_equal(np.isinf(got), np.isinf(exact))
+
+
 def test_identity_and_permutation_are_exact(ctx):
     """a @ I = a and a @ P = a with its columns permuted: no rounding anywhere."""
     import torch
