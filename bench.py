@@ -231,7 +231,7 @@ def make_add_rms_norm(ctx, n, d, dtype, w_dtype, gen, name):
     return Launch(name, ctx.lib.infiniopAddRMSNorm, (plan.desc, None, 0, y.data_ptr(), a.data_ptr(), a.data_ptr(), b.data_ptr(), w.data_ptr()), nbytes, (plan, a, b, w, y))
 
 
-def make_mlp(ctx, tokens, d, di, dtype, gen, name):
+def make_mlp(ctx, tokens, d, di, dtype, gen, name, hbm_bound=False):
     """The reference's MLP composite: x @ w12 -> SwiGLU on the fused gate/up halves -> @ w3, added onto y."""
     import torch
 
@@ -246,7 +246,7 @@ def make_mlp(ctx, tokens, d, di, dtype, gen, name):
     nbytes = (x.numel() + 2 * y.numel() + w12.numel() + w3.numel()) * es + 2 * (tokens * 2 * di + tokens * di) * es
     flops = 2 * tokens * d * 2 * di + 2 * tokens * di * d
     args = (plan.desc, plan.workspace.data_ptr(), plan.workspace_size, y.data_ptr(), x.data_ptr(), w12.data_ptr(), w3.data_ptr())
-    return Launch(name, ctx.lib.infiniopMLP, args, nbytes, (plan, x, y, w12, w3), flops)
+    return Launch(name, ctx.lib.infiniopMLP, args, nbytes, (plan, x, y, w12, w3), None if hbm_bound else flops)  # few tokens: bound by reading the weights once
 
 
 def make_attention(ctx, heads, kv_heads, seq, hd, dtype, gen, name):
@@ -471,6 +471,7 @@ def ops_table(ctx, args, gen):
         # GEMM-bound rows (a library GEMM; priced against the MFMA peak): the gate/up projection and the whole MLP of a Llama-70B layer
         f"M1 matmul bf16 [{T},8192] x [8192,57344]": lambda: [make_matmul(ctx, T, 8192, 57344, bf16, gen, "matmul") for _ in range(2)],
         f"M2 mlp bf16 tokens {T}, d 8192, di 28672 (matmul + swiglu + matmul, residual)": lambda: [make_mlp(ctx, T, 8192, 28672, bf16, gen, "mlp") for _ in range(2)],
+        "M3 mlp bf16 decoding: 1 token, d 8192, di 28672 (both weight matrices read once; the sums over the input widths split over workgroups by this library's own kernel)": lambda: [make_mlp(ctx, 1, 8192, 28672, bf16, gen, "mlp", True) for _ in range(2)],
         "A1 attention bf16 prefill: 64 q heads, 8 kv heads, seq 4096, head_dim 128 (2 rearranges + matmul + causal softmax + matmul + rearrange)": lambda: [make_attention(ctx, 64, 8, 4096, 128, bf16, gen, "attention") for _ in range(2)],
         "A2 attention bf16 decoding: 64 q heads, 8 kv heads, one token over 32767 cached ones, head_dim 128 (both products by this library's own kernels, bound by reading K and V once)": lambda: [make_attention_decode(ctx, 64, 8, 32767, 128, bf16, gen, "attention") for _ in range(sets_needed(2 * 8 * 32768 * 128 * 2, nset))],
         # sampling: one workgroup, latency-bound (64-300 KB of logits); the bandwidth columns say nothing here

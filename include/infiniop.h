@@ -287,10 +287,10 @@ INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopCreateMatmulDescriptor(
     infiniopHandle_t handle, infiniopMatmulDescriptor_t *desc_ptr,
     infiniopTensorDescriptor_t c_desc, float alpha,
     infiniopTensorDescriptor_t a_desc, infiniopTensorDescriptor_t b_desc, float beta);
-/* replaces include/ops/matmul/matmul.h:21 - 0 bytes, except where a product of up to 8 columns and up to 256
- * rows sums over 1024 and more k (the weighted values of an attention while decoding): 32 x rows bytes per 128
- * to 1024 of k, for the partial sums of the workgroups that share the sum.  A call that comes without that
- * workspace is served all the same, by the BLAS library. */
+/* replaces include/ops/matmul/matmul.h:21 - 0 bytes, except where up to 8 rows of a (tokens, or the queries of
+ * a decoding attention) meet 1024 and more of k: 32 bytes per column of c and chunk of 128 to 2048 of k, for the
+ * partial sums of the workgroups that share the sum.  A call that comes without that workspace is served all
+ * the same, by the BLAS library. */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopGetMatmulWorkspaceSize(infiniopMatmulDescriptor_t desc, uint64_t *size);
 /* replaces include/ops/matmul/matmul.h:23-29 */
 INFINIOP_C INFINIOP_EXPORT infiniopStatus_t infiniopMatmul(

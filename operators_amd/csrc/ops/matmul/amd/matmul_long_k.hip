@@ -9,6 +9,9 @@
 // K/V head, 8 heads, bf16: 152 us for 268 MB; 59 us at 32768 keys, 18 us at
 // 4096); it is bound by reading a once.
 //
+// The same two launches serve a few tokens through a weight matrix (m = the
+// layer's output width in the thousands: matmul_long_k_wide below).
+//
 // Two launches.  The first splits k into chunks, a workgroup of 256 lanes
 // each: m / 8 lanes cover a column of a (16 bytes, 8 rows, per lane), so a
 // wavefront takes 512 / m pairs of neighbouring columns per step; a lane
@@ -155,6 +158,99 @@ __global__ __launch_bounds__(kLanes) void matmul_long_k_partial(float *partial, 
     }
 }
 
+// The same product with many rows: a few tokens through a weight matrix while decoding (c^T = W^T x^T: m is the
+// layer's output width, k its input width, the n columns are the tokens).  A workgroup is one wavefront, a lane
+// takes 8 rows of a tile of 512 and every column of its chunk of k, so no two lanes share a row and nothing is
+// added across lanes; the tokens' pairs along k come from LDS, the same 32 bytes for every lane.
+constexpr int kWideRows = 512, kWideAhead = 4;
+
+template<bool BF>
+__global__ __launch_bounds__(kWave) void matmul_long_k_wide(float *partial, const uint16_t *a, const uint16_t *b, uint32_t m, uint32_t n,
+                                                             uint32_t k, uint32_t chunk, uint32_t tiles, int64_t lda, int64_t ldb,
+                                                             int64_t batch_a, int64_t batch_b) {
+    AMD_ARGS_NOW(partial, a, b, m, n, k, chunk, tiles, lda, ldb, batch_a, batch_b);
+    extern __shared__ __attribute__((aligned(16))) uint32_t staged[];// [pair of k][column of b]
+    const uint32_t lane = threadIdx.x;
+    const uint32_t ch = blockIdx.x / tiles, tile = blockIdx.x - ch * tiles;// neighbouring workgroups read neighbouring KiBs of the same columns
+    const uint32_t chunks = gridDim.x / tiles;
+    const uint32_t k0 = ch * chunk;
+    const uint32_t here = k - k0 < chunk ? k - k0 : chunk;
+    a += static_cast<int64_t>(blockIdx.y) * batch_a;
+    b += static_cast<int64_t>(blockIdx.y) * batch_b;
+    const uint32_t pairs = (here + 1) / 2;
+    for (uint32_t w = lane; w < pairs * kColumnsOfB; w += kWave) {
+        const uint32_t j = w / pairs, p = w - j * pairs;
+        uint32_t word = 0;
+        if (j < n) {
+            const uint16_t *at = b + static_cast<int64_t>(j) * ldb + k0 + 2 * p;
+            word = 2 * p + 1 < here ? *reinterpret_cast<const u32_any *>(at) : static_cast<uint32_t>(*at);
+        }
+        staged[p * kColumnsOfB + j] = word;
+    }
+    __syncthreads();
+
+    const uint32_t row0 = tile * kWideRows + lane * 8;
+    const bool rows_here = row0 < m;// m is a multiple of 8: a lane's rows are all there or none is
+    float acc[kColumnsOfB][8];
+#pragma unroll
+    for (int j = 0; j < kColumnsOfB; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.0f;
+    }
+    const uint16_t *mine = a + static_cast<int64_t>(k0) * lda + (rows_here ? row0 : 0);
+    // Two sets of registers take turns: the loads of the next kWideAhead pairs of columns go out before the work on
+    // the ones that have arrived, so a wavefront always has loads in flight.
+    const auto fetch = [&](uint32_t p0, u32x4(&lo)[kWideAhead], u32x4(&hi)[kWideAhead]) {
+#pragma unroll
+        for (int s = 0; s < kWideAhead; ++s) {
+            const uint32_t c0 = 2 * (p0 + s), c1 = c0 + 1;// a column past the end is the chunk's last one again, and is not used
+            lo[s] = ld16_stream(mine + static_cast<int64_t>(c0 < here ? c0 : here - 1) * lda);
+            hi[s] = ld16_stream(mine + static_cast<int64_t>(c1 < here ? c1 : here - 1) * lda);
+        }
+    };
+    const auto work = [&](uint32_t p0, const u32x4(&lo)[kWideAhead], const u32x4(&hi)[kWideAhead]) {
+#pragma unroll
+        for (int s = 0; s < kWideAhead; ++s) {
+            const uint32_t p = p0 + s;
+            if (p >= pairs) break;// uniform over the wavefront
+            const bool has1 = 2 * p + 1 < here;
+            const uint32_t x[4] = {lo[s].x, lo[s].y, lo[s].z, lo[s].w};
+            const uint32_t y[4] = {has1 ? hi[s].x : 0u, has1 ? hi[s].y : 0u, has1 ? hi[s].z : 0u, has1 ? hi[s].w : 0u};
+            uint32_t v[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[2 * i] = __builtin_amdgcn_perm(y[i], x[i], 0x05040100u);
+                v[2 * i + 1] = __builtin_amdgcn_perm(y[i], x[i], 0x07060302u);
+            }
+            const u32x4 w0 = *reinterpret_cast<const u32x4 *>(staged + p * kColumnsOfB);
+            const u32x4 w1 = *reinterpret_cast<const u32x4 *>(staged + p * kColumnsOfB + 4);
+            const uint32_t w[kColumnsOfB] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+            for (int j = 0; j < kColumnsOfB; ++j) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[j][e] = dot2<BF>(v[e], w[j], acc[j][e]);
+            }
+        }
+    };
+    u32x4 lo0[kWideAhead], hi0[kWideAhead], lo1[kWideAhead], hi1[kWideAhead];
+    fetch(0, lo0, hi0);
+    for (uint32_t p0 = 0; p0 < pairs; p0 += 2 * kWideAhead) {
+        fetch(p0 + kWideAhead, lo1, hi1);
+        work(p0, lo0, hi0);
+        fetch(p0 + 2 * kWideAhead, lo0, hi0);
+        work(p0 + kWideAhead, lo1, hi1);
+    }
+    if (!rows_here) return;
+    float *out = partial + (static_cast<size_t>(blockIdx.y) * chunks + ch) * (static_cast<size_t>(m) * kColumnsOfB) + row0;
+#pragma unroll
+    for (int j = 0; j < kColumnsOfB; ++j) {
+        if (static_cast<uint32_t>(j) >= n) break;// the sums of columns b does not have are never read
+        f32x4 *at = reinterpret_cast<f32x4 *>(out + static_cast<size_t>(j) * m);
+        at[0] = f32x4{acc[j][0], acc[j][1], acc[j][2], acc[j][3]};
+        at[1] = f32x4{acc[j][4], acc[j][5], acc[j][6], acc[j][7]};
+    }
+}
+
 template<bool BF>
 __global__ __launch_bounds__(256) void matmul_long_k_combine(uint16_t *c, const float *partial, uint32_t m, uint32_t n, uint32_t chunks,
                                                              int64_t ldc, int64_t batch_c, float alpha, float beta) {
@@ -180,64 +276,98 @@ __global__ __launch_bounds__(256) void matmul_long_k_combine(uint16_t *c, const 
     *out = narrow<BF>(v);
 }
 
-bool shape_fits(const MatmulAmdDescriptor &d) {
-    const bool sixteen_bit = d.elem == amd::Elem::F16 || d.elem == amd::Elem::BF16;
-    if (!sixteen_bit || d.n < 1 || d.n > kColumnsOfB || d.k < 1024 || d.k > 0x7FFFFFF0ll || d.batch < 1 || d.batch > 65535) return false;
-    if (d.m < 8 || d.m > 256 || (d.m & (d.m - 1)) != 0) return false;
-    // columns of a and of b contiguous, c's columns contiguous; 16-byte loads of a
-    if (d.a.row_stride != 1 || d.b.row_stride != 1 || d.c.row_stride != 1) return false;
-    if (d.a.col_stride % 8 != 0 || d.a.stride % 8 != 0 || d.a.col_stride < d.m || d.b.col_stride < d.k || d.c.col_stride < d.m) return false;
-    return true;
-}
+struct Plan {
+    int kind;// 0: not a shape for these kernels, 1: up to 256 rows (a workgroup covers them all), 2: many rows (tiles of 512)
+    uint32_t chunk, chunks, tiles;
+};
 
-// Columns of a per workgroup: the largest of 1024, 512, 256 that still gives the chip 512 workgroups, else 128.  A
+// Columns of a per workgroup, few rows: the largest of 1024, 512, 256 that still gives the chip 512 workgroups, else 128.  A
 // workgroup works through its chunk in turns of 128 columns, a memory latency each, and ends with a sum over its
 // lanes that costs as much as a turn or two.  Measured, 8 batches of [128 x k] x [k x 8] bf16, both launches, us,
 // chunks of 128 / 256 / 512 / 1024 / 2048: k = 4096: 11.1 / 11.6 / 14.7 / 22.4 / 36.1; 32768: 41.9 / 29.8 / 25.2 /
 // 28.4 / 43.7; 131072: 141 / 93.0 / 73.6 / 62.6 / 64.9.
-uint32_t chunk_of(const MatmulAmdDescriptor &d) {
-    for (const uint32_t c : {1024u, 512u, 256u}) {
-        if (static_cast<uint64_t>(d.batch) * ((d.k + c - 1) / c) >= 512) return c;
+Plan plan_of(const MatmulAmdDescriptor &d) {
+    const Plan none{0, 0, 0, 0};
+    const bool sixteen_bit = d.elem == amd::Elem::F16 || d.elem == amd::Elem::BF16;
+    if (!sixteen_bit || d.n < 1 || d.n > kColumnsOfB || d.k < 1024 || d.k > 0x7FFFFFF0ll || d.batch < 1 || d.batch > 65535) return none;
+    // columns of a and of b contiguous, c's columns contiguous; 16-byte loads of a
+    if (d.a.row_stride != 1 || d.b.row_stride != 1 || d.c.row_stride != 1) return none;
+    if (d.a.col_stride % 8 != 0 || d.a.stride % 8 != 0 || d.a.col_stride < d.m || d.b.col_stride < d.k || d.c.col_stride < d.m) return none;
+    if (d.m >= 8 && d.m <= 256 && (d.m & (d.m - 1)) == 0) {
+        uint32_t chunk = 128;
+        for (const uint32_t c : {1024u, 512u, 256u}) {
+            if (static_cast<uint64_t>(d.batch) * ((d.k + c - 1) / c) >= 512) {
+                chunk = c;
+                break;
+            }
+        }
+        return Plan{1, chunk, static_cast<uint32_t>((d.k + chunk - 1) / chunk), 1};
     }
-    return 128;
+    // Many rows: about 1024 wavefronts in all, chunks of 256 columns and more (a chunk leaves 32 bytes of partial
+    // sums per row and column of b behind).  Measured against the BLAS library, bf16, us, 1 / 8 columns of b:
+    // [8192 x 28672]: 81 / 91 against 127 / 132; [22016 x 4096]: 36 / 42 against 52 / 52; [10240 x 8192]: 36 / 42
+    // against 49 / 50; [8192 x 8192]: 38 / 42 against 43 / 44; [57344 x 8192]: 155 / 172 against 158 / 166 - the
+    // library reads that one at 5.7 TB/s, and keeps it from three columns of b on.
+    if (d.m >= 1024 && d.m % 8 == 0 && d.m <= 0x7FFFFFF0ll && d.m * kColumnsOfB < (1ll << 31)) {
+        const uint32_t tiles = static_cast<uint32_t>((d.m + kWideRows - 1) / kWideRows);
+        if (tiles >= 64 && d.n > 2) return none;
+        uint64_t chunks = 1024 / (static_cast<uint64_t>(tiles) * d.batch);
+        if (chunks < 1) chunks = 1;
+        uint64_t chunk = (d.k + chunks - 1) / chunks;
+        if (chunk < 256) chunk = 256;
+        chunk = (chunk + 15) / 16 * 16;
+        if (chunk > 2048) chunk = 2048;// 32 KiB of LDS for b's share
+        chunks = (d.k + chunk - 1) / chunk;
+        if (static_cast<uint64_t>(tiles) * chunks > 0x7FFFFFFFull) return none;
+        return Plan{2, static_cast<uint32_t>(chunk), static_cast<uint32_t>(chunks), tiles};
+    }
+    return none;
 }
 
 }// namespace
 
 // Bytes of workspace with which amd_matmul_long_k serves the descriptor's shape; 0: not a shape for it.
 uint64_t amd_matmul_long_k_workspace(const MatmulAmdDescriptor &d) {
-    if (!shape_fits(d)) return 0;
-    const uint64_t chunk = chunk_of(d), chunks = (d.k + chunk - 1) / chunk;
-    return static_cast<uint64_t>(d.batch) * chunks * d.m * kColumnsOfB * sizeof(float);
+    const Plan p = plan_of(d);
+    if (p.kind == 0) return 0;
+    return static_cast<uint64_t>(d.batch) * p.chunks * d.m * kColumnsOfB * sizeof(float);
 }
+
+namespace {
+
+template<bool BF>
+void launch_long_k(const MatmulAmdDescriptor &d, const Plan &p, float *partial, void *c, const void *a, const void *b, hipStream_t stream) {
+    const auto *pa = static_cast<const uint16_t *>(a);
+    const auto *pb = static_cast<const uint16_t *>(b);
+    const uint32_t m = static_cast<uint32_t>(d.m), n = static_cast<uint32_t>(d.n), k = static_cast<uint32_t>(d.k);
+    if (p.kind == 1) {
+        uint32_t lpc_shift = 0;
+        while ((8u << lpc_shift) < m) ++lpc_shift;
+        const size_t lds = std::max<size_t>(static_cast<size_t>(p.chunk / 2) * kColumnsOfB * sizeof(uint32_t),
+                                            static_cast<size_t>(kLanes / kWave) * (m / 8) * kColumnsOfB * 8 * sizeof(float));
+        matmul_long_k_partial<BF><<<dim3(p.chunks, static_cast<unsigned>(d.batch)), kLanes, lds, stream>>>(
+            partial, pa, pb, m, n, k, p.chunk, lpc_shift, d.a.col_stride, d.b.col_stride, d.a.stride, d.b.stride);
+    } else {
+        const size_t lds = static_cast<size_t>((p.chunk + 1) / 2) * kColumnsOfB * sizeof(uint32_t);
+        matmul_long_k_wide<BF><<<dim3(p.tiles * p.chunks, static_cast<unsigned>(d.batch)), kWave, lds, stream>>>(
+            partial, pa, pb, m, n, k, p.chunk, p.tiles, d.a.col_stride, d.b.col_stride, d.a.stride, d.b.stride);
+    }
+    const dim3 grid2(static_cast<unsigned>((d.m * d.n + 255) / 256), static_cast<unsigned>(d.batch));
+    matmul_long_k_combine<BF><<<grid2, 256, 0, stream>>>(static_cast<uint16_t *>(c), partial, m, n, p.chunks, d.c.col_stride, d.c.stride,
+                                                         d.alpha, d.beta);
+}
+
+}// namespace
 
 // a, b, c: the operands of the descriptor's column-major problem.  False: not of this shape, or the workspace is
 // missing or short; nothing was launched.
 bool amd_matmul_long_k(const MatmulAmdDescriptor &d, void *workspace, uint64_t workspace_size, void *c, const void *a, const void *b,
                        hipStream_t stream) {
+    const Plan p = plan_of(d);
     const uint64_t need = amd_matmul_long_k_workspace(d);
-    if (need == 0 || workspace == nullptr || workspace_size < need || !amd::aligned16(workspace) || !amd::aligned16(a)) return false;
+    if (p.kind == 0 || workspace == nullptr || workspace_size < need || !amd::aligned16(workspace) || !amd::aligned16(a)) return false;
     if ((reinterpret_cast<uintptr_t>(b) & 1u) != 0 || (reinterpret_cast<uintptr_t>(c) & 1u) != 0) return false;
-    const uint32_t chunk = chunk_of(d), chunks = static_cast<uint32_t>((d.k + chunk - 1) / chunk);
-    uint32_t lpc_shift = 0;
-    while ((8u << lpc_shift) < static_cast<uint32_t>(d.m)) ++lpc_shift;
-    const size_t lds = std::max<size_t>(static_cast<size_t>(chunk / 2) * kColumnsOfB * sizeof(uint32_t),
-                                        static_cast<size_t>(kLanes / kWave) * (d.m / 8) * kColumnsOfB * 8 * sizeof(float));
-    auto *partial = static_cast<float *>(workspace);
-    const dim3 grid(chunks, static_cast<unsigned>(d.batch));
-    const dim3 grid2(static_cast<unsigned>((d.m * d.n + 255) / 256), static_cast<unsigned>(d.batch));
-    if (d.elem == amd::Elem::BF16) {
-        matmul_long_k_partial<true><<<grid, kLanes, lds, stream>>>(partial, static_cast<const uint16_t *>(a), static_cast<const uint16_t *>(b),
-                                                                   static_cast<uint32_t>(d.m), static_cast<uint32_t>(d.n), static_cast<uint32_t>(d.k),
-                                                                   chunk, lpc_shift, d.a.col_stride, d.b.col_stride, d.a.stride, d.b.stride);
-        matmul_long_k_combine<true><<<grid2, 256, 0, stream>>>(static_cast<uint16_t *>(c), partial, static_cast<uint32_t>(d.m),
-                                                               static_cast<uint32_t>(d.n), chunks, d.c.col_stride, d.c.stride, d.alpha, d.beta);
-    } else {
-        matmul_long_k_partial<false><<<grid, kLanes, lds, stream>>>(partial, static_cast<const uint16_t *>(a), static_cast<const uint16_t *>(b),
-                                                                    static_cast<uint32_t>(d.m), static_cast<uint32_t>(d.n), static_cast<uint32_t>(d.k),
-                                                                    chunk, lpc_shift, d.a.col_stride, d.b.col_stride, d.a.stride, d.b.stride);
-        matmul_long_k_combine<false><<<grid2, 256, 0, stream>>>(static_cast<uint16_t *>(c), partial, static_cast<uint32_t>(d.m),
-                                                                static_cast<uint32_t>(d.n), chunks, d.c.col_stride, d.c.stride, d.alpha, d.beta);
-    }
+    if (d.elem == amd::Elem::BF16) launch_long_k<true>(d, p, static_cast<float *>(workspace), c, a, b, stream);
+    else launch_long_k<false>(d, p, static_cast<float *>(workspace), c, a, b, stream);
     return true;
 }

@@ -19,7 +19,13 @@ struct MlpDescriptor {
     uint64_t gate_up_bytes; // [tokens, 2*di]
     uint64_t hidden_bytes;  // [tokens, di]
     uint64_t up_offset_bytes;// where the `up` half of a gate/up row starts
+    uint64_t matmul_bytes;   // the larger of what the two Matmuls ask for (few tokens: their sums are split over workgroups), used by one after the other
 };
+
+uint64_t matmul_offset(const MlpDescriptor &d) { return (d.gate_up_bytes + d.hidden_bytes + 15) / 16 * 16; }
+uint64_t workspace_bytes(const MlpDescriptor &d) {
+    return d.matmul_bytes != 0 ? matmul_offset(d) + d.matmul_bytes : d.gate_up_bytes + d.hidden_bytes;
+}
 
 uint64_t elem_size(DataLayout dt) { return dt.size; }
 
@@ -55,7 +61,7 @@ INFINIOP_C infiniopStatus_t infiniopCreateMLPDescriptor(infiniopHandle_t handle,
         return STATUS_BAD_TENSOR_SHAPE;// the reference halves it without looking
     }
     const uint64_t tokens = x_desc->shape[0], two_di = w12_desc->shape[1], di = two_di / 2;
-    auto *d = new (std::nothrow) MlpDescriptor{handle->device, nullptr, nullptr, nullptr, 0, 0, 0};
+    auto *d = new (std::nothrow) MlpDescriptor{handle->device, nullptr, nullptr, nullptr, 0, 0, 0, 0};
     if (d == nullptr) {
         return STATUS_MEMORY_NOT_ALLOCATED;
     }
@@ -78,6 +84,10 @@ INFINIOP_C infiniopStatus_t infiniopCreateMLPDescriptor(infiniopHandle_t handle,
     d->gate_up_bytes = tokens * two_di * elem_size(x_desc->dt);
     d->hidden_bytes = tokens * di * elem_size(x_desc->dt);
     d->up_offset_bytes = di * elem_size(x_desc->dt);
+    uint64_t first = 0, second = 0;
+    infiniopGetMatmulWorkspaceSize(d->gate_up_proj, &first);
+    infiniopGetMatmulWorkspaceSize(d->down_proj, &second);
+    d->matmul_bytes = first > second ? first : second;
     *desc_ptr = reinterpret_cast<infiniopMLPDescriptor_t>(d);
     return STATUS_SUCCESS;
 }
@@ -87,7 +97,7 @@ INFINIOP_C infiniopStatus_t infiniopGetMLPWorkspaceSize(infiniopMLPDescriptor_t 
         return STATUS_BAD_PARAM;
     }
     auto *d = reinterpret_cast<MlpDescriptor *>(desc);
-    *size = d->gate_up_bytes + d->hidden_bytes;// both Matmul workspaces are 0 bytes
+    *size = workspace_bytes(*d);
     return STATUS_SUCCESS;
 }
 
@@ -97,16 +107,17 @@ INFINIOP_C infiniopStatus_t infiniopMLP(infiniopMLPDescriptor_t desc, void *work
         return STATUS_BAD_PARAM;
     }
     auto *d = reinterpret_cast<MlpDescriptor *>(desc);
-    if (workspace_size < d->gate_up_bytes + d->hidden_bytes || (workspace == nullptr && d->gate_up_bytes + d->hidden_bytes > 0)) {
+    if (workspace_size < workspace_bytes(*d) || (workspace == nullptr && workspace_bytes(*d) > 0)) {
         return STATUS_MEMORY_NOT_ALLOCATED;// the reference's answer to a short workspace (mlp/operator.cc:100-102)
     }
     char *gate_up = static_cast<char *>(workspace);
     char *hidden = gate_up + d->gate_up_bytes;
-    infiniopStatus_t st = infiniopMatmul(d->gate_up_proj, nullptr, 0, gate_up, x, w12, stream);
+    char *for_matmul = d->matmul_bytes != 0 ? static_cast<char *>(workspace) + matmul_offset(*d) : nullptr;
+    infiniopStatus_t st = infiniopMatmul(d->gate_up_proj, for_matmul, d->matmul_bytes, gate_up, x, w12, stream);
     if (st != STATUS_SUCCESS) return st;
     st = infiniopSwiGLU(d->activation, hidden, gate_up + d->up_offset_bytes, gate_up, stream);
     if (st != STATUS_SUCCESS) return st;
-    return infiniopMatmul(d->down_proj, nullptr, 0, y, hidden, w3, stream);
+    return infiniopMatmul(d->down_proj, for_matmul, d->matmul_bytes, y, hidden, w3, stream);
 }
 
 INFINIOP_C infiniopStatus_t infiniopDestroyMLPDescriptor(infiniopMLPDescriptor_t desc) {

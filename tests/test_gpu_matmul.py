@@ -131,6 +131,41 @@ def test_the_products_of_a_decoding_attention(ctx, dt, case, alpha, beta):
         assert np.all(np.abs(g - exact) <= 0.5 * ULP[dt] * np.abs(exact) + 4 * keys * 2.0 ** -24 * mag + 1e-30), f"weighted values case {case} {dt} workspace {use_workspace}"
 
 
+# tokens, input width, output width, row pitch of the weight matrix (a few tokens through a layer's weights while decoding:
+# the sum over the input width is split over workgroups, matmul_long_k_wide, through the workspace Matmul asks for)
+WEIGHT_CASES = [(1, 1024, 1024, 1024), (8, 4096, 2048, 2048), (3, 1031, 1544, 1544), (5, 2050, 8200, 8208), (8, 8192, 10240, 10240),
+                (2, 28672, 8192, 8192), (7, 1500, 1024, 4096), (9, 2048, 2048, 2048), (4, 2048, 1028, 1032)]
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("case", range(len(WEIGHT_CASES)))
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 0.25)])
+def test_few_tokens_through_a_weight_matrix(ctx, dt, case, alpha, beta):
+    import torch
+
+    from operators_amd.ops import MatmulPlan
+
+    tokens, d, n, pitch = WEIGHT_CASES[case]
+    rng = np.random.default_rng(4000 + case)
+    x = make((tokens, d), dt, rng, False)
+    w = (rng.standard_normal((d, n)).astype(np.float32) * 0.05)
+    w = oracle.encode(w, dt)
+    y0 = make((tokens, n), dt, rng, False)
+    tx = to_torch(x, dt)
+    tw = device(w, dt, (pitch, 1)) if pitch != n else to_torch(w, dt)
+    exact = alpha * np.matmul(as_f64(x, dt), as_f64(w, dt)) + beta * as_f64(y0, dt)
+    mag = abs(alpha) * np.matmul(np.abs(as_f64(x, dt)), np.abs(as_f64(w, dt))) + abs(beta) * np.abs(as_f64(y0, dt))
+    for use_workspace in (True, False):
+        ty = to_torch(y0, dt)
+        with MatmulPlan(ctx, ty, tx, tw, alpha, beta) as plan:
+            fits = tokens <= 8 and n % 8 == 0 and n >= 1024 and d >= 1024 and pitch % 8 == 0
+            assert (plan.workspace_size > 0) == fits, (case, plan.workspace_size)
+            plan(ty, tx, tw, None, use_workspace)
+        torch.cuda.synchronize()
+        g = as_f64(to_codes(ty), dt)
+        assert np.all(np.abs(g - exact) <= 0.5 * ULP[dt] * np.abs(exact) + 4 * d * 2.0 ** -24 * mag + 1e-30), f"case {case} {dt} workspace {use_workspace}"
+
+
 def test_decoding_products_with_special_values(ctx):
     """An infinity or a NaN in one key's values, or in one weight, reaches exactly the outputs it reaches in the float64
     product - also where the key count is odd and the last pair of keys is half empty."""
