@@ -89,18 +89,19 @@ __global__ __launch_bounds__(kLanes) void matmul_long_k_partial(float *partial, 
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[j][e] = 0.0f;
     }
-    constexpr int AHEAD = 4;// steps whose loads are in flight together
+    constexpr int AHEAD = 2;// steps per set of registers; two sets take turns, so loads are in flight while the arrived ones are worked on
     const uint16_t *mine = a + static_cast<int64_t>(k0) * lda + sub * 8;
-    for (uint32_t p0 = 0; p0 < pairs; p0 += pairs_per_step * AHEAD) {
-        u32x4 lo[AHEAD], hi[AHEAD];
+    const auto fetch = [&](uint32_t p0, u32x4(&lo)[AHEAD], u32x4(&hi)[AHEAD]) {
 #pragma unroll
         for (int s = 0; s < AHEAD; ++s) {
             const uint32_t p = p0 + s * pairs_per_step + slot;
             const uint32_t c0 = 2 * p, c1 = 2 * p + 1;
-            // a column past the end is the chunk's last one again, and counts as zeros below
+            // a column past the end is the chunk's last one again, and is not used
             lo[s] = ld16_stream(mine + static_cast<int64_t>(c0 < here ? c0 : here - 1) * lda);
             hi[s] = ld16_stream(mine + static_cast<int64_t>(c1 < here ? c1 : here - 1) * lda);
         }
+    };
+    const auto work = [&](uint32_t p0, const u32x4(&lo)[AHEAD], const u32x4(&hi)[AHEAD]) {
 #pragma unroll
         for (int s = 0; s < AHEAD; ++s) {
             const uint32_t p = p0 + s * pairs_per_step + slot;
@@ -123,6 +124,15 @@ __global__ __launch_bounds__(kLanes) void matmul_long_k_partial(float *partial, 
                 for (int e = 0; e < 8; ++e) acc[j][e] = dot2<BF>(v[e], w[j], acc[j][e]);
             }
         }
+    };
+    const uint32_t turn = pairs_per_step * AHEAD;
+    u32x4 lo0[AHEAD], hi0[AHEAD], lo1[AHEAD], hi1[AHEAD];
+    fetch(0, lo0, hi0);
+    for (uint32_t p0 = 0; p0 < pairs; p0 += 2 * turn) {
+        fetch(p0 + turn, lo1, hi1);
+        work(p0, lo0, hi0);
+        fetch(p0 + 2 * turn, lo0, hi0);
+        work(p0 + turn, lo1, hi1);
     }
 
     // the lanes of a wavefront that share rows (lanes sub, sub + lanes_per_column, ...), then the wavefronts through LDS
