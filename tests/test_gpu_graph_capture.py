@@ -147,3 +147,45 @@ def test_split_causal_softmax_replays_from_a_hip_graph(ctx):
         torch.cuda.synchronize()
         assert torch.equal(scores.view(torch.int16), want[i].view(torch.int16)), replay
     plan.close()
+
+
+def test_decoding_mlp_replays_from_a_hip_graph(ctx):
+    """One token through the MLP composite: both products are this library's own kernels (partial sums through the
+    composite's workspace), so the capture holds five kernels of this library and nothing else."""
+    import torch
+
+    from operators_amd.ops import MLPPlan
+
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(8)
+    d, di, bf16 = 2048, 4096, torch.bfloat16
+    rnd = lambda *s, scale=1.0: (torch.randn(s, device="cuda", dtype=torch.float32, generator=gen) * scale).to(bf16)  # noqa: E731
+    xs = [rnd(1, d) for _ in range(3)]
+    w12, w3 = rnd(d, 2 * di, scale=d ** -0.5), rnd(di, d, scale=di ** -0.5)
+    x, y = xs[0].clone(), torch.zeros((1, d), dtype=bf16, device="cuda")
+    plan = MLPPlan(ctx, y, x, w12, w3, 1.0, False)
+    want = []
+    for v in xs:
+        x.copy_(v)
+        plan(y, x, w12, w3)
+        torch.cuda.synchronize()
+        want.append(y.clone())
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            plan(y, x, w12, w3, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for replay in range(6):
+        i = replay % len(xs)
+        y.zero_()
+        plan.workspace.random_(0, 256)
+        x.copy_(xs[i])
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), want[i].view(torch.int16)), replay
+    plan.close()
