@@ -166,6 +166,50 @@ def test_few_tokens_through_a_weight_matrix(ctx, dt, case, alpha, beta):
         assert np.all(np.abs(g - exact) <= 0.5 * ULP[dt] * np.abs(exact) + 4 * d * 2.0 ** -24 * mag + 1e-30), f"case {case} {dt} workspace {use_workspace}"
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_random_decoding_products(ctx, seed):
+    """Random shapes, strides, scales and types around the three products this library serves itself (and just outside
+    them, where the BLAS library takes the call): each output within rounding of the float64 product."""
+    import torch
+
+    from operators_amd.ops import MatmulPlan
+
+    rng = np.random.default_rng(7000 + seed)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7000 + seed)
+    dt = torch.bfloat16 if rng.random() < 0.5 else torch.float16
+    ulp = 2.0 ** -7 if dt == torch.bfloat16 else 2.0 ** -10
+    randn = lambda *shape, scale=1.0: (torch.randn(shape, device="cuda", generator=gen) * scale).to(dt)  # noqa: E731
+    kind = seed % 3
+    batch = int(rng.choice([1, 1, 2, 3, 8]))
+    nq = int(rng.integers(1, 18))
+    alpha, beta = (1.0, 0.0) if rng.random() < 0.5 else (float(rng.choice([0.5, -1.25, 0.125])), float(rng.choice([0.0, 1.0, 0.25])))
+    if kind == 0:  # scores = q K^T
+        hd = int(rng.choice([32, 64, 96, 128, 160, 256, 384, 512, 48, 1024]))
+        keys = int(rng.integers(900, 40000))
+        rows = (keys + int(rng.integers(0, 9)) + 7) // 8 * 8
+        cache = randn(batch, rows, hd)
+        a, b, c, kk = randn(batch, nq, hd), cache[:, :keys, :].transpose(1, 2), randn(batch, nq, keys), hd
+    elif kind == 1:  # out = weights V
+        hd = int(rng.choice([8, 16, 32, 64, 128, 256, 96, 512]))
+        keys = int(rng.integers(900, 60000))
+        cache = randn(batch, keys + 3, hd)
+        a, b, c, kk = torch.rand((batch, nq, keys), device="cuda", generator=gen).to(dt), cache[:, :keys, :], randn(batch, nq, hd), keys
+    else:  # tokens through weights
+        d = int(rng.integers(900, 9000))
+        n = int(rng.choice([1024, 1536, 2048, 4096, 8200, 1000, 1028, 22016]))
+        wbuf = randn(d, n + int(rng.choice([0, 0, 8, 24, 4])), scale=0.05)
+        a, b, c, kk = randn(nq, d), wbuf[:, :n], randn(nq, n), d
+    c0 = c.clone()
+    with MatmulPlan(ctx, c, a, b, alpha, beta) as plan:
+        plan(c, a, b)
+    torch.cuda.synchronize()
+    want = alpha * torch.matmul(a.double(), b.double()) + beta * c0.double()
+    mag = abs(alpha) * torch.matmul(a.double().abs(), b.double().abs()) + abs(beta) * c0.double().abs()
+    outside = (c.double() - want).abs() > want.abs() * ulp * 0.5 + 4 * kk * 2.0 ** -24 * mag + 1e-30
+    assert not bool(outside.any()), f"seed {seed}: kind {kind} {dt} a {tuple(a.shape)} b {tuple(b.shape)} alpha {alpha} beta {beta}: {int(outside.sum())} outside rounding"
+
+
 def test_decoding_products_with_special_values(ctx):
     """An infinity or a NaN in one key's values, or in one weight, reaches exactly the outputs it reaches in the float64
     product - also where the key count is odd and the last pair of keys is half empty."""
