@@ -4,9 +4,11 @@
 // in the descriptor's column-major terms with n <= 16 columns (the queries of
 // one K/V head), m in the tens of thousands (the keys), k = head_dim, every
 // row of a (a key) and every column of b (a query) contiguous along k.  The
-// library GEMM reads such an a at a quarter of the memory rate ([8 x 128] x
-// [128 x 131072] per K/V head, 8 heads, bf16: 170 us for 268 MB); the product is
-// bound by reading a once, and this kernel does just that.
+// product is bound by reading a once, and this kernel does just that.
+// Measured on MI355X, bf16, 8 K/V heads of [8 x head_dim] x [head_dim x 32768],
+// us, this kernel / the library GEMM: head_dim 32: 5.5 / 17.6, 64: 9.5 / 17.7,
+// 128: 15.8 / 25.6, 256: 29.7 / 40.6, 512: 55.6 / 73.8 (4.3-4.8 TB/s from 128
+// on); 128 at 4096 keys 5.9 / 18, at 131072 keys 57 / 59.
 //
 // A wavefront takes 16 x TILES rows of a per turn.  Lane l holds 16 bytes of row
 // l % 16 of each tile per step of 32 along k (8 elements from k = 32 s +
@@ -53,8 +55,8 @@ __device__ __forceinline__ uint16_t narrow(float v) {// round to nearest even
 
 constexpr int kSkinnyLanes = 256;
 
-// KS steps of 32 along k.  TILES x KS 16-byte loads per lane are in flight together.
-template<bool BF, int KS, int TILES>
+// GROUPS turns of KS steps of 32 along k.  TILES x KS 16-byte loads per lane are in flight together.
+template<bool BF, int KS, int TILES, int GROUPS>
 __global__ __launch_bounds__(kSkinnyLanes) void matmul_skinny(uint16_t *c, const uint16_t *a, const uint16_t *b, uint32_t m, uint32_t n,
                                                               int64_t lda, int64_t ldb, int64_t ldc, int64_t batch_a, int64_t batch_b,
                                                               int64_t batch_c, float alpha, float beta, uint32_t c_in_eights) {
@@ -67,32 +69,41 @@ __global__ __launch_bounds__(kSkinnyLanes) void matmul_skinny(uint16_t *c, const
     b += static_cast<int64_t>(blockIdx.y) * batch_b;
     c += static_cast<int64_t>(blockIdx.y) * batch_c;
 
-    u32x4 x[TILES][KS];
+    f32x4 acc[TILES];
 #pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-        const uint32_t row = row0 + t * 16 + of16;
-        const uint16_t *at = a + static_cast<int64_t>(row < m ? row : m - 1) * lda + quad * 8;// rows past the end repeat the last one; nothing of them is stored
+    for (int t = 0; t < TILES; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 1
+    for (int g = 0; g < GROUPS; ++g) {
+        u32x4 x[TILES][KS];
 #pragma unroll
-        for (int s = 0; s < KS; ++s) x[t][s] = ld16_stream(at + s * 32);
-    }
-    u32x4 q[KS];
+        for (int t = 0; t < TILES; ++t) {
+            const uint32_t row = row0 + t * 16 + of16;
+            // rows past the end repeat the last one; nothing of them is stored
+            const uint16_t *at = a + static_cast<int64_t>(row < m ? row : m - 1) * lda + g * (KS * 32) + quad * 8;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        q[s] = u32x4{0, 0, 0, 0};
-        if (of16 < n) q[s] = *reinterpret_cast<const u32x4 *>(b + static_cast<int64_t>(of16) * ldb + s * 32 + quad * 8);
-    }
-#pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-        f32x4 acc{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int s = 0; s < KS; ++s) x[t][s] = ld16_stream(at + s * 32);
+        }
+        u32x4 q[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-            acc = mma<BF>(x[t][s].x, x[t][s].y, q[s].x, q[s].y, acc);
-            acc = mma<BF>(x[t][s].z, x[t][s].w, q[s].z, q[s].w, acc);
+            q[s] = u32x4{0, 0, 0, 0};
+            if (of16 < n) q[s] = *reinterpret_cast<const u32x4 *>(b + static_cast<int64_t>(of16) * ldb + g * (KS * 32) + s * 32 + quad * 8);
         }
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                acc[t] = mma<BF>(x[t][s].x, x[t][s].y, q[s].x, q[s].y, acc[t]);
+                acc[t] = mma<BF>(x[t][s].z, x[t][s].w, q[s].z, q[s].w, acc[t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
         const uint32_t first = row0 + t * 16 + quad * 4;// this lane's four rows of c, column of16
         if (of16 >= n || first >= m) continue;
         uint16_t *out = c + static_cast<int64_t>(of16) * ldc + first;
-        const float r[4] = {acc.x, acc.y, acc.z, acc.w};
+        const float r[4] = {acc[t].x, acc[t].y, acc[t].z, acc[t].w};
         uint16_t h[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -111,12 +122,12 @@ __global__ __launch_bounds__(kSkinnyLanes) void matmul_skinny(uint16_t *c, const
     }
 }
 
-template<bool BF, int KS>
+template<bool BF, int KS, int GROUPS>
 void launch(const MatmulAmdDescriptor &d, void *c, const void *a, const void *b, bool c_in_eights, hipStream_t stream) {
-    constexpr int TILES = KS >= 16 ? 1 : KS >= 8 ? 2 : 4;
+    constexpr int TILES = 4;
     const uint32_t rows_per_group = (kSkinnyLanes / kWave) * 16 * TILES;
     const dim3 grid(static_cast<unsigned>((d.m + rows_per_group - 1) / rows_per_group), static_cast<unsigned>(d.batch));
-    matmul_skinny<BF, KS, TILES><<<grid, kSkinnyLanes, 0, stream>>>(
+    matmul_skinny<BF, KS, TILES, GROUPS><<<grid, kSkinnyLanes, 0, stream>>>(
         static_cast<uint16_t *>(c), static_cast<const uint16_t *>(a), static_cast<const uint16_t *>(b), static_cast<uint32_t>(d.m),
         static_cast<uint32_t>(d.n), d.a.row_stride, d.b.col_stride, d.c.col_stride, d.a.stride, d.b.stride, d.c.stride, d.alpha, d.beta,
         c_in_eights ? 1u : 0u);
@@ -137,22 +148,24 @@ bool amd_matmul_skinny(const MatmulAmdDescriptor &d, void *c, const void *a, con
     if (d.m > 0x7FFFFFF0ll) return false;
     const bool c_in_eights = (reinterpret_cast<uintptr_t>(c) & 7u) == 0 && d.c.col_stride % 4 == 0 && d.c.stride % 4 == 0;
     const bool bf = d.elem == amd::Elem::BF16;
-#define SKINNY(KS)                                                \
-    case KS:                                                      \
-        if (bf) launch<true, KS>(d, c, a, b, c_in_eights, stream); \
-        else launch<false, KS>(d, c, a, b, c_in_eights, stream);   \
+#define SKINNY(STEPS, KS, GROUPS)                                          \
+    case STEPS:                                                            \
+        if (bf) launch<true, KS, GROUPS>(d, c, a, b, c_in_eights, stream); \
+        else launch<false, KS, GROUPS>(d, c, a, b, c_in_eights, stream);   \
         break
+    // head widths of 256 and more in turns of 128: with all of k in registers at once the compiler needs every one
+    // of them (8 x [8 x 256] x [256 x 32768] bf16: 49.5 us that way, 29.7 in two turns; 512: 64.9 and 55.6)
     switch (d.k / 32) {
-        SKINNY(1);
-        SKINNY(2);
-        SKINNY(3);
-        SKINNY(4);
-        SKINNY(5);
-        SKINNY(6);
-        SKINNY(7);
-        SKINNY(8);
-        SKINNY(12);
-        SKINNY(16);
+        SKINNY(1, 1, 1);
+        SKINNY(2, 2, 1);
+        SKINNY(3, 3, 1);
+        SKINNY(4, 4, 1);
+        SKINNY(5, 5, 1);
+        SKINNY(6, 6, 1);
+        SKINNY(7, 7, 1);
+        SKINNY(8, 4, 2);
+        SKINNY(12, 4, 3);
+        SKINNY(16, 4, 4);
         default: return false;
     }
 #undef SKINNY
