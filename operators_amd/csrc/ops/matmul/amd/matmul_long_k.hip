@@ -66,29 +66,11 @@ __global__ __launch_bounds__(kLanes) void matmul_long_k_partial(float *partial, 
     a += static_cast<int64_t>(blockIdx.y) * batch_a;
     b += static_cast<int64_t>(blockIdx.y) * batch_b;
 
-    // b's share of the chunk into LDS, pairs along k
     const uint32_t pairs = (here + 1) / 2;
-    for (uint32_t w = tid; w < pairs * kColumnsOfB; w += kLanes) {
-        const uint32_t j = w / pairs, p = w - j * pairs;// a column of b at a time: neighbouring lanes read neighbouring words
-        uint32_t word = 0;
-        if (j < n) {
-            const uint16_t *at = b + static_cast<int64_t>(j) * ldb + k0 + 2 * p;
-            word = 2 * p + 1 < here ? *reinterpret_cast<const u32_any *>(at) : static_cast<uint32_t>(*at);
-        }
-        staged[p * kColumnsOfB + j] = word;
-    }
-    __syncthreads();
-
     const uint32_t lanes_per_column = 1u << lpc_shift;
     const uint32_t sub = tid & (lanes_per_column - 1);// which 8 rows of a
     const uint32_t slot = tid >> lpc_shift;           // which pair of columns within a step
     const uint32_t pairs_per_step = kLanes >> lpc_shift;
-    float acc[kColumnsOfB][8];
-#pragma unroll
-    for (int j = 0; j < kColumnsOfB; ++j) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] = 0.0f;
-    }
     constexpr int AHEAD = 2;// steps per set of registers; two sets take turns, so loads are in flight while the arrived ones are worked on
     const uint16_t *mine = a + static_cast<int64_t>(k0) * lda + sub * 8;
     const auto fetch = [&](uint32_t p0, u32x4(&lo)[AHEAD], u32x4(&hi)[AHEAD]) {
@@ -101,6 +83,28 @@ __global__ __launch_bounds__(kLanes) void matmul_long_k_partial(float *partial, 
             hi[s] = ld16_stream(mine + static_cast<int64_t>(c1 < here ? c1 : here - 1) * lda);
         }
     };
+    // the first loads of a go out before b's share of the chunk is staged
+    u32x4 lo0[AHEAD], hi0[AHEAD], lo1[AHEAD], hi1[AHEAD];
+    fetch(0, lo0, hi0);
+
+    // b's share of the chunk into LDS, pairs along k
+    for (uint32_t w = tid; w < pairs * kColumnsOfB; w += kLanes) {
+        const uint32_t j = w / pairs, p = w - j * pairs;// a column of b at a time: neighbouring lanes read neighbouring words
+        uint32_t word = 0;
+        if (j < n) {
+            const uint16_t *at = b + static_cast<int64_t>(j) * ldb + k0 + 2 * p;
+            word = 2 * p + 1 < here ? *reinterpret_cast<const u32_any *>(at) : static_cast<uint32_t>(*at);
+        }
+        staged[p * kColumnsOfB + j] = word;
+    }
+    __syncthreads();
+
+    float acc[kColumnsOfB][8];
+#pragma unroll
+    for (int j = 0; j < kColumnsOfB; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.0f;
+    }
     const auto work = [&](uint32_t p0, const u32x4(&lo)[AHEAD], const u32x4(&hi)[AHEAD]) {
 #pragma unroll
         for (int s = 0; s < AHEAD; ++s) {
@@ -126,8 +130,6 @@ __global__ __launch_bounds__(kLanes) void matmul_long_k_partial(float *partial, 
         }
     };
     const uint32_t turn = pairs_per_step * AHEAD;
-    u32x4 lo0[AHEAD], hi0[AHEAD], lo1[AHEAD], hi1[AHEAD];
-    fetch(0, lo0, hi0);
     for (uint32_t p0 = 0; p0 < pairs; p0 += 2 * turn) {
         fetch(p0 + turn, lo1, hi1);
         work(p0, lo0, hi0);
@@ -188,25 +190,8 @@ __global__ __launch_bounds__(kWave) void matmul_long_k_wide(float *partial, cons
     a += static_cast<int64_t>(blockIdx.y) * batch_a;
     b += static_cast<int64_t>(blockIdx.y) * batch_b;
     const uint32_t pairs = (here + 1) / 2;
-    for (uint32_t w = lane; w < pairs * kColumnsOfB; w += kWave) {
-        const uint32_t j = w / pairs, p = w - j * pairs;
-        uint32_t word = 0;
-        if (j < n) {
-            const uint16_t *at = b + static_cast<int64_t>(j) * ldb + k0 + 2 * p;
-            word = 2 * p + 1 < here ? *reinterpret_cast<const u32_any *>(at) : static_cast<uint32_t>(*at);
-        }
-        staged[p * kColumnsOfB + j] = word;
-    }
-    __syncthreads();
-
     const uint32_t row0 = tile * kWideRows + lane * 8;
     const bool rows_here = row0 < m;// m is a multiple of 8: a lane's rows are all there or none is
-    float acc[kColumnsOfB][8];
-#pragma unroll
-    for (int j = 0; j < kColumnsOfB; ++j) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] = 0.0f;
-    }
     const uint16_t *mine = a + static_cast<int64_t>(k0) * lda + (rows_here ? row0 : 0);
     // Two sets of registers take turns: the loads of the next kWideAhead pairs of columns go out before the work on
     // the ones that have arrived, so a wavefront always has loads in flight.
@@ -218,6 +203,26 @@ __global__ __launch_bounds__(kWave) void matmul_long_k_wide(float *partial, cons
             hi[s] = ld16_stream(mine + static_cast<int64_t>(c1 < here ? c1 : here - 1) * lda);
         }
     };
+    // the first loads of a go out before b's share of the chunk is staged
+    u32x4 lo0[kWideAhead], hi0[kWideAhead], lo1[kWideAhead], hi1[kWideAhead];
+    fetch(0, lo0, hi0);
+    for (uint32_t w = lane; w < pairs * kColumnsOfB; w += kWave) {
+        const uint32_t j = w / pairs, p = w - j * pairs;
+        uint32_t word = 0;
+        if (j < n) {
+            const uint16_t *at = b + static_cast<int64_t>(j) * ldb + k0 + 2 * p;
+            word = 2 * p + 1 < here ? *reinterpret_cast<const u32_any *>(at) : static_cast<uint32_t>(*at);
+        }
+        staged[p * kColumnsOfB + j] = word;
+    }
+    __syncthreads();
+
+    float acc[kColumnsOfB][8];
+#pragma unroll
+    for (int j = 0; j < kColumnsOfB; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.0f;
+    }
     const auto work = [&](uint32_t p0, const u32x4(&lo)[kWideAhead], const u32x4(&hi)[kWideAhead]) {
 #pragma unroll
         for (int s = 0; s < kWideAhead; ++s) {
@@ -242,8 +247,6 @@ __global__ __launch_bounds__(kWave) void matmul_long_k_wide(float *partial, cons
             }
         }
     };
-    u32x4 lo0[kWideAhead], hi0[kWideAhead], lo1[kWideAhead], hi1[kWideAhead];
-    fetch(0, lo0, hi0);
     for (uint32_t p0 = 0; p0 < pairs; p0 += 2 * kWideAhead) {
         fetch(p0 + kWideAhead, lo1, hi1);
         work(p0, lo0, hi0);
