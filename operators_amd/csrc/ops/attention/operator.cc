@@ -11,7 +11,8 @@
 // contiguous, the final head transpose), two batched Matmuls and CausalSoftmax
 // in place on the scores.  Checks and status codes are the reference's.  The
 // caller provides the scratch memory: q made contiguous (when it is not),
-// the scores [n_q_head, seq, pos + seq] and the head-major result, in q's type.
+// the scores [n_q_head, seq, pos + seq] and the head-major result (unless seq or
+// n_q_head is 1, when it is out itself), in q's type.
 #include "../../devices/amd/common_amd.h"
 #include <cmath>
 #include <new>
@@ -131,7 +132,9 @@ INFINIOP_C infiniopStatus_t infiniopCreateAttentionDescriptor(infiniopHandle_t h
     if (ok()) st = infiniopCreateRearrangeDescriptor(handle, &p->store_v, v_slot, v_desc);
 
     // q as a dense [heads, seq, hd]; copied there unless it already is
-    const bool q_dense = q_desc->strides[1] == static_cast<int64_t>(hd) && q_desc->strides[0] == static_cast<int64_t>(seq * hd);
+    // (the stride of a dimension of extent 1 says nothing: one decoded token's q is dense whatever buffer its heads are a view of)
+    const bool q_dense = (seq == 1 || q_desc->strides[1] == static_cast<int64_t>(hd)) &&
+                         (heads == 1 || q_desc->strides[0] == static_cast<int64_t>(seq * hd));
     infiniopTensorDescriptor_t q_packed = d.dense(dt, heads, seq, hd);
     if (!q_dense) {
         if (ok()) st = infiniopCreateRearrangeDescriptor(handle, &p->pack_q, q_packed, q_desc);
@@ -155,11 +158,13 @@ INFINIOP_C infiniopStatus_t infiniopCreateAttentionDescriptor(infiniopHandle_t h
     infiniopTensorDescriptor_t result_grouped = d.dense(dt, kv_heads, group * seq, hd);
     if (ok()) st = infiniopCreateMatmulDescriptor(handle, &p->weighted, result_grouped, 1.0f, scores_grouped, v_full, 0.0f);
     if (ok()) st = infiniopGetMatmulWorkspaceSize(p->weighted, &p->weighted_bytes);
-    p->result_bytes = heads * seq * hd * es;
-
-    // out[seq, heads, hd] = result[heads, seq, hd] with its first two dimensions exchanged
-    infiniopTensorDescriptor_t result_t = d.make(dt, seq, heads, hd, static_cast<int64_t>(hd), static_cast<int64_t>(seq * hd), 1);
-    if (ok()) st = infiniopCreateRearrangeDescriptor(handle, &p->unpack_out, out_desc, result_t);
+    // out[seq, heads, hd] = result[heads, seq, hd] with its first two dimensions exchanged - which moves nothing when
+    // one of the two has extent 1 (one decoded token): the second Matmul then writes out itself
+    if (seq != 1 && heads != 1) {
+        p->result_bytes = heads * seq * hd * es;
+        infiniopTensorDescriptor_t result_t = d.make(dt, seq, heads, hd, static_cast<int64_t>(hd), static_cast<int64_t>(seq * hd), 1);
+        if (ok()) st = infiniopCreateRearrangeDescriptor(handle, &p->unpack_out, out_desc, result_t);
+    }
 
     if (!ok()) {
         destroy_all(p);
@@ -195,7 +200,7 @@ INFINIOP_C infiniopStatus_t infiniopAttention(infiniopAttentionDescriptor_t desc
     }
     char *q_packed = static_cast<char *>(workspace);
     char *scores = q_packed + p->q_bytes;
-    char *result = scores + p->scores_bytes;
+    char *result = p->unpack_out != nullptr ? scores + p->scores_bytes : static_cast<char *>(out);
     char *softmax_parts = p->softmax_bytes != 0 ? static_cast<char *>(workspace) + softmax_offset(*p) : nullptr;
     char *weighted_parts = p->weighted_bytes != 0 ? static_cast<char *>(workspace) + weighted_offset(*p) : nullptr;
 
@@ -208,7 +213,7 @@ INFINIOP_C infiniopStatus_t infiniopAttention(infiniopAttentionDescriptor_t desc
     if (st == STATUS_SUCCESS) st = infiniopMatmul(p->scores, nullptr, 0, scores, q, k_cache, stream);
     if (st == STATUS_SUCCESS) st = infiniopCausalSoftmax(p->softmax, softmax_parts, p->softmax_bytes, scores, stream);
     if (st == STATUS_SUCCESS) st = infiniopMatmul(p->weighted, weighted_parts, p->weighted_bytes, result, scores, v_cache, stream);
-    if (st == STATUS_SUCCESS) st = infiniopRearrange(p->unpack_out, out, result, stream);
+    if (st == STATUS_SUCCESS && p->unpack_out != nullptr) st = infiniopRearrange(p->unpack_out, out, result, stream);
     return st;
 }
 
