@@ -319,13 +319,14 @@ Plan plan_of(const MatmulAmdDescriptor &d) {
     // Many rows: about 1024 wavefronts in all, chunks of 256 columns and more (a chunk leaves 32 bytes of partial
     // sums per row and column of b behind).  Measured against the BLAS library, bf16, us, 1 / 8 columns of b:
     // [8192 x 28672]: 81 / 91 against 127 / 132; [22016 x 4096]: 36 / 42 against 52 / 52; [10240 x 8192]: 36 / 42
-    // against 49 / 50; [8192 x 8192]: 38 / 42 against 43 / 44; [57344 x 8192]: 155 / 172 against 158 / 166 - the
-    // library reads that one at 5.7 TB/s, and keeps it from three columns of b on.  (Room for 16 columns of b - 128
+    // against 49 / 50; [8192 x 8192]: 38 / 42 against 43 / 44; [57344 x 8192], 1 / 4 / 8 columns: 153 / 161 / 172
+    // against 158 / 165 / 166 - the library reads that one at 5.7 TB/s, and keeps it from five columns of b on
+    // (fewer, longer chunks there - 512 or 768 wavefronts - take 238 and 160 us).  (Room for 16 columns of b - 128
     // accumulators per lane - took 211 registers and 528 bytes of scratch and ran 9-10 times slower than the
     // library on every shape: 9 to 16 columns stay with the library.)
     if (d.m >= 1024 && d.m % 8 == 0 && d.m <= 0x7FFFFFF0ll && d.m * kColumnsOfB < (1ll << 31)) {
         const uint32_t tiles = static_cast<uint32_t>((d.m + kWideRows - 1) / kWideRows);
-        if (tiles >= 64 && d.n > 2) return none;
+        if (tiles >= 64 && d.n > 4) return none;
         uint64_t chunks = 1024 / (static_cast<uint64_t>(tiles) * d.batch);
         if (chunks < 1) chunks = 1;
         uint64_t chunk = (d.k + chunks - 1) / chunks;
